@@ -1,0 +1,151 @@
+"""ctypes front-end of the CPU oracle (oracle/refconv.c).
+
+TEST INFRASTRUCTURE ONLY: imported by tests/, by __graft_entry__.smoke() and by
+bench.py's cpu_baseline leg, never by the product package.
+"""
+import ctypes as C
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB = None
+
+S8, U8, I32, F32, NONE = 0, 1, 2, 3, -1
+ACT_NONE, ACT_RELU, ACT_RELU_SLOPE, ACT_CLAMP = 0, 1, 2, 3
+
+DT_OF = {np.dtype(np.int8): S8, np.dtype(np.uint8): U8, np.dtype(np.int32): I32, np.dtype(np.float32): F32}
+NP_OF = {S8: np.int8, U8: np.uint8, I32: np.int32, F32: np.float32}
+NAME_OF = {"s8": S8, "i8": S8, "u8": U8, "i32": I32, "f32": F32}
+ACT_OF = {"none": ACT_NONE, "relu": ACT_RELU, "relu_slope": ACT_RELU_SLOPE, "clamp": ACT_CLAMP}
+
+
+class Pitch(C.Structure):
+    _fields_ = [(n, C.c_int64) for n in ("off", "pb", "pf", "py", "px")]
+
+
+class Desc(C.Structure):
+    _fields_ = (
+        [(n, C.c_int) for n in ("in_dt", "w_dt", "bias_dt", "out_dt", "eltw_dt")]
+        + [(n, C.c_int) for n in ("B", "IFM", "IH", "IW", "OFM", "OH", "OW", "FY", "FX")]
+        + [(n, C.c_int) for n in ("sy", "sx", "dy", "dx", "pad_y", "pad_x", "groups")]
+        + [("has_wqf", C.c_int), ("has_calib", C.c_int), ("iqf", C.c_float), ("oqf", C.c_float)]
+        + [("act", C.c_int), ("act_m", C.c_float), ("act_n", C.c_float)]
+        + [("fused", C.c_int), ("non_conv_scale", C.c_float)]
+        + [("eltw_act", C.c_int), ("eltw_m", C.c_float), ("eltw_n", C.c_float)]
+        + [("has_eltw_calib", C.c_int), ("esy", C.c_int), ("esx", C.c_int)]
+        + [("in_p", Pitch), ("out_p", Pitch), ("eltw_p", Pitch)]
+        + [("round_even", C.c_int)]
+    )
+
+
+def build(force=False):
+    """Compile oracle/librefconv.so with the Makefile beside it."""
+    so = os.path.join(_HERE, "librefconv.so")
+    if force and os.path.exists(so):
+        os.remove(so)
+    subprocess.check_call(["make", "-s", "-C", _HERE, "librefconv.so"])
+    return so
+
+
+def lib():
+    global _LIB
+    if _LIB is None:
+        so = os.path.join(_HERE, "librefconv.so")
+        if not os.path.exists(so):
+            build()
+        L = C.CDLL(so)
+        L.rc_out_extent.restype = C.c_int
+        L.rc_out_extent.argtypes = [C.c_int] * 5
+        L.rc_conv.restype = C.c_int
+        L.rc_conv.argtypes = [C.POINTER(Desc)] + [C.c_void_p] * 9 + [C.c_int]
+        L.rc_epilogue.restype = C.c_double
+        L.rc_epilogue.argtypes = [C.POINTER(Desc), C.c_int32, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p,
+                                  C.c_double, C.c_void_p]
+        L.rc_round_half_away.restype = C.c_float
+        L.rc_round_half_away.argtypes = [C.c_float]
+        L.rc_threads_available.restype = C.c_int
+        _LIB = L
+    return _LIB
+
+
+def out_extent(n, pad, filt, dil, stride):
+    return lib().rc_out_extent(n, pad, filt, dil, stride)
+
+
+def _ptr(a):
+    return None if a is None else a.ctypes.data_as(C.c_void_p)
+
+
+def _dense(F, H, W):
+    return Pitch(0, F * H * W, H * W, W, 1)
+
+
+def conv(x, w, bias=None, wqf=None, calib=None, *, stride=(1, 1), pad=(0, 0), dilation=(1, 1), groups=1,
+         out_dt=None, iqf=1.0, oqf=1.0, act="none", act_m=0.0, act_n=0.0,
+         eltw=None, non_conv_scale=1.0, eltw_act="none", eltw_m=0.0, eltw_n=0.0, eltw_calib=None,
+         eltw_stride=(1, 1), round_even=False, want_acc=False, nthreads=0):
+    """Reference convolution on dense bfyx numpy arrays.
+
+    x [B,IFM,IH,IW]; w [OFM,IFM/groups,FY,FX]; bias/wqf/calib/eltw_calib [OFM];
+    eltw [B,OFM,>=OH*esy..,>=OW*esx..].  stride/pad/dilation are (y, x).
+    Returns out (and the int32 accumulators when want_acc).
+    """
+    L = lib()
+    x = np.ascontiguousarray(x)
+    w = np.ascontiguousarray(w)
+    B, IFM, IH, IW = x.shape
+    OFM, IFMg, FY, FX = w.shape
+    assert IFMg * groups == IFM, (IFMg, groups, IFM)
+    OH = out_extent(IH, pad[0], FY, dilation[0], stride[0])
+    OW = out_extent(IW, pad[1], FX, dilation[1], stride[1])
+    d = Desc()
+    d.in_dt, d.w_dt = DT_OF[x.dtype], DT_OF[w.dtype]
+    d.bias_dt = NONE if bias is None else DT_OF[np.asarray(bias).dtype]
+    if out_dt is None:
+        out_dt = d.in_dt
+    elif isinstance(out_dt, str):
+        out_dt = NAME_OF[out_dt]
+    d.out_dt = out_dt
+    d.B, d.IFM, d.IH, d.IW, d.OFM, d.OH, d.OW, d.FY, d.FX = B, IFM, IH, IW, OFM, OH, OW, FY, FX
+    d.sy, d.sx, d.dy, d.dx, d.pad_y, d.pad_x, d.groups = stride[0], stride[1], dilation[0], dilation[1], pad[0], pad[1], groups
+    d.has_wqf, d.has_calib = int(wqf is not None), int(calib is not None)
+    d.iqf, d.oqf = iqf, oqf
+    d.act, d.act_m, d.act_n = ACT_OF[act] if isinstance(act, str) else act, act_m, act_n
+    d.fused = int(eltw is not None)
+    d.non_conv_scale = non_conv_scale
+    d.eltw_act = ACT_OF[eltw_act] if isinstance(eltw_act, str) else eltw_act
+    d.eltw_m, d.eltw_n = eltw_m, eltw_n
+    d.has_eltw_calib = int(eltw_calib is not None)
+    d.esy, d.esx = eltw_stride
+    d.in_p = _dense(IFM, IH, IW)
+    d.out_p = _dense(OFM, OH, OW)
+    d.round_even = int(round_even)
+    if eltw is not None:
+        eltw = np.ascontiguousarray(eltw)
+        d.eltw_dt = DT_OF[eltw.dtype]
+        d.eltw_p = _dense(eltw.shape[1], eltw.shape[2], eltw.shape[3])
+    else:
+        d.eltw_dt = NONE
+    keep = []
+
+    def f32(a):
+        if a is None:
+            return None
+        a = np.ascontiguousarray(a, dtype=np.float32)
+        keep.append(a)
+        return a
+
+    if bias is not None:
+        bias = np.ascontiguousarray(bias)
+    wqf, calib, eltw_calib = f32(wqf), f32(calib), f32(eltw_calib)
+    out = np.zeros((B, OFM, OH, OW), dtype=NP_OF[out_dt])
+    acc = np.zeros((B, OFM, OH, OW), dtype=np.int32) if want_acc else None
+    if nthreads <= 0:
+        nthreads = L.rc_threads_available()
+    rc = L.rc_conv(C.byref(d), _ptr(x), _ptr(w), _ptr(bias), _ptr(wqf), _ptr(calib), _ptr(eltw), _ptr(eltw_calib),
+                   _ptr(out), _ptr(acc), nthreads)
+    if rc != 0:
+        raise ValueError("refconv: unsupported combination")
+    return (out, acc) if want_acc else out
