@@ -1,0 +1,369 @@
+// Convolution objects of the C-ABI: validation, arithmetic-mode selection, kernel-family and
+// tile choice (the gfx950 tile-config table stands where the reference has kernel_selector and
+// its tuning cache), weight pre-packing, launch.
+#include <cstring>
+#include <vector>
+
+#include "kernels.h"
+#include "runtime.h"
+
+using namespace chip;
+
+struct cldnn_hip_conv_s {
+    cldnn_hip_engine engine = nullptr;
+    cldnn_hip_conv_desc desc{};
+    ConvProblem p{};
+    Epilogue epi{};       // device pointers inside
+    int impl = CLDNN_HIP_IMPL_REF;
+    int epi_kind = EPI_GENERIC;
+    MfmaPlan mplan{};
+    DwPlan dplan{};
+    // device allocations
+    void* w_raw = nullptr;    // dense weights (reference kernel)
+    void* w_packed = nullptr; // MFMA / depthwise operand stream
+    void* ktab = nullptr;
+    void* acc_init = nullptr;      // int32: offset correction + int32 bias
+    void* acc_init_raw = nullptr;  // int32: offset correction only (accumulator probe)
+    void* bias = nullptr;
+    void* wqf = nullptr;
+    void* calib = nullptr;
+    void* ecal = nullptr;
+    cldnn_hip_conv_info info{};
+    std::vector<void*> owned;
+};
+
+namespace {
+
+bool is_int8(int dt) { return dt == CLDNN_HIP_S8 || dt == CLDNN_HIP_U8; }
+
+int out_extent(int in, int pad, int filt, int dil, int stride)
+{
+    // reference src/include/sliding_window_utils.h:113-126; a window larger than the padded input gives 1
+    const int wnd = (filt - 1) * dil + 1;
+    const int span = in + 2 * pad;
+    if (wnd > span) return 1;
+    return (span - wnd) / stride + 1;
+}
+
+void* upload(cldnn_hip_conv c, const void* host, size_t bytes, size_t padded_bytes = 0)
+{
+    if (padded_bytes < bytes) padded_bytes = bytes;
+    void* d = nullptr;
+    hipError_t r = hipMalloc(&d, padded_bytes + 64);
+    if (r != hipSuccess) {
+        (void)hipGetLastError();
+        throw error(CLDNN_HIP_OUT_OF_RESOURCES, std::string("hipMalloc: ") + hipGetErrorString(r));
+    }
+    c->owned.push_back(d);
+    CHIP_CHECK(hipMemsetAsync(d, 0, padded_bytes + 64, c->engine->stream));
+    if (host && bytes) CHIP_CHECK(hipMemcpyAsync(d, host, bytes, hipMemcpyHostToDevice, c->engine->stream));
+    CHIP_CHECK(hipStreamSynchronize(c->engine->stream));
+    return d;
+}
+
+// gfx950 tile-config table lookup: largest tile that still gives every CU a couple of workgroups.
+int choose_tile(const ConvProblem& p, int cus)
+{
+    static const int by_size[] = {5, 0, 1, 3, 2, 4};  // p256_f128, p128_f128, p256_f64, p128_f64, p64_f128, p64_f64
+    const int64_t m = (int64_t)p.B * p.OH * p.OW;
+    int best = 4;
+    int64_t best_grid = -1;
+    for (int idx : by_size) {
+        const TileConfig& tc = tile_config(idx);
+        if (p.OFM <= 64 && tc.tile_ofm > 64) continue;
+        const int64_t grid = ((m + tc.tile_pixels - 1) / tc.tile_pixels) * ((p.OFM + tc.tile_ofm - 1) / tc.tile_ofm);
+        if (grid >= 2 * (int64_t)cus) return idx;
+        if (grid > best_grid) best_grid = grid, best = idx;
+    }
+    return best;
+}
+
+void build(cldnn_hip_conv c, const void* weights, const void* bias, const float* wqf, const float* calib,
+           const float* eltw_calib)
+{
+    const cldnn_hip_conv_desc& d = c->desc;
+    ConvProblem& p = c->p;
+    CHIP_REQUIRE(weights, CLDNN_HIP_INVALID_ARG, "convolution without weights");
+    CHIP_REQUIRE(d.groups >= 1 && d.ifm % d.groups == 0 && d.ofm % d.groups == 0, CLDNN_HIP_INVALID_ARG,
+                 "feature counts must divide into groups");
+    CHIP_REQUIRE(d.fy > 0 && d.fx > 0 && d.stride_y > 0 && d.stride_x > 0 && d.dilation_y > 0 && d.dilation_x > 0,
+                 CLDNN_HIP_INVALID_ARG, "filter size, stride and dilation must be positive");
+    CHIP_REQUIRE(d.pad_y >= 0 && d.pad_x >= 0, CLDNN_HIP_INVALID_ARG, "negative padding");
+    CHIP_REQUIRE(d.input.f == d.ifm, CLDNN_HIP_DIMENSION_MISMATCH, "input feature count differs from weights");
+    CHIP_REQUIRE(d.output.f == d.ofm && d.output.b == d.input.b, CLDNN_HIP_DIMENSION_MISMATCH,
+                 "output batch/feature count mismatch");
+    CHIP_REQUIRE((d.has_wqf != 0) == (wqf != nullptr), CLDNN_HIP_INVALID_ARG, "has_wqf does not match the wqf pointer");
+    CHIP_REQUIRE((d.has_calib != 0) == (calib != nullptr), CLDNN_HIP_INVALID_ARG, "has_calib does not match the calib pointer");
+    CHIP_REQUIRE((d.has_eltw_calib != 0) == (eltw_calib != nullptr), CLDNN_HIP_INVALID_ARG,
+                 "has_eltw_calib does not match the eltw_calib pointer");
+    CHIP_REQUIRE((d.bias_dtype != CLDNN_HIP_NO_TYPE) == (bias != nullptr), CLDNN_HIP_INVALID_ARG,
+                 "bias_dtype does not match the bias pointer");
+    if (bias) CHIP_REQUIRE(d.bias_dtype == CLDNN_HIP_I32 || d.bias_dtype == CLDNN_HIP_F32, CLDNN_HIP_INVALID_ARG, "bias must be i32 or f32");
+
+    p.B = d.input.b, p.IFM = d.ifm, p.IH = d.input.y, p.IW = d.input.x, p.OFM = d.ofm;
+    p.FY = d.fy, p.FX = d.fx, p.sy = d.stride_y, p.sx = d.stride_x, p.dy = d.dilation_y, p.dx = d.dilation_x;
+    p.py = d.pad_y, p.px = d.pad_x, p.groups = d.groups;
+    p.OH = out_extent(p.IH, p.py, p.FY, p.dy, p.sy);
+    p.OW = out_extent(p.IW, p.px, p.FX, p.dx, p.sx);
+    CHIP_REQUIRE(d.output.y == p.OH && d.output.x == p.OW, CLDNN_HIP_DIMENSION_MISMATCH,
+                 "output spatial size differs from the computed one");
+    p.in_dt = d.input.dtype, p.w_dt = d.weights_dtype, p.out_dt = d.output.dtype;
+    p.eltw_dt = d.fused ? d.eltw.dtype : CLDNN_HIP_NO_TYPE;
+    p.in_t = d.input, p.out_t = d.output;
+    p.in_p = make_pitch(d.input), p.out_p = make_pitch(d.output);
+    p.esy = d.fused ? (d.eltw_stride_y > 0 ? d.eltw_stride_y : 1) : 1;
+    p.esx = d.fused ? (d.eltw_stride_x > 0 ? d.eltw_stride_x : 1) : 1;
+    if (d.fused) {
+        if (d.second_input_in_output) {
+            p.eltw_t = d.output;
+            p.eltw_dt = d.output.dtype;
+        } else {
+            p.eltw_t = d.eltw;
+        }
+        p.eltw_p = make_pitch(p.eltw_t);
+        CHIP_REQUIRE(p.eltw_t.f == p.OFM && p.eltw_t.b == p.B && p.eltw_t.y >= (p.OH - 1) * p.esy + 1
+                         && p.eltw_t.x >= (p.OW - 1) * p.esx + 1,
+                     CLDNN_HIP_DIMENSION_MISMATCH, "second input of fused_conv_eltwise does not cover the output");
+    }
+
+    // ---- data-type legality (reference convolution_kernel_ref.cpp:124-166, fused ..._kernel_ref.cpp:21-47)
+    const bool in8 = is_int8(p.in_dt);
+    CHIP_REQUIRE(in8 || p.in_dt == CLDNN_HIP_F32, CLDNN_HIP_INVALID_ARG, "input must be s8, u8 or f32");
+    CHIP_REQUIRE(is_int8(p.out_dt) || p.out_dt == CLDNN_HIP_F32, CLDNN_HIP_INVALID_ARG, "output must be s8, u8 or f32");
+    if (in8) CHIP_REQUIRE(p.w_dt == CLDNN_HIP_S8, CLDNN_HIP_INVALID_ARG, "int8 activations need s8 weights");
+    else CHIP_REQUIRE(p.w_dt == CLDNN_HIP_F32, CLDNN_HIP_INVALID_ARG, "f32 activations need f32 weights");
+
+    // ---- arithmetic mode (reference fused_conv_eltwise_gpu_ref.cl:18-48 and the flags the host emits)
+    Epilogue& e = c->epi;
+    if (d.fused) {
+        if (d.has_wqf) e.mode = MODE_Q;
+        else if (in8 || is_int8(p.out_dt) || is_int8(p.eltw_dt)) e.mode = MODE_FINT;
+        else e.mode = MODE_NAT;
+    } else {
+        e.mode = (d.has_wqf || d.has_calib || d.output_quantization_factor != 1.0f) ? MODE_Q : MODE_NAT;
+    }
+    if (e.mode == MODE_NAT && in8)
+        CHIP_REQUIRE(p.in_dt == CLDNN_HIP_S8 && p.out_dt == CLDNN_HIP_S8, CLDNN_HIP_INVALID_ARG,
+                     "u8 data and precision changes need weights_quantization_factors");
+    const bool calib_on = d.fused ? (d.has_wqf && d.has_calib) : (d.has_calib != 0);
+    e.bias_dt = d.bias_dtype;
+    e.bias_after = (!d.fused && d.has_wqf && bias && d.bias_dtype == CLDNN_HIP_F32) ? 1 : 0;
+    e.oqf_on = d.fused ? 1 : (d.output_quantization_factor != 1.0f);
+    e.iqf = d.input_quantization_factor, e.oqf = d.output_quantization_factor;
+    e.act = d.activation, e.act_m = d.activation_m, e.act_n = d.activation_n;
+    e.fused = d.fused ? 1 : 0;
+    e.ncs = d.non_conv_scale, e.ncs_on = d.fused && d.non_conv_scale != 1.0f;
+    e.eltw_act = d.eltw_activation, e.eltw_m = d.eltw_activation_m, e.eltw_n = d.eltw_activation_n;
+    e.out_dt = p.out_dt, e.eltw_dt = p.eltw_dt, e.in_dt = p.in_dt;
+    e.round_even = d.round_to_even;
+
+    // ---- kernel family
+    const bool blocked = d.input.format == CLDNN_HIP_FMT_FS_B_YX_FSV16 && d.output.format == CLDNN_HIP_FMT_FS_B_YX_FSV16
+                         && (!d.fused || p.eltw_t.format == CLDNN_HIP_FMT_FS_B_YX_FSV16);
+    const bool int_path = in8 && p.w_dt == CLDNN_HIP_S8 && e.mode != MODE_NAT;
+    const bool depthwise = d.groups > 1 && d.groups == d.ifm && d.groups == d.ofm;
+    int impl = d.impl;
+    if (impl == CLDNN_HIP_IMPL_AUTO) {
+        if (blocked && int_path && d.groups == 1) impl = CLDNN_HIP_IMPL_MFMA;
+        else if (blocked && int_path && depthwise) impl = CLDNN_HIP_IMPL_DEPTHWISE;
+        else impl = CLDNN_HIP_IMPL_REF;
+    }
+    if (impl == CLDNN_HIP_IMPL_MFMA)
+        CHIP_REQUIRE(blocked && int_path && d.groups == 1, CLDNN_HIP_UNSUPPORTED_FORMAT,
+                     "the MFMA kernel needs int8 data in fs_b_yx_fsv16, quantisation and groups == 1");
+    if (impl == CLDNN_HIP_IMPL_DEPTHWISE)
+        CHIP_REQUIRE(blocked && int_path && depthwise, CLDNN_HIP_UNSUPPORTED_FORMAT,
+                     "the depthwise kernel needs int8 data in fs_b_yx_fsv16, quantisation and groups == features");
+    c->impl = impl;
+
+    const int ifm_g = p.IFM / p.groups;
+    const size_t wcount = (size_t)p.OFM * ifm_g * p.FY * p.FX;
+    c->engine->make_current();
+
+    // per-feature vectors, zero padded so that vector loads of a partly filled tile stay in bounds
+    const size_t ofm_pad = ((size_t)p.OFM + 255) / 256 * 256;
+    if (wqf) c->wqf = upload(c, wqf, p.OFM * 4, ofm_pad * 4);
+    if (calib && calib_on) c->calib = upload(c, calib, p.OFM * 4, ofm_pad * 4);
+    if (eltw_calib) c->ecal = upload(c, eltw_calib, p.OFM * 4, ofm_pad * 4);
+    e.wqf = (const float*)c->wqf, e.calib = (const float*)c->calib, e.eltw_calib = (const float*)c->ecal;
+
+    cldnn_hip_conv_info& inf = c->info;
+    inf.impl = impl;
+    inf.tile_index = -1;
+    inf.ops = 2ll * p.B * p.OH * p.OW * p.OFM * ifm_g * p.FY * p.FX;
+    inf.bytes = (int64_t)p.B * p.IH * p.IW * p.IFM * (int64_t)dtype_size(p.in_dt)
+                + (int64_t)p.B * p.OH * p.OW * p.OFM * (int64_t)dtype_size(p.out_dt)
+                + (int64_t)wcount * (int64_t)dtype_size(p.w_dt)
+                + 4ll * p.OFM * ((bias ? 1 : 0) + (wqf ? 1 : 0) + (calib ? 1 : 0) + (eltw_calib ? 1 : 0))
+                + (d.fused ? (int64_t)p.B * p.OH * p.OW * p.OFM * (int64_t)dtype_size(p.eltw_dt) : 0);
+
+    if (impl == CLDNN_HIP_IMPL_REF) {
+        c->w_raw = upload(c, weights, wcount * dtype_size(p.w_dt));
+        if (bias) c->bias = upload(c, bias, p.OFM * 4, ofm_pad * 4);
+        e.bias = c->bias;
+        inf.block = 256;
+        inf.grid = (int)(((int64_t)p.B * p.OFM * p.OH * p.OW + 255) / 256);
+        std::snprintf(inf.kernel_name, sizeof(inf.kernel_name), "conv_ref_kernel");
+        return;
+    }
+
+    // ---- accumulator start values: 128*sum(w) for u8 on the signed matrix cores, plus an int32 bias
+    const int8_t* w8 = (const int8_t*)weights;
+    std::vector<int32_t> init(ofm_pad, 0), init_raw(ofm_pad, 0);
+    const bool xor_u8 = impl == CLDNN_HIP_IMPL_MFMA && p.in_dt == CLDNN_HIP_U8;
+    for (int f = 0; f < p.OFM; ++f) {
+        int64_t s = 0;
+        if (xor_u8)
+            for (size_t i = 0; i < (size_t)ifm_g * p.FY * p.FX; ++i) s += w8[(size_t)f * ifm_g * p.FY * p.FX + i];
+        uint32_t v = (uint32_t)(int32_t)(128 * s);
+        init_raw[f] = (int32_t)v;
+        if (bias && d.bias_dtype == CLDNN_HIP_I32 && !e.bias_after) v += (uint32_t)((const int32_t*)bias)[f];
+        init[f] = (int32_t)v;
+    }
+    c->acc_init = upload(c, init.data(), ofm_pad * 4);
+    c->acc_init_raw = upload(c, init_raw.data(), ofm_pad * 4);
+    if (bias && d.bias_dtype == CLDNN_HIP_F32) {
+        c->bias = upload(c, bias, p.OFM * 4, ofm_pad * 4);
+        e.bias = c->bias;
+    } else {
+        e.bias = nullptr;  // folded into acc_init
+        e.bias_dt = CLDNN_HIP_NO_TYPE;
+    }
+
+    if (impl == CLDNN_HIP_IMPL_MFMA) {
+        int tile = d.tile_override > 0 ? d.tile_override - 1 : choose_tile(p, c->engine->props.multiProcessorCount);
+        CHIP_REQUIRE(tile >= 0 && tile < tile_config_count(), CLDNN_HIP_INVALID_ARG, "tile_override out of range");
+        c->mplan = mfma_plan(p, tile);
+        std::vector<int8_t> packed(c->mplan.packed_bytes);
+        std::vector<int32_t> ktab(c->mplan.ksteps * 4);
+        mfma_pack_weights(p, c->mplan, w8, packed.data(), ktab.data());
+        c->w_packed = upload(c, packed.data(), packed.size());
+        c->ktab = upload(c, ktab.data(), ktab.size() * 4);
+        c->epi_kind = mfma_fast_epilogue_ok(p, e, calib_on ? calib : nullptr, eltw_calib, wqf, p.OFM) ? EPI_FAST : EPI_GENERIC;
+        const TileConfig& tc = tile_config(tile);
+        inf.tile_index = tile, inf.tile_pixels = tc.tile_pixels, inf.tile_ofm = tc.tile_ofm;
+        inf.grid = c->mplan.grid, inf.block = 256, inf.lds_bytes = c->mplan.lds_bytes;
+        std::snprintf(inf.kernel_name, sizeof(inf.kernel_name), "conv_mfma_kernel<%d,%d,%d,%s>", tc.tile_pixels,
+                      tc.tile_ofm, tc.wave_pixels, c->epi_kind == EPI_FAST ? "fast" : "generic");
+    } else {
+        c->dplan = dw_plan(p);
+        std::vector<int8_t> packed(c->dplan.packed_bytes);
+        dw_pack_weights(p, w8, packed.data());
+        c->w_packed = upload(c, packed.data(), packed.size());
+        inf.grid = c->dplan.grid * ((p.OFM + 15) / 16), inf.block = c->dplan.block, inf.lds_bytes = p.FY * p.FX * 16;
+        std::snprintf(inf.kernel_name, sizeof(inf.kernel_name), "conv_dw_kernel<%s>", p.in_dt == CLDNN_HIP_U8 ? "u8" : "s8");
+    }
+}
+
+}  // namespace
+
+extern "C" {
+
+int32_t cldnn_hip_conv_out_extent(int32_t in, int32_t pad, int32_t filt, int32_t dil, int32_t stride)
+{
+    return out_extent(in, pad, filt, dil, stride);
+}
+
+int32_t cldnn_hip_tile_config_count(void) { return tile_config_count(); }
+const char* cldnn_hip_tile_config_name(int32_t i)
+{
+    return (i >= 0 && i < tile_config_count()) ? tile_config(i).name : nullptr;
+}
+
+cldnn_hip_status cldnn_hip_conv_create(cldnn_hip_engine e, const cldnn_hip_conv_desc* desc, const void* weights,
+                                       const void* bias, const float* wqf, const float* calib,
+                                       const float* eltw_calib, cldnn_hip_conv* out)
+{
+    return guarded([&] {
+        CHIP_REQUIRE(e && desc && out, CLDNN_HIP_INVALID_ARG, "null argument");
+        *out = nullptr;
+        auto* c = new cldnn_hip_conv_s();
+        c->engine = e;
+        c->desc = *desc;
+        e->refs.fetch_add(1);
+        try {
+            build(c, weights, bias, wqf, calib, eltw_calib);
+        } catch (...) {
+            cldnn_hip_conv_release(c);
+            throw;
+        }
+        *out = c;
+    });
+}
+
+cldnn_hip_status cldnn_hip_conv_release(cldnn_hip_conv c)
+{
+    return guarded([&] {
+        CHIP_REQUIRE(c, CLDNN_HIP_INVALID_ARG, "null convolution");
+        cldnn_hip_engine e = c->engine;
+        (void)hipSetDevice(e->device);
+        (void)hipStreamSynchronize(e->stream);
+        for (void* d : c->owned) (void)hipFree(d);
+        delete c;
+        cldnn_hip_engine_release(e);
+    });
+}
+
+static void run(cldnn_hip_conv c, const void* in, void* out, const void* eltw, int32_t* raw)
+{
+    CHIP_REQUIRE(c && in && (out || raw), CLDNN_HIP_INVALID_ARG, "null argument");
+    const ConvProblem& p = c->p;
+    if (c->desc.fused && !raw) {
+        if (c->desc.second_input_in_output) eltw = out;
+        CHIP_REQUIRE(eltw, CLDNN_HIP_INVALID_ARG, "fused convolution without its second input");
+    }
+    c->engine->make_current();
+    hipStream_t s = c->engine->stream;
+    switch (c->impl) {
+    case CLDNN_HIP_IMPL_REF:
+        launch_conv_ref(s, p, c->epi, in, c->w_raw, eltw, out, raw);
+        break;
+    case CLDNN_HIP_IMPL_MFMA: {
+        MfmaBuffers wb{(const int8_t*)c->w_packed, (const int32_t*)c->ktab};
+        if (raw)
+            launch_conv_mfma(s, p, c->mplan, wb, (const int32_t*)c->acc_init_raw, c->epi, EPI_RAW, in, nullptr, nullptr, raw);
+        else
+            launch_conv_mfma(s, p, c->mplan, wb, (const int32_t*)c->acc_init, c->epi, c->epi_kind, in, eltw, out, nullptr);
+        break;
+    }
+    case CLDNN_HIP_IMPL_DEPTHWISE:
+        launch_conv_dw(s, p, c->dplan, (const int8_t*)c->w_packed,
+                       (const int32_t*)(raw ? c->acc_init_raw : c->acc_init), c->epi, in, eltw, out, raw);
+        break;
+    default: throw error(CLDNN_HIP_ERROR, "convolution without an implementation");
+    }
+}
+
+cldnn_hip_status cldnn_hip_conv_enqueue(cldnn_hip_conv c, const void* input_dev, void* output_dev, const void* eltw_dev)
+{
+    return guarded([&] { run(c, input_dev, output_dev, eltw_dev, nullptr); });
+}
+
+cldnn_hip_status cldnn_hip_conv_accumulators(cldnn_hip_conv c, const void* input_dev, int32_t* acc_dev)
+{
+    return guarded([&] {
+        CHIP_REQUIRE(acc_dev, CLDNN_HIP_INVALID_ARG, "null accumulator buffer");
+        CHIP_REQUIRE(c && c->epi.mode != MODE_NAT, CLDNN_HIP_INVALID_ARG, "accumulators exist in the integer modes only");
+        run(c, input_dev, nullptr, nullptr, acc_dev);
+    });
+}
+
+cldnn_hip_status cldnn_hip_conv_get_info(cldnn_hip_conv c, cldnn_hip_conv_info* info)
+{
+    return guarded([&] {
+        CHIP_REQUIRE(c && info, CLDNN_HIP_INVALID_ARG, "null argument");
+        *info = c->info;
+    });
+}
+
+cldnn_hip_status cldnn_hip_reorder(cldnn_hip_engine e, const void* src_dev, const cldnn_hip_tensor* src, void* dst_dev,
+                                   const cldnn_hip_tensor* dst)
+{
+    return guarded([&] {
+        CHIP_REQUIRE(e && src_dev && src && dst_dev && dst, CLDNN_HIP_INVALID_ARG, "null argument");
+        e->make_current();
+        launch_reorder(e->stream, *src, src_dev, *dst, dst_dev);
+    });
+}
+
+}  // extern "C"

@@ -1,0 +1,235 @@
+/*
+ * cldnn_hip.h -- thin C-ABI HIP layer underneath the clDNN-compatible host
+ * library.  It stands where the reference's OpenCL "gpu toolkit" stands
+ * (engine, buffers, events, kernel enqueue) and additionally exposes the
+ * quantized convolution as a directly callable operator.
+ *
+ * Plain C: opaque handles, pointers and sizes only.  Every function returns
+ * a cldnn_hip_status (0 = success) unless stated otherwise; the message of
+ * the last failure on the calling thread is available from
+ * cldnn_hip_last_error() (same contract as cldnn_get_last_error_message,
+ * reference src/cldnn.cpp:27-33).
+ *
+ * The library never falls back to host computation: without a usable HIP
+ * device every compute entry point fails with CLDNN_HIP_DEVICE_ERROR.
+ */
+#ifndef CLDNN_HIP_H
+#define CLDNN_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef int32_t cldnn_hip_status;
+/* values mirror reference api/C/cldnn.h:70-79 */
+#define CLDNN_HIP_SUCCESS 0
+#define CLDNN_HIP_ERROR -1
+#define CLDNN_HIP_INVALID_ARG -2
+#define CLDNN_HIP_OUT_OF_RESOURCES -3
+#define CLDNN_HIP_DEVICE_ERROR -4
+#define CLDNN_HIP_UNSUPPORTED_SIZE -5
+#define CLDNN_HIP_UNSUPPORTED_FORMAT -6
+#define CLDNN_HIP_DIMENSION_MISMATCH -7
+
+typedef struct cldnn_hip_engine_s* cldnn_hip_engine;
+typedef struct cldnn_hip_buffer_s* cldnn_hip_buffer;
+typedef struct cldnn_hip_event_s* cldnn_hip_event;
+typedef struct cldnn_hip_conv_s* cldnn_hip_conv;
+
+const char* cldnn_hip_last_error(void);
+
+/* ------------------------------------------------------------------ engine
+ * replaces gpu_toolkit construction / device pick
+ * (reference src/gpu/ocl_toolkit.cpp:104-151, src/gpu/ocl_builder.cpp:79-160)
+ * and engine_info (reference src/gpu/engine_info.cpp, api/C/cldnn.h:167-188). */
+typedef struct {
+    uint32_t cores_count;        /* compute units */
+    uint32_t core_frequency;     /* MHz */
+    uint64_t max_work_group_size;
+    uint64_t max_local_mem_size; /* LDS bytes per workgroup */
+    uint64_t max_global_mem_size;
+    uint64_t max_alloc_mem_size;
+    uint32_t wavefront_size;
+    uint32_t xcd_count;          /* accelerator dies (each with its own L2) */
+    char name[64];
+    char arch[32];               /* e.g. "gfx950" */
+} cldnn_hip_engine_info;
+
+uint32_t cldnn_hip_device_count(void);
+cldnn_hip_status cldnn_hip_engine_create(uint32_t device, uint32_t enable_profiling, cldnn_hip_engine* out);
+cldnn_hip_status cldnn_hip_engine_retain(cldnn_hip_engine e);
+cldnn_hip_status cldnn_hip_engine_release(cldnn_hip_engine e);
+cldnn_hip_status cldnn_hip_engine_get_info(cldnn_hip_engine e, cldnn_hip_engine_info* info);
+/* the engine's HIP stream as a void* (hipStream_t); all work of an engine is ordered on it */
+void* cldnn_hip_engine_stream(cldnn_hip_engine e);
+/* replaces gpu_toolkit::flush / finish (reference src/gpu/ocl_toolkit.cpp:291-300) */
+cldnn_hip_status cldnn_hip_engine_flush(cldnn_hip_engine e);
+cldnn_hip_status cldnn_hip_engine_finish(cldnn_hip_engine e);
+/* bytes currently / at most allocated through this engine (reference src/include/engine_impl.h:123-124) */
+int64_t cldnn_hip_engine_used_memory(cldnn_hip_engine e);
+int64_t cldnn_hip_engine_max_used_memory(cldnn_hip_engine e);
+
+/* ------------------------------------------------------------------ buffers
+ * replaces gpu_buffer (reference src/gpu/memory_gpu.cpp:37-90): zero-filled at
+ * allocation; lock() hands out a host pointer valid for read AND write,
+ * reference-counted; the first lock copies device -> pinned shadow, the last
+ * unlock copies the shadow back to the device. */
+cldnn_hip_status cldnn_hip_buffer_alloc(cldnn_hip_engine e, size_t bytes, cldnn_hip_buffer* out);
+cldnn_hip_status cldnn_hip_buffer_retain(cldnn_hip_buffer b);
+cldnn_hip_status cldnn_hip_buffer_release(cldnn_hip_buffer b);
+void* cldnn_hip_buffer_lock(cldnn_hip_buffer b);     /* NULL on failure */
+cldnn_hip_status cldnn_hip_buffer_unlock(cldnn_hip_buffer b);
+/* gpu_buffer::fill (reference src/gpu/memory_gpu.cpp:87-90) */
+cldnn_hip_status cldnn_hip_buffer_fill(cldnn_hip_buffer b, uint8_t pattern);
+void* cldnn_hip_buffer_device_ptr(cldnn_hip_buffer b);
+size_t cldnn_hip_buffer_size(cldnn_hip_buffer b);
+/* direct copies ordered on the engine stream (blocking) */
+cldnn_hip_status cldnn_hip_buffer_write(cldnn_hip_buffer b, size_t offset, const void* host, size_t bytes);
+cldnn_hip_status cldnn_hip_buffer_read(cldnn_hip_buffer b, size_t offset, void* host, size_t bytes);
+
+/* ------------------------------------------------------------------ events
+ * replaces base_event / user_event / events_pool
+ * (reference src/gpu/ocl_base_event.cpp:23-159, src/gpu/ocl_user_event.cpp, src/gpu/events_pool.h:25-139). */
+typedef void (*cldnn_hip_event_handler)(void*);
+cldnn_hip_status cldnn_hip_event_create_user(cldnn_hip_engine e, uint32_t set, cldnn_hip_event* out);
+/* marker after everything enqueued so far (gpu_toolkit::enqueue_marker, reference src/gpu/ocl_toolkit.cpp:197-230) */
+cldnn_hip_status cldnn_hip_event_record(cldnn_hip_engine e, cldnn_hip_event* out);
+/* bracket the work enqueued between the two calls; with profiling enabled the event then carries
+ * its execution time (reference src/gpu/ocl_toolkit.cpp:170-178 returns such an event per kernel) */
+cldnn_hip_status cldnn_hip_event_record_begin(cldnn_hip_engine e, cldnn_hip_event* out);
+cldnn_hip_status cldnn_hip_event_record_end(cldnn_hip_event ev);
+cldnn_hip_status cldnn_hip_event_retain(cldnn_hip_event ev);
+cldnn_hip_status cldnn_hip_event_release(cldnn_hip_event ev);
+cldnn_hip_status cldnn_hip_event_wait(cldnn_hip_event ev);
+int32_t cldnn_hip_event_is_set(cldnn_hip_event ev);
+int32_t cldnn_hip_event_is_user(cldnn_hip_event ev);
+cldnn_hip_status cldnn_hip_event_set(cldnn_hip_event ev);
+cldnn_hip_status cldnn_hip_event_add_handler(cldnn_hip_event ev, cldnn_hip_event_handler h, void* param);
+/* "executing" interval in ns (reference src/gpu/ocl_base_event.cpp:68-96); 0 when profiling is off */
+cldnn_hip_status cldnn_hip_event_elapsed_ns(cldnn_hip_event ev, uint64_t* ns);
+/* make the engine stream wait for events before later work (gpu_toolkit::sync_events, reference src/gpu/ocl_toolkit.cpp:313-346) */
+cldnn_hip_status cldnn_hip_engine_wait_events(cldnn_hip_engine e, const cldnn_hip_event* evs, size_t n);
+
+/* ------------------------------------------------------------------ tensors */
+enum { CLDNN_HIP_S8 = 0, CLDNN_HIP_U8 = 1, CLDNN_HIP_I32 = 2, CLDNN_HIP_F32 = 3, CLDNN_HIP_NO_TYPE = -1 };
+
+enum {
+    CLDNN_HIP_FMT_BFYX = 0,
+    CLDNN_HIP_FMT_YXFB = 1,
+    CLDNN_HIP_FMT_BYXF = 2,
+    /* [fs][b][y][x][16 features]: the 16-byte feature slice of one pixel is one lane's
+       int8 MFMA K-fragment and one 128-bit load.  Chosen by the layout rule that replaces
+       byxf_af32 / fs_bs_yx_bsv4_fsv32 (reference src/layout_optimizer.cpp:187-291,
+       kernel_selector/core/cl_kernels/include/fetch.cl:126-196). */
+    CLDNN_HIP_FMT_FS_B_YX_FSV16 = 3,
+    /* [b][fs][y][x][4 features] (reference fetch.cl:453-476) */
+    CLDNN_HIP_FMT_B_FS_YX_FSV4 = 4
+};
+
+/* logical size + physical spatial/feature padding (reference api/CPP/layout.hpp:387-433) */
+typedef struct {
+    int32_t dtype;
+    int32_t format;
+    int32_t b, f, y, x;
+    int32_t pad_lo_b, pad_lo_f, pad_lo_y, pad_lo_x;
+    int32_t pad_hi_b, pad_hi_f, pad_hi_y, pad_hi_x;
+} cldnn_hip_tensor;
+
+/* bytes a buffer for this tensor must have */
+size_t cldnn_hip_tensor_bytes(const cldnn_hip_tensor* t);
+/* element index of logical (b,f,y,x) inside the buffer (get_linear_offset, reference api/CPP/layout.hpp:407-433) */
+int64_t cldnn_hip_tensor_offset(const cldnn_hip_tensor* t, int32_t b, int32_t f, int32_t y, int32_t x);
+
+/* layout / precision change; replaces the reorder kernels the path needs
+ * (reference src/gpu/reorder_gpu.cpp, kernel_selector/core/cl_kernels/reorder_data.cl).
+ * f32 -> int8 conversions saturate and round half away from zero; padding of dst is left untouched. */
+cldnn_hip_status cldnn_hip_reorder(cldnn_hip_engine e, const void* src_dev, const cldnn_hip_tensor* src,
+                                   void* dst_dev, const cldnn_hip_tensor* dst);
+
+/* ------------------------------------------------------------------ convolution
+ * One object per convolution / fused_conv_eltwise node; replaces
+ * convolution_gpu::create + kernel selection + weight reordering
+ * (reference src/gpu/convolution_gpu.cpp:71-162, src/gpu/fused_conv_eltwise_gpu.cpp:70-200,
+ *  kernel_selector/core/kernel_selector.cpp:80-207, src/graph_optimizer/post_optimize_weights.cpp:36-66)
+ * and, at run time, execute_impl (reference src/gpu/primitive_gpu_base.h:117-168).
+ * Arithmetic follows the reference semantic kernel
+ * (kernel_selector/core/cl_kernels/fused_conv_eltwise_gpu_ref.cl:93-233). */
+enum { CLDNN_HIP_ACT_NONE = 0, CLDNN_HIP_ACT_RELU = 1, CLDNN_HIP_ACT_RELU_SLOPE = 2, CLDNN_HIP_ACT_CLAMP = 3 };
+
+/* which kernel family may be used */
+enum {
+    CLDNN_HIP_IMPL_AUTO = 0,      /* tile-config table decides */
+    CLDNN_HIP_IMPL_REF = 1,       /* one work-item per output, any layout */
+    CLDNN_HIP_IMPL_MFMA = 2,      /* implicit GEMM on int8 MFMA, fs_b_yx_fsv16 */
+    CLDNN_HIP_IMPL_DEPTHWISE = 3  /* bandwidth kernel, fs_b_yx_fsv16, groups == features */
+};
+
+typedef struct {
+    cldnn_hip_tensor input;       /* activations */
+    cldnn_hip_tensor output;      /* logical size must equal the computed output size */
+    cldnn_hip_tensor eltw;        /* second input of fused_conv_eltwise (ignored unless fused) */
+    int32_t weights_dtype;        /* CLDNN_HIP_S8 (or F32 for the float reference path) */
+    int32_t bias_dtype;           /* CLDNN_HIP_I32 / F32 / NO_TYPE */
+    int32_t ofm, ifm;             /* totals over all groups */
+    int32_t fy, fx;
+    int32_t stride_y, stride_x;
+    int32_t dilation_y, dilation_x;
+    int32_t pad_y, pad_x;         /* = max(-input_offset, 0) */
+    int32_t groups;
+    int32_t has_wqf;              /* weights_quantization_factors given */
+    int32_t has_calib;            /* output_calibration_factors given */
+    float input_quantization_factor;
+    float output_quantization_factor;
+    int32_t activation;           /* CLDNN_HIP_ACT_* applied to the dequantised conv result */
+    float activation_m, activation_n;
+    /* fused_conv_eltwise part */
+    int32_t fused;
+    float non_conv_scale;
+    int32_t eltw_activation;
+    float eltw_activation_m, eltw_activation_n;
+    int32_t has_eltw_calib;
+    int32_t eltw_stride_y, eltw_stride_x;
+    int32_t second_input_in_output; /* residual is read from the output buffer itself */
+    int32_t round_to_even;        /* 0 = reference behaviour (half away from zero) */
+    int32_t impl;                 /* CLDNN_HIP_IMPL_* */
+    int32_t tile_override;        /* 0 = table; otherwise index+1 into the tile-config table (tuning / tests) */
+} cldnn_hip_conv_desc;
+
+/* Host pointers: weights [ofm][ifm/groups][fy][fx] dense, bias/wqf/calib/eltw_calib [ofm] or NULL.
+ * Everything is copied / pre-packed into device memory owned by the object. */
+cldnn_hip_status cldnn_hip_conv_create(cldnn_hip_engine e, const cldnn_hip_conv_desc* desc, const void* weights,
+                                       const void* bias, const float* wqf, const float* calib,
+                                       const float* eltw_calib, cldnn_hip_conv* out);
+cldnn_hip_status cldnn_hip_conv_release(cldnn_hip_conv c);
+/* asynchronous on the engine stream; device pointers */
+cldnn_hip_status cldnn_hip_conv_enqueue(cldnn_hip_conv c, const void* input_dev, void* output_dev,
+                                        const void* eltw_dev);
+/* raw int32 accumulators (before bias), dense [b][ofm][oy][ox]; test / verification hook */
+cldnn_hip_status cldnn_hip_conv_accumulators(cldnn_hip_conv c, const void* input_dev, int32_t* acc_dev);
+
+typedef struct {
+    int32_t impl;                 /* CLDNN_HIP_IMPL_* actually chosen */
+    int32_t tile_index;           /* row of the tile-config table (-1 when not applicable) */
+    int32_t tile_pixels, tile_ofm;
+    int32_t grid, block;
+    int32_t lds_bytes;
+    int64_t ops;                  /* 2*B*OY*OX*OFM*(IFM/groups)*FY*FX */
+    int64_t bytes;                /* algorithmic bytes: input + output + weights + per-ofm vectors (+ residual) */
+    char kernel_name[96];
+} cldnn_hip_conv_info;
+cldnn_hip_status cldnn_hip_conv_get_info(cldnn_hip_conv c, cldnn_hip_conv_info* info);
+
+/* computed output extent along one axis (reference src/include/sliding_window_utils.h:90-129) */
+int32_t cldnn_hip_conv_out_extent(int32_t in, int32_t pad, int32_t filt, int32_t dil, int32_t stride);
+
+/* number of rows of the gfx950 tile-config table and a printable description of one row */
+int32_t cldnn_hip_tile_config_count(void);
+const char* cldnn_hip_tile_config_name(int32_t index);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

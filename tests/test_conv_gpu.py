@@ -1,0 +1,316 @@
+"""Parity of the HIP convolution (through the C-ABI) with the CPU oracle and with the
+reference's known-answer tables.  Integer results must be bit-exact; float outputs are
+compared at 1e-5 relative (they are the same sequence of float operations)."""
+import numpy as np
+import pytest
+
+import kat
+from cldnn_amd import hip
+from oracle import refconv as rc
+
+pytestmark = pytest.mark.gpu
+K = kat.load()
+
+
+@pytest.fixture(scope="module")
+def eng():
+    e = hip.Engine()
+    yield e
+    e.close()
+
+
+def both(eng, x, w, bias=None, wqf=None, calib=None, fmt="bfyx", impl=hip.IMPL_AUTO, tile=0, in_pad=(0, 0),
+         out_pad=(0, 0), acc=True, **kw):
+    ref = rc.conv(x, w, bias, wqf=wqf, calib=calib, want_acc=acc, **kw)
+    got = hip.conv_forward(eng, x, w, bias, wqf, calib, fmt=fmt, impl=impl, tile=tile, in_pad=in_pad, out_pad=out_pad,
+                           want_acc=acc, want_info=True, **kw)
+    return ref, got
+
+
+def assert_same(ref_out, got_out):
+    assert ref_out.shape == got_out.shape and ref_out.dtype == got_out.dtype
+    if ref_out.dtype == np.float32:
+        np.testing.assert_allclose(got_out, ref_out, rtol=1e-5, atol=0)
+    else:
+        bad = np.argwhere(ref_out != got_out)
+        assert bad.size == 0, "first mismatch at %s: ref %s got %s (%d of %d differ)" % (
+            bad[0], ref_out[tuple(bad[0])], got_out[tuple(bad[0])], len(bad), ref_out.size)
+
+
+# ------------------------------------------------------------------ the reference's own tables
+@pytest.mark.parametrize("fmt", ["bfyx", "fs_b_yx_fsv16"])
+@pytest.mark.parametrize("case", K["conv_quantized"], ids=lambda c: c["name"])
+def test_kat_conv_quantized(eng, case, fmt):
+    p = kat.diag_problem(case)
+    out = hip.conv_forward(eng, p["x"], p["w"], p["bias"], p["wqf"], out_dt=case["out_dt"], act="relu", fmt=fmt)
+    if case["out_dt"] == "f32":
+        np.testing.assert_allclose(out, p["expected"], atol=case["tol"], rtol=0)
+    else:
+        np.testing.assert_array_equal(out.astype(np.int64), p["expected"].astype(np.int64))
+
+
+@pytest.mark.parametrize("fmt", ["bfyx", "fs_b_yx_fsv16"])
+@pytest.mark.parametrize("case", K["fused"], ids=lambda c: c["name"])
+def test_kat_fused(eng, case, fmt):
+    if fmt != "bfyx" and case["in_dt"] == "f32":
+        pytest.skip("the blocked int8 layout carries int8 data")
+    p = kat.diag_problem(case, fused=True)
+    out = hip.conv_forward(eng, p["x"], p["w"], p["bias"],
+                           p["wqf"] if case["pass_wqf"] else None,
+                           p["conv_calib"] if case["pass_conv_calib"] else None,
+                           out_dt=case["out_dt"], act="none", eltw=p["nci"],
+                           non_conv_scale=float(p["non_conv_scale"]), eltw_act="relu",
+                           eltw_calib=p["eltw_calib"] if case["pass_eltw_calib"] else None, fmt=fmt)
+    if case["out_dt"] == "f32":
+        np.testing.assert_allclose(out, p["expected"], atol=case["tol"], rtol=0)
+    else:
+        np.testing.assert_array_equal(out.astype(np.int64), p["expected"].astype(np.int64))
+
+
+@pytest.mark.parametrize("case", K["indexing"], ids=lambda c: c["name"])
+def test_kat_indexing(eng, case):
+    p = kat.indexing_problem(case, K["indexing"])
+    out = hip.conv_forward(eng, p["x"], p["w"], p["bias"], stride=p["stride"], pad=p["pad"], groups=p["groups"],
+                           act=p["act"])
+    assert out.shape == p["expected"].shape
+    np.testing.assert_allclose(out.astype(np.float64), p["expected"], atol=max(p["tol"], 1e-5), rtol=0)
+
+
+# ------------------------------------------------------------------ seeded random problems vs the oracle
+def problem(seed, B, IFM, H, W, OFM, FY, FX, in_dt=np.uint8, groups=1, spread=True):
+    r = np.random.default_rng(seed)
+    lo, hi = (0, 256) if in_dt == np.uint8 else (-128, 128)
+    x = r.integers(lo, hi, (B, IFM, H, W)).astype(in_dt)
+    w = r.integers(-127, 128, (OFM, IFM // groups, FY, FX)).astype(np.int8)
+    bias = r.integers(-1000, 1001, OFM).astype(np.int32)
+    k = (IFM // groups) * FY * FX
+    sigma = np.sqrt(k) * 147.4 * 73.3 if in_dt == np.uint8 else np.sqrt(k) * 73.9 * 73.3
+    if spread:  # outputs spread over the int8 range so rounding and both saturation ends are hit
+        calib = (40.0 / sigma * r.uniform(0.5, 2.0, OFM)).astype(np.float32)
+    else:       # the benchmark's data: log-uniform in [1e-4, 1e-2]
+        calib = np.exp(r.uniform(np.log(1e-4), np.log(1e-2), OFM)).astype(np.float32)
+    wqf = np.ones(OFM, np.float32)
+    return x, w, bias, wqf, calib
+
+
+SHAPES = [
+    # B IFM H  W  OFM FY FX stride pad
+    (1, 64, 56, 56, 64, 3, 3, (1, 1), (1, 1)),     # BASELINE config 1
+    (2, 64, 14, 14, 256, 1, 1, (1, 1), (0, 0)),
+    (3, 256, 14, 14, 128, 1, 1, (2, 2), (0, 0)),   # strided 1x1
+    (2, 32, 9, 11, 48, 3, 3, (1, 1), (1, 1)),      # ragged: ofm 48, odd sizes
+    (1, 3, 32, 32, 64, 7, 7, (2, 2), (3, 3)),      # stem shape, IFM = 3
+    (2, 128, 7, 7, 128, 3, 3, (1, 1), (1, 1)),
+    (1, 40, 10, 6, 24, 5, 3, (2, 1), (2, 1)),      # ifm 40 -> 3 slices, asymmetric filter
+    (1, 16, 5, 5, 16, 1, 1, (1, 1), (0, 0)),       # one k-chunk: padded K-step
+]
+
+
+@pytest.mark.parametrize("shape", SHAPES, ids=lambda s: "x".join(map(str, s[:7])))
+@pytest.mark.parametrize("in_dt", [np.uint8, np.int8], ids=["u8", "s8"])
+def test_ref_kernel_bfyx(eng, shape, in_dt):
+    B, IFM, H, W, OFM, FY, FX, stride, pad = shape
+    x, w, bias, wqf, calib = problem(11, B, IFM, H, W, OFM, FY, FX, in_dt)
+    (ro, ra), (go, ga, info) = both(eng, x, w, bias, wqf, calib, stride=stride, pad=pad, out_dt="s8", act="relu")
+    assert info.impl == hip.IMPL_REF
+    np.testing.assert_array_equal(ga, ra)
+    assert_same(ro, go)
+
+
+def tiles():
+    return list(range(1, hip.lib().cldnn_hip_tile_config_count() + 1))
+
+
+@pytest.mark.parametrize("shape", SHAPES, ids=lambda s: "x".join(map(str, s[:7])))
+@pytest.mark.parametrize("in_dt", [np.uint8, np.int8], ids=["u8", "s8"])
+def test_mfma_kernel_all_tiles(eng, shape, in_dt):
+    B, IFM, H, W, OFM, FY, FX, stride, pad = shape
+    x, w, bias, wqf, calib = problem(12, B, IFM, H, W, OFM, FY, FX, in_dt)
+    ref_o, ref_a = rc.conv(x, w, bias, wqf=wqf, calib=calib, stride=stride, pad=pad, out_dt="s8", act="relu",
+                           want_acc=True)
+    for tile in [0] + tiles():
+        go, ga, info = hip.conv_forward(eng, x, w, bias, wqf, calib, stride=stride, pad=pad, out_dt="s8", act="relu",
+                                        fmt="fs_b_yx_fsv16", tile=tile, want_acc=True, want_info=True)
+        assert info.impl == hip.IMPL_MFMA, info.kernel_name
+        assert b"fast" in info.kernel_name
+        np.testing.assert_array_equal(ga, ref_a, err_msg=info.kernel_name.decode())
+        assert_same(ref_o, go)
+
+
+@pytest.mark.parametrize("out_dt", ["s8", "u8", "f32"])
+@pytest.mark.parametrize("act", [("none", 0, 0), ("relu", 0, 0), ("relu_slope", 0.1, 0), ("clamp", 0.0, 6.0)],
+                         ids=lambda a: a[0])
+def test_mfma_generic_epilogue_variants(eng, out_dt, act):
+    x, w, bias, wqf, calib = problem(13, 2, 64, 12, 12, 96, 3, 3)
+    r = np.random.default_rng(3)
+    wqf = (3.0 / (np.sqrt(576) * 147.4 * 73.3) * r.uniform(0.5, 2, 96)).astype(np.float32)
+    calib = np.full(96, 127 / 6, np.float32) * r.uniform(0.9, 1.1, 96).astype(np.float32)
+    calib[::7] *= -1  # negative scale: not eligible for the short epilogue
+    kw = dict(stride=(1, 1), pad=(1, 1), out_dt=out_dt, act=act[0], act_m=act[1], act_n=act[2], iqf=0.75)
+    (ro, ra), (go, ga, info) = both(eng, x, w, bias, wqf, calib, fmt="fs_b_yx_fsv16", **kw)
+    assert b"generic" in info.kernel_name
+    np.testing.assert_array_equal(ga, ra)
+    assert_same(ro, go)
+
+
+def test_mfma_f32_bias_added_after_dequantisation(eng):
+    x, w, _, wqf, calib = problem(14, 1, 32, 8, 8, 32, 3, 3, np.int8)
+    bias = np.random.default_rng(1).uniform(-50, 50, 32).astype(np.float32)
+    wqf = np.full(32, 1e-3, np.float32)
+    (ro, ra), (go, ga, info) = both(eng, x, w, bias, wqf, None, fmt="fs_b_yx_fsv16", pad=(1, 1), out_dt="f32")
+    np.testing.assert_array_equal(ga, ra)
+    assert_same(ro, go)
+
+
+def test_mfma_round_to_even_variant(eng):
+    case = next(c for c in K["conv_quantized"] if c["name"] == "i8_to_u8")
+    p = kat.diag_problem(case)
+    got = hip.conv_forward(eng, p["x"], p["w"], p["bias"], p["wqf"], out_dt="u8", act="relu", fmt="fs_b_yx_fsv16",
+                           round_even=True)
+    ref = rc.conv(p["x"], p["w"], p["bias"], wqf=p["wqf"], out_dt="u8", act="relu", round_even=True)
+    np.testing.assert_array_equal(got, ref)
+    assert got[0, 5, 0, 1] == 126  # 126.5 -> 126 under round-to-even, 127 in the reference
+
+
+@pytest.mark.parametrize("fast", [True, False], ids=["fast", "generic"])
+@pytest.mark.parametrize("eltw_dt", [np.int8, np.uint8], ids=["s8", "u8"])
+def test_mfma_fused_eltwise(eng, fast, eltw_dt):
+    x, w, bias, wqf, calib = problem(15, 2, 64, 14, 14, 256, 1, 1)
+    r = np.random.default_rng(5)
+    lo, hi = (-128, 128) if eltw_dt == np.int8 else (0, 256)
+    e = r.integers(lo, hi, (2, 256, 14, 14)).astype(eltw_dt)
+    ecal = r.uniform(0.3, 1.2, 256).astype(np.float32)
+    kw = dict(out_dt="s8", act="none", eltw=e, eltw_act="relu", eltw_calib=ecal,
+              non_conv_scale=1.0 if fast else 0.5)
+    (ro, ra), (go, ga, info) = both(eng, x, w, bias, wqf, calib, fmt="fs_b_yx_fsv16", **kw)
+    assert (b"fast" in info.kernel_name) == fast
+    np.testing.assert_array_equal(ga, ra)
+    assert_same(ro, go)
+
+
+def test_mfma_padded_buffers(eng):
+    # physical zero borders on input and output (what a following 3x3 layer asks of its producer)
+    x, w, bias, wqf, calib = problem(16, 2, 64, 14, 14, 64, 3, 3)
+    kw = dict(stride=(1, 1), pad=(1, 1), out_dt="s8", act="relu")
+    (ro, ra), (go, ga, info) = both(eng, x, w, bias, wqf, calib, fmt="fs_b_yx_fsv16", in_pad=(1, 1), out_pad=(1, 2), **kw)
+    np.testing.assert_array_equal(ga, ra)
+    assert_same(ro, go)
+
+
+def test_output_border_stays_zero(eng):
+    x, w, bias, wqf, calib = problem(17, 1, 32, 6, 6, 32, 1, 1)
+    xin = hip.upload(eng, x, "fs_b_yx_fsv16")
+    d = hip.conv_desc(xin.tensor, w.shape, "s8", out_pad=(1, 1), bias_dt=hip.I32, has_wqf=True, has_calib=True, act="relu")
+    c = hip.Conv(eng, d, w, bias, wqf, calib)
+    out = hip.Buffer(eng, d.output)
+    c.enqueue(xin, out)
+    eng.finish()
+    raw = out.read_raw().reshape(2, 1, 8, 8, 16)
+    assert raw[:, :, 0].any() == 0 and raw[:, :, -1].any() == 0 and raw[:, :, :, 0].any() == 0 and raw[:, :, :, -1].any() == 0
+    assert raw[:, :, 1:-1, 1:-1].any()
+
+
+@pytest.mark.parametrize("shape", [(2, 32, 20, 20, 3, 1, 1), (1, 96, 15, 17, 3, 2, 1), (2, 144, 9, 9, 5, 1, 2),
+                                   (1, 960, 7, 7, 3, 1, 1)], ids=lambda s: "x".join(map(str, s)))
+@pytest.mark.parametrize("in_dt", [np.uint8, np.int8], ids=["u8", "s8"])
+def test_depthwise_kernel(eng, shape, in_dt):
+    B, C, H, W, F, s, p = shape
+    x, w, bias, wqf, calib = problem(18, B, C, H, W, C, F, F, in_dt, groups=C)
+    r = np.random.default_rng(2)
+    sig = np.sqrt(F * F) * 147.4 * 73.3
+    wqf = (3.0 / sig * r.uniform(0.5, 2, C)).astype(np.float32)
+    calib = np.full(C, 127 / 6, np.float32)
+    kw = dict(stride=(s, s), pad=(p, p), groups=C, out_dt="s8", act="clamp", act_m=0.0, act_n=6.0)
+    (ro, ra), (go, ga, info) = both(eng, x, w, bias, wqf, calib, fmt="fs_b_yx_fsv16", **kw)
+    assert info.impl == hip.IMPL_DEPTHWISE
+    np.testing.assert_array_equal(ga, ra)
+    assert_same(ro, go)
+    # the layout-agnostic kernel must agree as well (grouped path, one launch)
+    (ro2, _), (go2, _, info2) = both(eng, x, w, bias, wqf, calib, fmt="bfyx", acc=True, **kw)
+    assert info2.impl == hip.IMPL_REF
+    assert_same(ro2, go2)
+
+
+def test_benchmark_calibration_data(eng):
+    # the benchmark's own factor distribution (mostly saturated outputs) on config 1
+    x, w, bias, wqf, calib = problem(19, 1, 64, 56, 56, 64, 3, 3, spread=False)
+    (ro, ra), (go, ga, info) = both(eng, x, w, bias, wqf, calib, fmt="fs_b_yx_fsv16", pad=(1, 1), out_dt="s8", act="relu")
+    np.testing.assert_array_equal(ga, ra)
+    assert_same(ro, go)
+
+
+@pytest.mark.parametrize("fmt", ["yxfb", "byxf", "fs_b_yx_fsv16", "b_fs_yx_fsv4"])
+def test_reorder_round_trip_and_layout_independence(eng, fmt):
+    r = np.random.default_rng(20)
+    x = r.integers(0, 256, (2, 21, 5, 7)).astype(np.uint8)
+    buf = hip.upload(eng, x, fmt, (1, 2))
+    np.testing.assert_array_equal(hip.download(eng, buf), x)
+    # raw bytes sit where the layout formula says
+    raw = buf.read_raw()
+    import ctypes as C
+    L = hip.lib()
+    for (b, f, y, xx) in [(0, 0, 0, 0), (1, 20, 4, 6), (1, 16, 2, 3), (0, 5, 1, 1)]:
+        assert raw[L.cldnn_hip_tensor_offset(C.byref(buf.tensor), b, f, y, xx)] == x[b, f, y, xx]
+    # result of a convolution does not depend on the storage layout
+    w = r.integers(-127, 128, (8, 21, 3, 3)).astype(np.int8)
+    one = np.ones(8, np.float32)
+    a = hip.conv_forward(eng, x, w, None, one, pad=(1, 1), out_dt="f32", fmt="bfyx")
+    b_ = hip.conv_forward(eng, x, w, None, one, pad=(1, 1), out_dt="f32", fmt=fmt)
+    np.testing.assert_array_equal(a, b_)
+
+
+def test_reorder_f32_to_int8_rounds_half_away_and_saturates(eng):
+    v = np.array([0.5, 1.5, -0.5, -1.5, 2.4, 300.0, -300.0, 127.5], np.float32).reshape(1, 8, 1, 1)
+    src = hip.upload(eng, v)
+    dst = hip.Buffer(eng, hip.Tensor.make("s8", "bfyx", 1, 8, 1, 1))
+    hip.reorder(eng, src, dst)
+    np.testing.assert_array_equal(hip.download(eng, dst).ravel(), [1, 2, -1, -2, 2, 127, -128, 127])
+
+
+def test_lock_unlock_and_events(eng):
+    import ctypes as C
+    L = hip.lib()
+    t = hip.Tensor.make("u8", "bfyx", 1, 1, 4, 4)
+    b = hip.Buffer(eng, t)
+    p = L.cldnn_hip_buffer_lock(b.h)
+    assert p
+    host = (C.c_uint8 * 16).from_address(p)
+    assert list(host) == [0] * 16  # zero-initialised at allocation
+    for i in range(16):
+        host[i] = i
+    hip.check(L.cldnn_hip_buffer_unlock(b.h))
+    np.testing.assert_array_equal(b.read_raw(), np.arange(16, dtype=np.uint8))
+    ev = C.c_void_p()
+    hip.check(L.cldnn_hip_event_record(eng.h, C.byref(ev)))
+    hip.check(L.cldnn_hip_event_wait(ev))
+    assert L.cldnn_hip_event_is_set(ev) == 1
+    hip.check(L.cldnn_hip_event_release(ev))
+    uev = C.c_void_p()
+    hip.check(L.cldnn_hip_event_create_user(eng.h, 0, C.byref(uev)))
+    assert L.cldnn_hip_event_is_set(uev) == 0 and L.cldnn_hip_event_is_user(uev) == 1
+    fired = []
+    cb = hip.EVENT_HANDLER(lambda _: fired.append(1))
+    hip.check(L.cldnn_hip_event_add_handler(uev, cb, None))
+    hip.check(L.cldnn_hip_event_set(uev))
+    assert fired == [1] and L.cldnn_hip_event_is_set(uev) == 1
+    hip.check(L.cldnn_hip_event_release(uev))
+
+
+def test_error_paths(eng):
+    x = np.zeros((1, 16, 4, 4), np.uint8)
+    w = np.zeros((16, 16, 3, 3), np.int8)
+    xin = hip.upload(eng, x, "fs_b_yx_fsv16")
+    d = hip.conv_desc(xin.tensor, w.shape, "s8", pad=(1, 1), has_wqf=True)
+    d.output.y += 1
+    with pytest.raises(hip.HipError) as ei:
+        hip.Conv(eng, d, w, None, np.ones(16, np.float32))
+    assert ei.value.status == -7
+    d = hip.conv_desc(xin.tensor, w.shape, "s8", pad=(1, 1), has_wqf=False)  # u8 without quantisation
+    with pytest.raises(hip.HipError) as ei:
+        hip.Conv(eng, d, w)
+    assert ei.value.status == -2
+    d = hip.conv_desc(xin.tensor, w.shape, "s8", pad=(1, 1), has_wqf=True, groups=2, impl=hip.IMPL_MFMA)
+    d.ifm = 16
+    with pytest.raises(hip.HipError) as ei:
+        hip.Conv(eng, d, np.zeros((16, 8, 3, 3), np.int8), None, np.ones(16, np.float32))
+    assert ei.value.status == -6
