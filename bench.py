@@ -1,0 +1,280 @@
+#!/usr/bin/env python3
+"""Benchmark of the quantized convolution hot path on one MI355X.
+
+A "step" is one pass of a whole int8 convolution stack over one batch of synthetic input:
+every layer is one launch of the HIP convolution through the C-ABI, inputs already resident in
+HBM.  Default workload: the 53 convolutions of ResNet-50 at batch 32 with the residual add fused
+into the 16 block-closing 1x1 convolutions (fused_conv_eltwise).
+
+Prints ONE JSON line (metric, value, roofline, cpu_baseline, ...).
+"""
+import argparse
+import ctypes as C
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+from cldnn_amd import hip, workloads  # noqa: E402
+
+PEAK_INT8_OPS = 5.0e15   # MI355X dense int8 MFMA peak, op/s
+PEAK_HBM = 8.0e12        # bytes/s
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+class Layer:
+    pass
+
+
+def build_stack(eng, layers, batch, fuse_residual, seed=1337, tile=0, in_dt=np.uint8):
+    """Create device tensors and convolution objects for every layer (seeded synthetic data)."""
+    out = []
+    for i, l in enumerate(layers):
+        r = np.random.default_rng(seed + i)
+        L = Layer()
+        L.spec = l
+        ifm, ofm, k, g = l["ifm"], l["ofm"], l["k"], l["groups"]
+        hw, ohw = l["in_hw"], l["out_hw"]
+        lo, hi = (0, 256) if in_dt == np.uint8 else (-128, 128)
+        L.x = r.integers(lo, hi, (batch, ifm, hw, hw), dtype=np.int16).astype(in_dt)
+        L.w = r.integers(-127, 128, (ofm, ifm // g, k, k), dtype=np.int16).astype(np.int8)
+        L.bias = r.integers(-1000, 1001, ofm).astype(np.int32)
+        L.wqf = np.ones(ofm, np.float32)
+        L.calib = np.exp(r.uniform(np.log(1e-4), np.log(1e-2), ofm)).astype(np.float32)
+        L.fused = bool(fuse_residual and l["closes_block"])
+        L.eltw = L.ecal = None
+        act = l["act"]
+        kw = dict(stride=(l["stride"],) * 2, pad=(l["pad"],) * 2, groups=g, bias_dt=hip.I32, has_wqf=True, has_calib=True)
+        if act == "relu6":
+            kw.update(act="clamp", act_m=0.0, act_n=6.0)
+            # the clamp acts on the dequantised value: scale it into range, requantise with 127/6
+            sig = np.sqrt((ifm // g) * k * k) * 147.4 * 73.3
+            L.wqf = (3.0 / sig * r.uniform(0.5, 2.0, ofm)).astype(np.float32)
+            L.calib = np.full(ofm, 127.0 / 6.0, np.float32)
+        else:
+            kw.update(act=act)
+        L.xin = hip.upload(eng, L.x, "fs_b_yx_fsv16")
+        L.ein = None
+        if L.fused:
+            L.eltw = r.integers(-128, 128, (batch, ofm, ohw, ohw), dtype=np.int16).astype(np.int8)
+            L.ecal = r.uniform(0.25, 1.0, ofm).astype(np.float32)
+            L.ein = hip.upload(eng, L.eltw, "fs_b_yx_fsv16")
+            kw.update(act="none", eltw_t=L.ein.tensor, eltw_act="relu", has_eltw_calib=True)
+        L.kw = kw
+        L.desc = hip.conv_desc(L.xin.tensor, L.w.shape, "s8", tile=tile, **kw)
+        L.conv = hip.Conv(eng, L.desc, L.w, L.bias, L.wqf, L.calib, L.ecal)
+        L.out = hip.Buffer(eng, L.desc.output)
+        L.info = L.conv.info()
+        out.append(L)
+    return out
+
+
+def run_step(stack):
+    enq = hip.lib().cldnn_hip_conv_enqueue
+    for L in stack:
+        st = enq(L.conv.h, L.xin.ptr, L.out.ptr, L.ein.ptr if L.ein is not None else None)
+        if st:
+            hip.check(st)
+
+
+class GpuTimer:
+    """HIP events on the engine's own stream (the stream the kernels are launched on)."""
+
+    def __init__(self, eng):
+        self.eng, self.ev = eng, None
+
+    def __enter__(self):
+        self.ev = C.c_void_p()
+        hip.check(hip.lib().cldnn_hip_event_record_begin(self.eng.h, C.byref(self.ev)))
+        return self
+
+    def __exit__(self, *a):
+        hip.check(hip.lib().cldnn_hip_event_record_end(self.ev))
+
+    def seconds(self):
+        ns = C.c_uint64()
+        hip.check(hip.lib().cldnn_hip_event_elapsed_ns(self.ev, C.byref(ns)))
+        hip.check(hip.lib().cldnn_hip_event_release(self.ev))
+        return ns.value * 1e-9
+
+
+def cpu_pass(eng, stack, images, verify):
+    """Run the CPU oracle on the first `images` image(s) of every layer; optionally compare with the
+    GPU results of the same images (a convolution is independent per image)."""
+    from oracle import refconv as rc
+    threads = rc.lib().rc_threads_available()
+    t_total, checked, mism = 0.0, 0, 0
+    for L in stack:
+        l = L.spec
+        kw = dict(stride=(l["stride"],) * 2, pad=(l["pad"],) * 2, groups=l["groups"], out_dt="s8",
+                  act=L.kw.get("act", "none"), act_m=L.kw.get("act_m", 0.0), act_n=L.kw.get("act_n", 0.0))
+        if L.fused:
+            kw.update(eltw=L.eltw[:images], eltw_act="relu", eltw_calib=L.ecal)
+        t0 = time.perf_counter()
+        ref = rc.conv(L.x[:images], L.w, L.bias, wqf=L.wqf, calib=L.calib, nthreads=threads, **kw)
+        t_total += time.perf_counter() - t0
+        if verify:
+            got = hip.download(eng, L.out)[:images]
+            checked += ref.size
+            mism += int(np.count_nonzero(ref != got))
+    return t_total, threads, checked, mism
+
+
+def cpu_baseline_and_check(eng, stack, batch, budget_seconds):
+    """Bounded CPU sample: probe with one image, then as many images as fit the time budget."""
+    t1, threads, checked, mism = cpu_pass(eng, stack, 1, verify=True)
+    n = max(1, min(batch, int(budget_seconds / max(t1, 1e-3))))
+    tn = t1
+    if n > 1:
+        tn, threads, checked, mism = cpu_pass(eng, stack, n, verify=True)
+    return dict(images=n, seconds=tn, threads=threads, checked=checked, mismatches=mism)
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=30)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", default="resnet50_b32_fused",
+                    choices=["resnet50_b32_fused", "resnet50_b32", "resnet50_b1", "vgg16_b16", "mobilenet_v2_b32", "c1"])
+    ap.add_argument("--tile", type=int, default=0, help="force one row (index+1) of the tile table on every layer")
+    ap.add_argument("--per-layer", action="store_true", help="time every layer on its own and print a table to stderr")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline / full-size check")
+    ap.add_argument("--cpu-seconds", type=float, default=15.0)
+    args = ap.parse_args()
+    if args.gpus != 1:
+        log("bench.py: this build runs on one GPU; --gpus %d is not supported (the path shards by batch, no "
+            "figure at several GPUs is produced)" % args.gpus)
+        sys.exit(2)
+
+    wl = args.workload
+    if wl.startswith("resnet50"):
+        layers, batch, fuse = workloads.resnet50(), (1 if wl.endswith("b1") else 32), wl.endswith("fused")
+    elif wl == "vgg16_b16":
+        layers, batch, fuse = workloads.vgg16(), 16, False
+    elif wl == "mobilenet_v2_b32":
+        layers, batch, fuse = workloads.mobilenet_v2(), 32, False
+    else:
+        layers, batch, fuse = [workloads._layer("c1", 64, 64, 3, 1, 1, 56)], 1, False
+
+    eng = hip.Engine(0, profiling=True)
+    info = eng.info()
+    log("device: %s (%s), %d CUs @ %d MHz" % (info.name.decode(), info.arch.decode(), info.cores_count, info.core_frequency))
+    t0 = time.perf_counter()
+    stack = build_stack(eng, layers, batch, fuse, tile=args.tile)
+    eng.finish()
+    log("built %d layers in %.1f s" % (len(stack), time.perf_counter() - t0))
+
+    ops = sum(L.info.ops for L in stack)
+    nbytes = sum(L.info.bytes for L in stack)
+
+    for _ in range(args.warmup):
+        run_step(stack)
+    eng.finish()
+    t_wall0 = time.perf_counter()
+    with GpuTimer(eng) as tm:
+        for _ in range(args.steps):
+            run_step(stack)
+    eng.finish()
+    t_wall = time.perf_counter() - t_wall0
+    t_gpu = tm.seconds()
+    launches = len(stack) * args.steps
+    ms_per_step = t_wall / args.steps * 1e3
+    value = batch * args.steps / t_wall
+
+    per_layer = None
+    if args.per_layer:
+        per_layer = []
+        reps = max(5, args.steps // 2)
+        for L in stack:
+            for _ in range(2):
+                L.conv.enqueue(L.xin, L.out, L.ein)
+            with GpuTimer(eng) as lt:
+                for _ in range(reps):
+                    L.conv.enqueue(L.xin, L.out, L.ein)
+            eng.finish()
+            dt = lt.seconds() / reps
+            per_layer.append((L, dt))
+        log("%-18s %-34s %6s %9s %8s %8s %7s" % ("layer", "kernel", "grid", "us", "TOP/s", "GB/s", "bound"))
+        for L, dt in per_layer:
+            tops, gbs = L.info.ops / dt / 1e12, L.info.bytes / dt / 1e9
+            t_m, t_h = L.info.ops / PEAK_INT8_OPS, L.info.bytes / PEAK_HBM
+            log("%-18s %-34s %6d %9.1f %8.1f %8.0f %7s %5.1f%%" % (
+                L.spec["name"], L.info.kernel_name.decode(), L.info.grid, dt * 1e6, tops, gbs,
+                "mfma" if t_m > t_h else "hbm", 100 * max(t_m, t_h) / dt))
+        log("sum of per-layer times: %.1f us" % (sum(dt for _, dt in per_layer) * 1e6))
+
+    res = {
+        "metric": "ResNet-50 int8 conv stack images/sec @b32; achieved TOPS vs INT8 MFMA peak"
+        if wl.startswith("resnet50_b32") else "int8 conv stack images/sec",
+        "value": value,
+        "unit": "images/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": ms_per_step,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "i8xi8->i32 (f32 requantisation)",
+        "data": "synthetic",
+        "config": {"workload": wl, "batch": batch, "layers": len(stack), "layout": "fs_b_yx_fsv16",
+                   "variant": "stride on the first 1x1 (Caffe form)" if wl.startswith("resnet50") else wl,
+                   "fused_residual_layers": sum(1 for L in stack if L.fused)},
+        "achieved_tops": ops * args.steps / t_gpu / 1e12,
+        "roofline": {
+            "bound": "mfma",
+            "achieved": ops * args.steps / t_gpu / 1e12,
+            "peak": PEAK_INT8_OPS / 1e12,
+            "unit": "TOP/s",
+            "frac": ops * args.steps / t_gpu / PEAK_INT8_OPS,
+            "traffic": None,
+            "kernel": "conv_mfma_kernel (all tile instances)",
+            "launches": launches,
+            "avg_launch_us": t_gpu / launches * 1e6,
+            "ops_per_launch": ops / len(stack),
+        },
+        "roofline_hbm": {
+            "bound": "hbm",
+            "achieved": nbytes * args.steps / t_gpu / 1e9,
+            "peak": PEAK_HBM / 1e9,
+            "unit": "GB/s",
+            "frac": nbytes * args.steps / t_gpu / PEAK_HBM,
+            "bytes_per_launch": nbytes / len(stack),
+        },
+        "gpu_seconds_events": t_gpu,
+        "wall_seconds": t_wall,
+    }
+
+    if not args.no_cpu:
+        cb = cpu_baseline_and_check(eng, stack, batch, args.cpu_seconds)
+        res["cpu_baseline"] = {
+            "value": cb["images"] / cb["seconds"],
+            "unit": "images/s",
+            "cores": cb["threads"],
+            "kind": "port",
+            "sample": "first %d image(s) of every layer of the same stack through oracle/refconv.c "
+                      "(OpenMP over batch x ofm), %.1f s of CPU time" % (cb["images"], cb["seconds"]),
+        }
+        res["verified"] = {"outputs_compared": cb["checked"], "mismatches": cb["mismatches"],
+                           "what": "GPU batch-%d results of the first %d image(s), every layer, vs the CPU oracle "
+                                   "(bit-exact)" % (batch, cb["images"])}
+        if cb["mismatches"]:
+            log("PARITY FAILURE: %d mismatching outputs" % cb["mismatches"])
+    print(json.dumps(res), flush=True)
+    for L in stack:
+        L.conv.close()
+    if not args.no_cpu and res["verified"]["mismatches"]:
+        sys.exit(1)
+
+
+if __name__ == "__main__":
+    main()
