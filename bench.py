@@ -61,7 +61,7 @@ def build_stack(eng, layers, batch, fuse_residual, seed=1337, tile=0, in_dt=np.u
             L.calib = np.full(ofm, 127.0 / 6.0, np.float32)
         else:
             kw.update(act=act)
-        L.xin = hip.upload(eng, L.x, "fs_b_yx_fsv16")
+        L.xin = hip.upload(eng, L.x, "fs_b_yx_fsv16", (l["pad"], l["pad"]))  # zero border as wide as the padding
         L.ein = None
         if L.fused:
             L.eltw = r.integers(-128, 128, (batch, ofm, ohw, ohw), dtype=np.int16).astype(np.int8)
@@ -70,7 +70,13 @@ def build_stack(eng, layers, batch, fuse_residual, seed=1337, tile=0, in_dt=np.u
             kw.update(act="none", eltw_t=L.ein.tensor, eltw_act="relu", has_eltw_calib=True)
         L.kw = kw
         L.desc = hip.conv_desc(L.xin.tensor, L.w.shape, "s8", tile=tile, **kw)
-        L.conv = hip.Conv(eng, L.desc, L.w, L.bias, L.wqf, L.calib, L.ecal)
+        try:
+            L.conv = hip.Conv(eng, L.desc, L.w, L.bias, L.wqf, L.calib, L.ecal)
+        except hip.HipError:
+            if not tile:
+                raise
+            L.desc = hip.conv_desc(L.xin.tensor, L.w.shape, "s8", tile=0, **kw)  # forced row not applicable here
+            L.conv = hip.Conv(eng, L.desc, L.w, L.bias, L.wqf, L.calib, L.ecal)
         L.out = hip.Buffer(eng, L.desc.output)
         L.info = L.conv.info()
         out.append(L)

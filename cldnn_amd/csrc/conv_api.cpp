@@ -15,7 +15,8 @@ struct cldnn_hip_conv_s {
     ConvProblem p{};
     Epilogue epi{};       // device pointers inside
     int impl = CLDNN_HIP_IMPL_REF;
-    int epi_kind = EPI_GENERIC;
+    bool fast = false;
+    FastEpi fe{};
     MfmaPlan mplan{};
     DwPlan dplan{};
     // device allocations
@@ -59,23 +60,6 @@ void* upload(cldnn_hip_conv c, const void* host, size_t bytes, size_t padded_byt
     if (host && bytes) CHIP_CHECK(hipMemcpyAsync(d, host, bytes, hipMemcpyHostToDevice, c->engine->stream));
     CHIP_CHECK(hipStreamSynchronize(c->engine->stream));
     return d;
-}
-
-// gfx950 tile-config table lookup: largest tile that still gives every CU a couple of workgroups.
-int choose_tile(const ConvProblem& p, int cus)
-{
-    static const int by_size[] = {5, 0, 1, 3, 2, 4};  // p256_f128, p128_f128, p256_f64, p128_f64, p64_f128, p64_f64
-    const int64_t m = (int64_t)p.B * p.OH * p.OW;
-    int best = 4;
-    int64_t best_grid = -1;
-    for (int idx : by_size) {
-        const TileConfig& tc = tile_config(idx);
-        if (p.OFM <= 64 && tc.tile_ofm > 64) continue;
-        const int64_t grid = ((m + tc.tile_pixels - 1) / tc.tile_pixels) * ((p.OFM + tc.tile_ofm - 1) / tc.tile_ofm);
-        if (grid >= 2 * (int64_t)cus) return idx;
-        if (grid > best_grid) best_grid = grid, best = idx;
-    }
-    return best;
 }
 
 void build(cldnn_hip_conv c, const void* weights, const void* bias, const float* wqf, const float* calib,
@@ -231,20 +215,20 @@ void build(cldnn_hip_conv c, const void* weights, const void* bias, const float*
     }
 
     if (impl == CLDNN_HIP_IMPL_MFMA) {
-        int tile = d.tile_override > 0 ? d.tile_override - 1 : choose_tile(p, c->engine->props.multiProcessorCount);
+        int tile = d.tile_override > 0 ? d.tile_override - 1 : mfma_choose(p, c->engine->props.multiProcessorCount);
         CHIP_REQUIRE(tile >= 0 && tile < tile_config_count(), CLDNN_HIP_INVALID_ARG, "tile_override out of range");
         c->mplan = mfma_plan(p, tile);
         std::vector<int8_t> packed(c->mplan.packed_bytes);
-        std::vector<int32_t> ktab(c->mplan.ksteps * 4);
+        std::vector<int32_t> ktab(c->mplan.ktab_bytes / sizeof(int32_t));
         mfma_pack_weights(p, c->mplan, w8, packed.data(), ktab.data());
         c->w_packed = upload(c, packed.data(), packed.size());
         c->ktab = upload(c, ktab.data(), ktab.size() * 4);
-        c->epi_kind = mfma_fast_epilogue_ok(p, e, calib_on ? calib : nullptr, eltw_calib, wqf, p.OFM) ? EPI_FAST : EPI_GENERIC;
+        c->fast = mfma_fast_epilogue(p, e, calib_on ? calib : nullptr, eltw_calib, wqf, &c->fe);
         const TileConfig& tc = tile_config(tile);
         inf.tile_index = tile, inf.tile_pixels = tc.tile_pixels, inf.tile_ofm = tc.tile_ofm;
         inf.grid = c->mplan.grid, inf.block = 256, inf.lds_bytes = c->mplan.lds_bytes;
-        std::snprintf(inf.kernel_name, sizeof(inf.kernel_name), "conv_mfma_kernel<%d,%d,%d,%s>", tc.tile_pixels,
-                      tc.tile_ofm, tc.wave_pixels, c->epi_kind == EPI_FAST ? "fast" : "generic");
+        std::snprintf(inf.kernel_name, sizeof(inf.kernel_name), "conv_%s<%s,%s,%s>", c->mplan.stream ? "stream" : "mfma",
+                      tc.name, c->mplan.checked ? "checked" : "border", c->fast ? "fast" : "generic");
     } else {
         c->dplan = dw_plan(p);
         std::vector<int8_t> packed(c->dplan.packed_bytes);
@@ -321,9 +305,10 @@ static void run(cldnn_hip_conv c, const void* in, void* out, const void* eltw, i
     case CLDNN_HIP_IMPL_MFMA: {
         MfmaBuffers wb{(const int8_t*)c->w_packed, (const int32_t*)c->ktab};
         if (raw)
-            launch_conv_mfma(s, p, c->mplan, wb, (const int32_t*)c->acc_init_raw, c->epi, EPI_RAW, in, nullptr, nullptr, raw);
+            launch_conv_mfma(s, p, c->mplan, wb, (const int32_t*)c->acc_init_raw, c->epi, nullptr, in, nullptr, nullptr, raw);
         else
-            launch_conv_mfma(s, p, c->mplan, wb, (const int32_t*)c->acc_init, c->epi, c->epi_kind, in, eltw, out, nullptr);
+            launch_conv_mfma(s, p, c->mplan, wb, (const int32_t*)c->acc_init, c->epi, c->fast ? &c->fe : nullptr, in, eltw,
+                             out, nullptr);
         break;
     }
     case CLDNN_HIP_IMPL_DEPTHWISE:

@@ -1,294 +1,123 @@
-// Dense quantized convolution as an implicit GEMM on the gfx950 int8 matrix cores.
-//
-//   D[ofm][pixel] = sum_k W[ofm][k] * X[pixel][k],   k = (tap, input feature)
-//
-// computed with v_mfma_i32_16x16x64_i8: the A operand is a 16(ofm) x 64(k) weight tile, the
-// B operand a 64(k) x 16(pixel) activation tile; every lane feeds 16 consecutive k bytes of one
-// row / column, and that is exactly one 16-feature slice of one pixel in fs_b_yx_fsv16 memory
-// (one 128-bit load, one 128-bit LDS read, no byte shuffling anywhere).
-//
-// Workgroup = 256 threads = 4 waves, output tile BM pixels x BN features; each wave owns
-// 64 features x WP pixels.  Per K-step (4 k-chunks = 64 k values) the workgroup stages
-// BN x 64 weight bytes and BM x 64 activation bytes in LDS (double buffered, one barrier
-// per step).  Pixels are the linear index over (batch, oy, ox), so a tile may span rows and
-// images; taps outside the image read as zero.
-//
-// u8 activations: the MFMA multiplies signed bytes, so activations are fed as (a ^ 0x80) = a - 128
-// and the accumulators start from 128 * sum(w[f]) (+ the int32 bias), which is exact in int32.
-//
-// Weight rows are stored permuted inside each 64-feature span so that a lane's 16 accumulators
-// of one pixel are 16 CONSECUTIVE features: the int8 result is written with one 128-bit store.
-#include "epilogue.h"
-#include "kernels.h"
-
+// Host side of the int8 MFMA convolution: the gfx950 tile-config table, plans, weight
+// pre-packing, eligibility of the short epilogue and the launch.
+#include <cmath>
 #include <cstring>
-#include <vector>
+
+#include "conv_mfma_kernel.h"
 
 namespace chip {
 
-typedef int v4i __attribute__((ext_vector_type(4)));
+#define DECL_TILE(i) void launch_mfma_tile_##i(hipStream_t, const MfmaArgs&, int, int, bool, int);
+DECL_TILE(0) DECL_TILE(1) DECL_TILE(2) DECL_TILE(3) DECL_TILE(4) DECL_TILE(5)
+#undef DECL_TILE
+void launch_stream(hipStream_t s, const MfmaArgs& a, int nt, int grid, int epi);
 
-struct MfmaArgs {
-    const int8_t* in;
-    const int8_t* wpk;
-    const int32_t* ktab;
-    const int32_t* acc_init;  // [ofm_tiles * BN], natural feature order, zero padded
-    void* out;
-    const void* eltw;
-    int32_t* raw;
-    Pitch in_p, out_p, eltw_p;
-    int B, IH, IW, OH, OW, OFM, OHW;
-    int64_t M;
-    int sy, sx, py, px, esy, esx;
-    int ksteps;
-    uint32_t xor_mask;  // 0x80808080 for u8 activations, 0 for s8
-    Epilogue epi;
-    // EPI_FAST parameters
-    float fast_lo, fast_hi;
-};
+typedef void (*tile_launcher)(hipStream_t, const MfmaArgs&, int, int, bool, int);
 
 static const TileConfig g_tiles[] = {
-    {"mfma_i8_p128_f128", 128, 128, 64},
-    {"mfma_i8_p256_f64", 256, 64, 64},
-    {"mfma_i8_p64_f128", 64, 128, 32},
-    {"mfma_i8_p128_f64", 128, 64, 32},
-    {"mfma_i8_p64_f64", 64, 64, 16},
-    {"mfma_i8_p256_f128", 256, 128, 128},
+    {"p128_f128", 128, 128, 64},
+    {"p256_f64", 256, 64, 64},
+    {"p64_f128", 64, 128, 32},
+    {"p128_f64", 128, 64, 32},
+    {"p64_f64", 64, 64, 16},
+    {"p256_f128", 256, 128, 128},
+    // rows of the streaming kernel: a wave owns one span of 64 features of one tile of wave_pixels pixels
+    {"stream_p16", 16, 64, 16},
+    {"stream_p32", 32, 64, 32},
 };
+enum { FIRST_STREAM_ROW = 6 };
+enum { MFMA_SLACK_STEPS = 10 };  // >= largest prefetch distance + 1
+static const tile_launcher g_launch[] = {launch_mfma_tile_0, launch_mfma_tile_1, launch_mfma_tile_2, launch_mfma_tile_3,
+                                         launch_mfma_tile_4, launch_mfma_tile_5};
+
 int tile_config_count() { return (int)(sizeof(g_tiles) / sizeof(g_tiles[0])); }
 const TileConfig& tile_config(int i) { return g_tiles[i]; }
 
-// ktab entry: bits 0..9 = fy*dilation_y, 10..19 = fx*dilation_x, 20..30 = feature slice, bit 31 = padding chunk
-__host__ __device__ inline int32_t ktab_pack(int fyd, int fxd, int cb) { return fyd | (fxd << 10) | (cb << 20); }
-
-template <int BM, int BN, int WP, int EPI>
-__global__ void __launch_bounds__(256) conv_mfma_kernel(MfmaArgs a)
+static FastDiv make_div(uint32_t d)
 {
-    constexpr int NT = WP / 16;        // pixel tiles per wave
-    constexpr int WAVES_F = BN / 64;   // waves along features
-    constexpr int A_LOADS = BN / 64;   // 16-byte weight chunks per thread per K-step
-    constexpr int B_LOADS = BM / 64;   // 16-byte activation chunks per thread per K-step
-    constexpr int KC_STRIDE = 256 / BM;  // k-chunk distance between a thread's activation loads
-    static_assert((BM / WP) * WAVES_F == 4, "tile must map onto 4 waves");
-
-    extern __shared__ __align__(16) unsigned char smem[];
-    v4i* ldsA = reinterpret_cast<v4i*>(smem);                 // [2][4 * BN]
-    v4i* ldsB = reinterpret_cast<v4i*>(smem) + 2 * 4 * BN;    // [2][4 * BM]
-
-    const int t = threadIdx.x;
-    const int lane = t & 63;
-    const int wave = t >> 6;
-    const int wave_f = wave % WAVES_F;
-    const int wave_p = wave / WAVES_F;
-
-    // feature tiles vary fastest so that workgroups sharing activation pixels run together
-    const int ofm_tiles = (a.OFM + BN - 1) / BN;
-    const int ntile = blockIdx.x % ofm_tiles;
-    const int64_t m0 = (int64_t)(blockIdx.x / ofm_tiles) * BM;
-
-    // ---- this thread's activation pixel
-    const int lp = t % BM;
-    const int kc0 = t / BM;
-    const int64_t m_ld = m0 + lp;
-    const bool ld_valid = m_ld < a.M;
-    int iy0, ix0;
-    int64_t in_base;
-    {
-        const int64_t mm = ld_valid ? m_ld : 0;
-        const int b = (int)(mm / a.OHW);
-        const int r = (int)(mm % a.OHW);
-        const int oy = r / a.OW, ox = r % a.OW;
-        iy0 = oy * a.sy - a.py;
-        ix0 = ox * a.sx - a.px;
-        in_base = a.in_p.off + (int64_t)b * a.in_p.pb;
+    FastDiv f{};
+    if (d <= 1) {
+        f.one = 1;
+        return f;
     }
-    const v4i* wsrc = reinterpret_cast<const v4i*>(a.wpk) + (int64_t)ntile * a.ksteps * (4 * BN) + t;
-
-    v4i ra[A_LOADS], rb[B_LOADS];
-
-    auto load_global = [&](int ks) {
-#pragma unroll
-        for (int j = 0; j < A_LOADS; ++j) ra[j] = wsrc[(int64_t)ks * (4 * BN) + j * 256];
-#pragma unroll
-        for (int j = 0; j < B_LOADS; ++j) {
-            const int kc = ks * 4 + kc0 + j * KC_STRIDE;
-            const int e = a.ktab[kc];
-            const int iy = iy0 + (e & 1023), ix = ix0 + ((e >> 10) & 1023);
-            const int cb = (e >> 20) & 2047;
-            const bool ok = ld_valid && e >= 0 && iy >= 0 && iy < a.IH && ix >= 0 && ix < a.IW;
-            v4i v = {0, 0, 0, 0};
-            if (ok) {
-                const int64_t off = in_base + (int64_t)cb * a.in_p.pf + (int64_t)iy * a.in_p.py + (int64_t)ix * 16;
-                v = *reinterpret_cast<const v4i*>(a.in + off);
-            }
-            rb[j] = v;
-        }
-    };
-    auto store_lds = [&](int buf) {
-#pragma unroll
-        for (int j = 0; j < A_LOADS; ++j) ldsA[buf * 4 * BN + t + j * 256] = ra[j];
-#pragma unroll
-        for (int j = 0; j < B_LOADS; ++j) ldsB[buf * 4 * BM + (kc0 + j * KC_STRIDE) * BM + lp] = rb[j];
-    };
-
-    // ---- accumulators start from the per-feature constant (u8 offset correction + int32 bias)
-    v4i acc[4][NT];
-    {
-        const int g = lane >> 4;
-        const int fbase = ntile * BN + wave_f * 64 + g * 16;
-#pragma unroll
-        for (int mt = 0; mt < 4; ++mt) {
-            const v4i init = *reinterpret_cast<const v4i*>(a.acc_init + fbase + mt * 4);
-#pragma unroll
-            for (int nt = 0; nt < NT; ++nt) acc[mt][nt] = init;
-        }
-    }
-
-    load_global(0);
-    store_lds(0);
-    __syncthreads();
-
-    const int arow = wave_f * 64 + (lane & 15);
-    const int bcol = wave_p * WP + (lane & 15);
-    const int kq = lane >> 4;
-    const v4i xm = {(int)a.xor_mask, (int)a.xor_mask, (int)a.xor_mask, (int)a.xor_mask};
-
-    for (int ks = 0; ks < a.ksteps; ++ks) {
-        const int buf = ks & 1;
-        if (ks + 1 < a.ksteps) load_global(ks + 1);
-
-        v4i fa[4], fb[NT];
-#pragma unroll
-        for (int mt = 0; mt < 4; ++mt) fa[mt] = ldsA[buf * 4 * BN + kq * BN + arow + mt * 16];
-#pragma unroll
-        for (int nt = 0; nt < NT; ++nt) fb[nt] = ldsB[buf * 4 * BM + kq * BM + bcol + nt * 16] ^ xm;
-#pragma unroll
-        for (int mt = 0; mt < 4; ++mt)
-#pragma unroll
-            for (int nt = 0; nt < NT; ++nt)
-                acc[mt][nt] = __builtin_amdgcn_mfma_i32_16x16x64_i8(fa[mt], fb[nt], acc[mt][nt], 0, 0, 0);
-
-        if (ks + 1 < a.ksteps) store_lds(buf ^ 1);
-        __syncthreads();
-    }
-
-    // ---- epilogue: lane (g, col) holds, for each pixel tile, features fs*16 .. fs*16+15 of one pixel
-    const int g = lane >> 4;
-    const int f0 = ntile * BN + wave_f * 64 + g * 16;
-    if (f0 >= a.OFM) return;
-    const int fs = f0 >> 4;
-    const Epilogue& e = a.epi;
-
-#pragma unroll
-    for (int nt = 0; nt < NT; ++nt) {
-        const int64_t m = m0 + wave_p * WP + nt * 16 + (lane & 15);
-        if (m >= a.M) continue;
-        const int b = (int)(m / a.OHW);
-        const int r = (int)(m % a.OHW);
-        const int oy = r / a.OW, ox = r % a.OW;
-
-        if (EPI == EPI_RAW) {
-#pragma unroll
-            for (int mt = 0; mt < 4; ++mt)
-#pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    const int f = f0 + mt * 4 + i;
-                    if (f < a.OFM) a.raw[(((int64_t)b * a.OFM + f) * a.OH + oy) * a.OW + ox] = acc[mt][nt][i];
-                }
-            continue;
-        }
-
-        const int64_t obase = a.out_p.off + (int64_t)b * a.out_p.pb + (int64_t)fs * a.out_p.pf
-                              + (int64_t)oy * a.out_p.py + (int64_t)ox * a.out_p.px;
-        int64_t ebase = 0;
-        if (e.fused)
-            ebase = a.eltw_p.off + (int64_t)b * a.eltw_p.pb + (int64_t)fs * a.eltw_p.pf
-                    + (int64_t)(oy * a.esy) * a.eltw_p.py + (int64_t)(ox * a.esx) * a.eltw_p.px;
-
-        if (EPI == EPI_FAST) {
-            // relu, non-negative per-feature scale, unit wqf/iqf, int8 output, optional int8 residual with
-            // unit scale + relu: cvt, mul, clamp, +0.49999997 and truncate.
-            // trunc(y + pred(0.5)) == round-half-away(y) for 0 <= y < 2^22.
-            v4i ev4 = {0, 0, 0, 0};
-            if (e.fused) ev4 = *reinterpret_cast<const v4i*>((const int8_t*)a.eltw + ebase);
-            v4i packed;
-#pragma unroll
-            for (int mt = 0; mt < 4; ++mt) {
-                const float4 cal = *reinterpret_cast<const float4*>(e.calib + f0 + mt * 4);
-                const float cs[4] = {cal.x, cal.y, cal.z, cal.w};
-                float4 ecal = {1.f, 1.f, 1.f, 1.f};
-                if (e.fused && e.eltw_calib) ecal = *reinterpret_cast<const float4*>(e.eltw_calib + f0 + mt * 4);
-                const float ecs[4] = {ecal.x, ecal.y, ecal.z, ecal.w};
-                unsigned word = 0;
-#pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    float v = (float)acc[mt][nt][i] * cs[i];
-                    int q;
-                    if (!e.fused) {
-                        v = fminf(fmaxf(v, 0.0f), a.fast_hi);
-                        q = (int)(v + 0.49999997f);
-                    } else {
-                        // conv part: relu is absent in the fused form handled here (act == none):
-                        // round half away on a signed value, then add the residual
-                        float rr = truncf(v + copysignf(0.49999997f, v));
-                        int ebyte = (int)(int8_t)((unsigned)ev4[mt] >> (8 * i));
-                        if (e.eltw_dt == CLDNN_HIP_U8) ebyte &= 255;
-                        float s = rr + (float)ebyte;
-                        s = fmaxf(s, 0.0f) * ecs[i];
-                        s = fminf(fmaxf(s, a.fast_lo), a.fast_hi);
-                        q = (int)(s + copysignf(0.49999997f, s));
-                    }
-                    word |= ((unsigned)q & 255u) << (8 * i);
-                }
-                packed[mt] = (int)word;
-            }
-            *reinterpret_cast<v4i*>((int8_t*)a.out + obase) = packed;
-            continue;
-        }
-
-        // generic epilogue
-        const bool out8 = e.out_dt == CLDNN_HIP_S8 || e.out_dt == CLDNN_HIP_U8;
-        v4i packed = {0, 0, 0, 0};
-#pragma unroll
-        for (int mt = 0; mt < 4; ++mt)
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                const int ci = mt * 4 + i;
-                const int f = f0 + ci;
-                EpiOut o;
-                o.f = 0.f, o.i = 0;
-                if (f < a.OFM) {
-                    float ev = 0.f;
-                    if (e.fused) ev = load_as_float(a.eltw, e.eltw_dt, ebase + ci);
-                    o = epilogue_generic(e, acc[mt][nt][i], f, ev);
-                }
-                if (out8) packed[mt] |= (int)(((unsigned)o.i & 255u) << (8 * i));
-                else store_out(a.out, e.out_dt, obase + ci, o);
-            }
-        if (out8) *reinterpret_cast<v4i*>((int8_t*)a.out + obase) = packed;
-    }
+    uint32_t s = 0;
+    while ((1ull << s) < d) ++s;              // s = ceil(log2 d) >= 1
+    const unsigned p = 31 + s;
+    f.mul = (uint32_t)(((1ull << p) + d - 1) / d);  // ceil(2^p / d) < 2^32
+    f.shift = p - 32;
+    return f;
 }
 
-// ------------------------------------------------------------------------------------------ host side
+// does the input buffer carry a zero border that covers every tap of every output pixel?
+static bool border_covers(const ConvProblem& p)
+{
+    const cldnn_hip_tensor& t = p.in_t;
+    const int hi_y = (p.OH - 1) * p.sy - p.py + (p.FY - 1) * p.dy - (p.IH - 1);
+    const int hi_x = (p.OW - 1) * p.sx - p.px + (p.FX - 1) * p.dx - (p.IW - 1);
+    return t.pad_lo_y >= p.py && t.pad_lo_x >= p.px && t.pad_hi_y >= hi_y && t.pad_hi_x >= hi_x;
+}
+
+// ---- the gfx950 tile-config table lookup.  Key: (pixels M, OFM, K-steps, border available); value: table row.
+int mfma_choose(const ConvProblem& p, int cus)
+{
+    const int64_t m = (int64_t)p.B * p.OH * p.OW;
+    const int ksteps = (p.FY * p.FX * ((p.IFM + 15) / 16) + 3) / 4;
+    if (ksteps <= 8 && border_covers(p)) {
+        // short K: bound by HBM bandwidth.  Stream unless there are too few pixels to occupy the chip
+        const int64_t waves = ((m + 31) / 32) * ((p.OFM + 63) / 64);
+        if (waves >= 4ll * cus) return FIRST_STREAM_ROW + 1;
+        if (waves * 2 >= 4ll * cus) return FIRST_STREAM_ROW;
+    }
+    static const int order_f128[] = {5, 0, 2, 1, 3, 4};
+    static const int order_f64[] = {1, 3, 4};
+    const int* order = p.OFM > 64 ? order_f128 : order_f64;
+    const int n = p.OFM > 64 ? 6 : 3;
+    int best = order[n - 1];
+    int64_t best_grid = -1;
+    for (int i = 0; i < n; ++i) {
+        const TileConfig& tc = g_tiles[order[i]];
+        const int64_t grid = ((m + tc.tile_pixels - 1) / tc.tile_pixels) * ((p.OFM + tc.tile_ofm - 1) / tc.tile_ofm);
+        if (grid >= 2 * (int64_t)cus) return order[i];
+        if (grid > best_grid) best_grid = grid, best = order[i];
+    }
+    return best;
+}
+
 MfmaPlan mfma_plan(const ConvProblem& p, int tile)
 {
     const TileConfig& tc = g_tiles[tile];
     MfmaPlan pl{};
     pl.tile = tile;
+    pl.checked = border_covers(p) ? 0 : 1;
+    pl.stream = tile >= FIRST_STREAM_ROW ? 1 : 0;
+    CHIP_REQUIRE(!(pl.stream && pl.checked), CLDNN_HIP_INVALID_ARG,
+                 "the streaming kernel needs an input whose physical zero border covers the convolution's padding");
     pl.cb = (p.IFM + 15) / 16;
     pl.kchunks = p.FY * p.FX * pl.cb;
     pl.ksteps = (pl.kchunks + 3) / 4;
+    if (pl.stream) {
+        CHIP_REQUIRE(pl.ksteps <= 8, CLDNN_HIP_INVALID_ARG, "the streaming kernel handles at most 8 K-steps (K <= 512)");
+        int ks = 1;
+        while (ks < pl.ksteps) ks *= 2;  // compile-time K-step counts: 1, 2, 4, 8 (zero-weight padding chunks)
+        pl.ksteps = ks;
+    }
     pl.ofm_tiles = (p.OFM + tc.tile_ofm - 1) / tc.tile_ofm;
     pl.m_total = (int64_t)p.B * p.OH * p.OW;
-    const int64_t mtiles = (pl.m_total + tc.tile_pixels - 1) / tc.tile_pixels;
-    const int64_t grid = mtiles * pl.ofm_tiles;
+    CHIP_REQUIRE(pl.m_total < (1ll << 31), CLDNN_HIP_UNSUPPORTED_SIZE, "more than 2^31 output pixels");
+    pl.mtiles = (int)((pl.m_total + tc.tile_pixels - 1) / tc.tile_pixels);
+    int64_t grid = (int64_t)((pl.mtiles + 7) / 8) * 8 * pl.ofm_tiles;
+    if (pl.stream) grid = ((int64_t)pl.mtiles * pl.ofm_tiles + 3) / 4;  // one wave per (pixel tile, span)
     CHIP_REQUIRE(grid < (1ll << 31), CLDNN_HIP_UNSUPPORTED_SIZE, "convolution too large for one launch");
     pl.grid = (int)grid;
-    pl.lds_bytes = 2 * 4 * (tc.tile_ofm + tc.tile_pixels) * 16;
-    pl.packed_bytes = (size_t)pl.ofm_tiles * pl.ksteps * 4 * tc.tile_ofm * 16;
-    pl.ktab_bytes = (size_t)pl.ksteps * 4 * sizeof(int32_t);
+    pl.lds_bytes = pl.stream ? 0 : 2 * 4 * (tc.tile_ofm + tc.tile_pixels) * 16;
+    // the tile kernel requests operands up to MFMA_SLACK_STEPS K-steps past the end (zero weights there)
+    pl.packed_bytes = ((size_t)pl.ofm_tiles * pl.ksteps + MFMA_SLACK_STEPS) * 4 * tc.tile_ofm * 16;
+    pl.ktab_bytes = (size_t)(pl.ksteps + MFMA_SLACK_STEPS) * 4 * sizeof(int32_t);
     CHIP_REQUIRE((p.FY - 1) * p.dy < 1024 && (p.FX - 1) * p.dx < 1024 && pl.cb < 2048, CLDNN_HIP_UNSUPPORTED_SIZE,
                  "filter extent or feature count beyond the tap table encoding");
+    // 32-bit offsets inside the kernel
+    CHIP_REQUIRE(tensor_elems(p.in_t) < (1ull << 31) && tensor_elems(p.out_t) * dtype_size(p.out_dt) < (1ull << 31),
+                 CLDNN_HIP_UNSUPPORTED_SIZE, "tensor of 2 GiB or more");
     return pl;
 }
 
@@ -298,13 +127,15 @@ void mfma_pack_weights(const ConvProblem& p, const MfmaPlan& pl, const int8_t* w
     const int BN = tc.tile_ofm;
     std::memset(packed, 0, pl.packed_bytes);
     // k-chunk order: tap-major, feature slice minor
-    for (int kc = 0; kc < pl.ksteps * 4; ++kc) {
+    for (int kc = 0; kc < (pl.ksteps + MFMA_SLACK_STEPS) * 4; ++kc) {
         if (kc >= pl.kchunks) {
-            ktab[kc] = (int32_t)0x80000000;
+            ktab[kc] = pl.checked ? (int32_t)0x80000000 : 0;  // padding chunk: zero weights
             continue;
         }
         const int tap = kc / pl.cb, cb = kc % pl.cb;
-        ktab[kc] = ktab_pack((tap / p.FX) * p.dy, (tap % p.FX) * p.dx, cb);
+        const int fyd = (tap / p.FX) * p.dy, fxd = (tap % p.FX) * p.dx;
+        if (pl.checked) ktab[kc] = fyd | (fxd << 10) | (cb << 20);
+        else ktab[kc] = (int32_t)(cb * p.in_p.pf + fyd * p.in_p.py + fxd * 16);
     }
     for (int f = 0; f < p.OFM; ++f) {
         const int nt = f / BN, fl = f % BN;
@@ -322,77 +153,116 @@ void mfma_pack_weights(const ConvProblem& p, const MfmaPlan& pl, const int8_t* w
     }
 }
 
-template <int BM, int BN, int WP>
-static void launch_tile(hipStream_t s, const MfmaArgs& a, int grid, int lds, int epi)
+static bool tame(const float* v, int n)
 {
-    switch (epi) {
-    case EPI_RAW:
-        hipLaunchKernelGGL((conv_mfma_kernel<BM, BN, WP, EPI_RAW>), dim3(grid), dim3(256), lds, s, a);
-        break;
-    case EPI_FAST:
-        hipLaunchKernelGGL((conv_mfma_kernel<BM, BN, WP, EPI_FAST>), dim3(grid), dim3(256), lds, s, a);
-        break;
-    default:
-        hipLaunchKernelGGL((conv_mfma_kernel<BM, BN, WP, EPI_GENERIC>), dim3(grid), dim3(256), lds, s, a);
-        break;
-    }
+    for (int i = 0; i < n; ++i)
+        if (!(std::fabs(v[i]) < 1.0e9f)) return false;  // also rejects NaN
+    return true;
 }
 
-// Can the short epilogue reproduce the generic one bit for bit?  (decided per convolution at creation)
-bool mfma_fast_epilogue_ok(const ConvProblem& p, const Epilogue& e, const float* calib_host, const float* ecal_host,
-                           const float* wqf_host, int ofm)
+// Can the short epilogue reproduce the long one bit for bit?  Decided once per convolution.
+bool mfma_fast_epilogue(const ConvProblem& p, const Epilogue& e, const float* calib, const float* ecal, const float* wqf,
+                        FastEpi* out)
 {
+    FastEpi F{};
     if (e.mode != MODE_Q || e.round_even) return false;
-    if (e.bias) return false;  // int32 bias is folded into the accumulator start; a float bias needs the long path
+    if (e.bias) return false;  // an int32 bias is folded into the accumulator start; a float bias takes the long path
     if (!(e.out_dt == CLDNN_HIP_S8 || e.out_dt == CLDNN_HIP_U8)) return false;
-    if (!calib_host) return false;
-    if (e.iqf != 1.0f) return false;
-    if (wqf_host)
-        for (int f = 0; f < ofm; ++f)
-            if (wqf_host[f] != 1.0f) return false;
-    for (int f = 0; f < ofm; ++f)
-        if (!(calib_host[f] >= 0.0f) || !(calib_host[f] < 3.0e38f)) return false;
-    if (!e.fused) return e.act == CLDNN_HIP_ACT_RELU;
-    // fused: conv result without activation, int8 residual with unit scale, relu, optional non-negative scale
-    if (e.act != CLDNN_HIP_ACT_NONE || e.eltw_act != CLDNN_HIP_ACT_RELU || e.ncs_on) return false;
-    if (!(e.eltw_dt == CLDNN_HIP_S8 || e.eltw_dt == CLDNN_HIP_U8)) return false;
-    if (p.eltw_p.fsv != 16 || p.esy != 1 || p.esx != 1) return false;
-    if (ecal_host)
-        for (int f = 0; f < ofm; ++f)
-            if (!(ecal_host[f] >= 0.0f) || !(ecal_host[f] < 3.0e38f)) return false;
+    if (!(e.act == CLDNN_HIP_ACT_NONE || e.act == CLDNN_HIP_ACT_RELU || e.act == CLDNN_HIP_ACT_CLAMP)) return false;
+    if (e.act == CLDNN_HIP_ACT_CLAMP && !(e.act_m <= e.act_n)) return false;  // the median form needs ordered bounds
+    // factors small enough that no product can overflow into inf * 0
+    if (calib && !tame(calib, p.OFM)) return false;
+    if (ecal && !tame(ecal, p.OFM)) return false;
+    if (wqf && !tame(wqf, p.OFM)) return false;
+    if (!tame(&e.iqf, 1) || !tame(&e.oqf, 1) || !tame(&e.act_m, 1) || !tame(&e.act_n, 1)) return false;
+    F.lo = e.out_dt == CLDNN_HIP_S8 ? -128.0f : 0.0f;
+    F.hi = e.out_dt == CLDNN_HIP_S8 ? 127.0f : 255.0f;
+    F.iqf = e.iqf;
+    F.act = e.act, F.act_m = e.act_m, F.act_n = e.act_n;
+    F.has_wqf = 0;
+    if (wqf) {
+        bool unit = e.iqf == 1.0f;
+        for (int f = 0; f < p.OFM && unit; ++f) unit = wqf[f] == 1.0f;
+        F.has_wqf = unit ? 0 : 1;  // x * 1.0f * 1.0f == x
+    }
+    F.fused = e.fused;
+    if (e.fused) {
+        if (e.ncs_on) return false;
+        if (!(e.eltw_dt == CLDNN_HIP_S8 || e.eltw_dt == CLDNN_HIP_U8) || p.eltw_p.fsv != 16) return false;
+        if (!(e.eltw_act == CLDNN_HIP_ACT_NONE || e.eltw_act == CLDNN_HIP_ACT_RELU || e.eltw_act == CLDNN_HIP_ACT_CLAMP))
+            return false;
+        if (!tame(&e.eltw_m, 1) || !tame(&e.eltw_n, 1)) return false;
+        F.eltw_act = e.eltw_act, F.eltw_m = e.eltw_m, F.eltw_n = e.eltw_n;
+        F.has_ecal = ecal ? 1 : 0;
+        F.eltw_u8 = e.eltw_dt == CLDNN_HIP_U8;
+        if (e.eltw_act == CLDNN_HIP_ACT_CLAMP && !(e.eltw_m <= e.eltw_n)) return false;
+        if (e.eltw_act == CLDNN_HIP_ACT_RELU) {
+            bool nonneg = true;
+            if (ecal)
+                for (int f = 0; f < p.OFM && nonneg; ++f) nonneg = ecal[f] >= 0.0f;
+            F.eltw_relu_folded = nonneg ? 1 : 0;
+        }
+    } else if (e.act == CLDNN_HIP_ACT_RELU) {
+        bool nonneg = true;
+        if (calib)
+            for (int f = 0; f < p.OFM && nonneg; ++f) nonneg = calib[f] >= 0.0f;
+        else if (e.oqf_on) nonneg = e.oqf >= 0.0f;
+        F.relu_folded = nonneg ? 1 : 0;
+    }
+    *out = F;
     return true;
 }
 
 void launch_conv_mfma(hipStream_t s, const ConvProblem& p, const MfmaPlan& pl, const MfmaBuffers& wb,
-                         const int32_t* acc_init, const Epilogue& epi, int epi_kind, const void* in, const void* eltw,
-                         void* out, int32_t* raw)
+                      const int32_t* acc_init, const Epilogue& epi, const FastEpi* fast, const void* in, const void* eltw,
+                      void* out, int32_t* raw)
 {
     const TileConfig& tc = g_tiles[pl.tile];
     MfmaArgs a{};
     a.in = (const int8_t*)in;
-    a.wpk = wb.packed;
+    a.wpk = (const v4i*)wb.packed;
     a.ktab = wb.ktab;
     a.acc_init = acc_init;
     a.out = out;
     a.eltw = eltw;
     a.raw = raw;
-    a.in_p = p.in_p, a.out_p = p.out_p, a.eltw_p = p.eltw_p;
-    a.B = p.B, a.IH = p.IH, a.IW = p.IW, a.OH = p.OH, a.OW = p.OW, a.OFM = p.OFM, a.OHW = p.OH * p.OW;
-    a.M = pl.m_total;
+    a.M = (uint32_t)pl.m_total;
+    a.OFM = p.OFM, a.ofm_tiles = pl.ofm_tiles, a.mtiles = pl.mtiles;
+    a.OHW = p.OH * p.OW, a.OW = p.OW, a.OH = p.OH, a.IH = p.IH, a.IW = p.IW;
+    a.div_ohw = make_div((uint32_t)a.OHW), a.div_ow = make_div((uint32_t)a.OW);
     a.sy = p.sy, a.sx = p.sx, a.py = p.py, a.px = p.px, a.esy = p.esy, a.esx = p.esx;
+    a.in_off = (int32_t)p.in_p.off, a.in_pb = (int32_t)p.in_p.pb, a.in_pf = (int32_t)p.in_p.pf, a.in_py = (int32_t)p.in_p.py;
+    a.out_off = (int32_t)p.out_p.off, a.out_pb = (int32_t)p.out_p.pb, a.out_pf = (int32_t)p.out_p.pf;
+    a.out_py = (int32_t)p.out_p.py;
+    a.el_off = (int32_t)p.eltw_p.off, a.el_pb = (int32_t)p.eltw_p.pb, a.el_pf = (int32_t)p.eltw_p.pf;
+    a.el_py = (int32_t)p.eltw_p.py;
     a.ksteps = pl.ksteps;
+    a.CB = pl.cb, a.FX = p.FX, a.kchunks = pl.kchunks;
+    a.tap_dy = p.dy * (int32_t)p.in_p.py, a.tap_dx = p.dx * 16;
+    a.div_cb = make_div((uint32_t)pl.cb), a.div_fx = make_div((uint32_t)p.FX);
+    {
+        // dense tensors and a 1x1 / stride-1 convolution: pixel m sits at byte m * 16 of every feature slice
+        auto dense = [](const cldnn_hip_tensor& t) {
+            return t.pad_lo_y == 0 && t.pad_lo_x == 0 && t.pad_hi_y == 0 && t.pad_hi_x == 0;
+        };
+        a.linear = p.FY == 1 && p.FX == 1 && p.sy == 1 && p.sx == 1 && p.py == 0 && p.px == 0 && dense(p.in_t)
+                   && dense(p.out_t) && p.out_dt != CLDNN_HIP_F32
+                   && (!epi.fused || (dense(p.eltw_t) && p.esy == 1 && p.esx == 1 && p.eltw_t.y == p.OH && p.eltw_t.x == p.OW));
+    }
     a.xor_mask = p.in_dt == CLDNN_HIP_U8 ? 0x80808080u : 0u;
     a.epi = epi;
-    a.fast_lo = epi.out_dt == CLDNN_HIP_S8 ? -128.0f : 0.0f;
-    a.fast_hi = epi.out_dt == CLDNN_HIP_S8 ? 127.0f : 255.0f;
-    const int g = pl.grid, l = pl.lds_bytes;
-    if (tc.tile_pixels == 128 && tc.tile_ofm == 128) launch_tile<128, 128, 64>(s, a, g, l, epi_kind);
-    else if (tc.tile_pixels == 256 && tc.tile_ofm == 64) launch_tile<256, 64, 64>(s, a, g, l, epi_kind);
-    else if (tc.tile_pixels == 64 && tc.tile_ofm == 128) launch_tile<64, 128, 32>(s, a, g, l, epi_kind);
-    else if (tc.tile_pixels == 128 && tc.tile_ofm == 64) launch_tile<128, 64, 32>(s, a, g, l, epi_kind);
-    else if (tc.tile_pixels == 64 && tc.tile_ofm == 64) launch_tile<64, 64, 16>(s, a, g, l, epi_kind);
-    else if (tc.tile_pixels == 256 && tc.tile_ofm == 128) launch_tile<256, 128, 128>(s, a, g, l, epi_kind);
-    else throw error(CLDNN_HIP_ERROR, "tile configuration without a kernel instance");
+    int kind = EPI_KIND_GENERIC;
+    if (fast && !raw) {
+        a.fe = *fast;
+        kind = EPI_KIND_FAST;
+        // the two branch-free forms (the host keeps vectors of ones where the primitive has no factors)
+        if (!fast->has_wqf && epi.calib) {
+            if (!fast->fused && fast->relu_folded) kind = EPI_KIND_RELU;
+            if (fast->fused && fast->act == CLDNN_HIP_ACT_NONE && fast->eltw_relu_folded && epi.eltw_calib) kind = EPI_KIND_FUSED;
+        }
+    }
+    if (pl.stream) launch_stream(s, a, tc.wave_pixels / 16, pl.grid, kind);
+    else g_launch[pl.tile](s, a, pl.grid, pl.lds_bytes, pl.checked != 0, kind);
     CHIP_CHECK(hipGetLastError());
 }
 

@@ -1,0 +1,617 @@
+// Dense quantized convolution as an implicit GEMM on the gfx950 int8 matrix cores.
+//
+//   D[ofm][pixel] = sum_k W[ofm][k] * X[pixel][k],   k = (tap, input feature)
+//
+// computed with v_mfma_i32_16x16x64_i8: the A operand is a 16(ofm) x 64(k) weight tile, the
+// B operand a 64(k) x 16(pixel) activation tile; every lane feeds 16 consecutive k bytes of one
+// row / column, and that is exactly one 16-feature slice of one pixel in fs_b_yx_fsv16 memory
+// (one 128-bit load, no byte shuffling anywhere).
+//
+// Two kernels share this mapping and the epilogue:
+//   conv_mfma_kernel    workgroup = 4 waves, output tile BM pixels x BN features, each wave 64 features x
+//                       WP pixels; per K-step (4 k-chunks = 64 k values) the workgroup stages BN x 64
+//                       weight bytes and BM x 64 activation bytes in LDS (double buffered, one barrier per
+//                       step).  For long K (3x3 and wide 1x1 layers), where operand reuse matters.
+//   conv_stream_kernel  no LDS, no barriers: every wave loads its own fragments straight from global
+//                       memory and walks over all output features.  For short K, where the layer is bound
+//                       by HBM bandwidth and what matters is the number of independent requests in flight.
+// Pixels are the linear index over (batch, oy, ox), so a tile may span rows and images.
+// Two addressing modes:
+//   !CHECKED  the input buffer carries a physical zero border at least as wide as the convolution's
+//             padding, so tap (fy, fx, slice) is a constant byte offset from the pixel: ktab[kc].
+//   CHECKED   taps outside the image are detected per load and read as zero (tile kernel only).
+//
+// u8 activations: the MFMA multiplies signed bytes, so activations are fed as (a ^ 0x80) = a - 128
+// and the accumulators start from 128 * sum(w[f]) (+ the int32 bias), which is exact in int32.
+//
+// Weight rows are stored permuted inside each 64-feature span so that a lane's 16 accumulators
+// of one pixel are 16 CONSECUTIVE features: the int8 result is written with one 128-bit store.
+#pragma once
+#include "epilogue.h"
+#include "kernels.h"
+
+namespace chip {
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+
+// q = n / d for 0 <= n < 2^31 by multiply-high and shift
+struct FastDiv {
+    uint32_t mul, shift, one;
+    __device__ __forceinline__ uint32_t div(uint32_t n) const { return one ? n : (__umulhi(n, mul) >> shift); }
+};
+
+struct MfmaArgs {
+    const int8_t* in;
+    const v4i* wpk;
+    const int32_t* ktab;
+    const int32_t* acc_init;  // [ofm_tiles * BN], natural feature order, zero padded
+    void* out;
+    const void* eltw;
+    int32_t* raw;
+    uint32_t M;
+    int32_t OFM, ofm_tiles, mtiles;
+    int32_t OHW, OW, OH, IH, IW;
+    FastDiv div_ohw, div_ow;
+    int32_t sy, sx, py, px, esy, esx;
+    int32_t in_off, in_pb, in_pf, in_py;       // bytes
+    int32_t out_off, out_pb, out_pf, out_py;   // elements
+    int32_t el_off, el_pb, el_pf, el_py;       // elements
+    int32_t ksteps;
+    // streaming kernel: tap offsets by arithmetic, dense-tensor shortcut
+    int32_t CB, FX, kchunks, tap_dy, tap_dx, linear;
+    FastDiv div_cb, div_fx;
+    uint32_t xor_mask;  // 0x80808080 for u8 activations, 0 for s8
+    FastEpi fe;
+    Epilogue epi;
+};
+
+// epilogue kinds.  GENERIC: every mode and output type, element by element.  FAST: int8 output in the
+// float-requantisation mode, options chosen by run-time flags.  RELU / FUSED: the two forms the ResNet /
+// VGG stacks consist of, with nothing left to decide at run time:
+//   RELU   clamp(acc * cal, 0, hi)                                    (relu, scales >= 0, unit wqf)
+//   FUSED  clamp((round(acc * cal) + residual) * ecal, 0, hi)         (residual relu, scales >= 0)
+enum { EPI_KIND_GENERIC = 0, EPI_KIND_FAST = 1, EPI_KIND_RELU = 2, EPI_KIND_FUSED = 3 };
+template <int EPI> struct epi_is_short { static constexpr bool value = EPI != EPI_KIND_GENERIC; };
+
+// Workgroup barrier that orders LDS traffic only.  __syncthreads() also drains every outstanding
+// global load (loads and stores share one counter on this architecture), which would serialise the
+// K loop on memory latency; the K loop shares nothing through global memory.
+__device__ __forceinline__ void lds_barrier()
+{
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+}
+
+// Uniform table lookups go through the scalar data path (constant address space): a vector load here
+// would sit in the same in-order counter as the prefetched operand loads and force them to drain.
+typedef const int32_t __attribute__((address_space(4))) * const_i32_ptr;
+__device__ __forceinline__ int32_t scalar_table_load(const int32_t* table, int index)
+{
+    return ((const_i32_ptr)(uintptr_t)table)[index];
+}
+
+__device__ __forceinline__ float rha(float v) { return truncf(v + copysignf(0.49999997f, v)); }
+// median of three: one instruction; equals min(max(x, lo), hi) for lo <= hi and x not NaN
+__device__ __forceinline__ float med3(float x, float lo, float hi) { return __builtin_amdgcn_fmed3f(x, lo, hi); }
+__device__ __forceinline__ float relu1(float x) { return __builtin_amdgcn_fmed3f(x, 0.0f, __builtin_inff()); }
+
+// four values already inside [0, 255] -> one dword
+__device__ __forceinline__ int pack_nonneg(const float* v)
+{
+    const unsigned q0 = (unsigned)(int)v[0], q1 = (unsigned)(int)v[1], q2 = (unsigned)(int)v[2], q3 = (unsigned)(int)v[3];
+    return (int)(q0 | (q1 << 8) | (q2 << 16) | (q3 << 24));
+}
+// four values inside [-128, 255] -> one dword of bytes
+__device__ __forceinline__ int pack_signed(const float* v)
+{
+    const unsigned q0 = (unsigned)(int)v[0] & 255u, q1 = (unsigned)(int)v[1] & 255u, q2 = (unsigned)(int)v[2] & 255u;
+    const unsigned q3 = (unsigned)(int)v[3];
+    return (int)(q0 | (q1 << 8) | (q2 << 16) | (q3 << 24));
+}
+
+// ---------------------------------------------------------------------------------------------------
+// Short epilogue for int8 outputs in the float-requantisation mode.  Same operations in the same
+// order as the long form, with three exact rewrites: "round then saturate" becomes "clamp then round"
+// (the bounds are integers), round-half-away is trunc(x + copysign(0.49999997f, x)), and
+// max(0, x) * s becomes clamp(x * s, 0, hi) when s >= 0.  The truncating float->int conversion
+// completes the rounding.
+template <int NT, int EPI>
+__device__ __forceinline__ v4i epilogue_fast16(const MfmaArgs& a, const v4i (&acc)[4][NT], int nt, const float (&wq)[16],
+                                               const float (&cal)[16], const float (&ecal)[16], const v4i& ev4,
+                                               int valid)
+{
+    const FastEpi& F = a.fe;
+    float v[16];
+#pragma unroll
+    for (int c = 0; c < 16; ++c) v[c] = (float)acc[c >> 2][nt][c & 3];
+    if constexpr (EPI == EPI_KIND_RELU || EPI == EPI_KIND_FUSED) {
+        v4i packed;
+        if constexpr (EPI == EPI_KIND_RELU) {
+#pragma unroll
+            for (int c = 0; c < 16; ++c) v[c] = med3(v[c] * cal[c], 0.0f, F.hi) + 0.49999997f;
+        } else {
+            if (F.eltw_u8) {
+#pragma unroll
+                for (int c = 0; c < 16; ++c)
+                    v[c] = rha(v[c] * cal[c]) + (float)(((unsigned)ev4[c >> 2] >> (8 * (c & 3))) & 255u);
+            } else {
+#pragma unroll
+                for (int c = 0; c < 16; ++c)
+                    v[c] = rha(v[c] * cal[c]) + (float)(int)(int8_t)((unsigned)ev4[c >> 2] >> (8 * (c & 3)));
+            }
+#pragma unroll
+            for (int c = 0; c < 16; ++c) v[c] = med3(v[c] * ecal[c], 0.0f, F.hi) + 0.49999997f;
+        }
+#pragma unroll
+        for (int d = 0; d < 4; ++d) packed[d] = pack_nonneg(v + d * 4);
+        if (valid < 16) {
+#pragma unroll
+            for (int d = 0; d < 4; ++d) {
+                unsigned keep = 0;
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                    if (d * 4 + i < valid) keep |= 255u << (8 * i);
+                packed[d] &= (int)keep;
+            }
+        }
+        return packed;
+    }
+    if (F.has_wqf) {
+#pragma unroll
+        for (int c = 0; c < 16; ++c) {
+            v[c] = v[c] * wq[c];
+            v[c] = v[c] * F.iqf;
+        }
+    }
+    v4i packed;
+    bool finished = false;
+    if (F.relu_folded) {
+#pragma unroll
+        for (int c = 0; c < 16; ++c) v[c] = med3(v[c] * cal[c], 0.0f, F.hi) + 0.49999997f;
+#pragma unroll
+        for (int d = 0; d < 4; ++d) packed[d] = pack_nonneg(v + d * 4);
+    } else {
+        if (F.act == CLDNN_HIP_ACT_RELU) {
+#pragma unroll
+            for (int c = 0; c < 16; ++c) v[c] = relu1(v[c]);
+        } else if (F.act == CLDNN_HIP_ACT_CLAMP) {
+#pragma unroll
+            for (int c = 0; c < 16; ++c) v[c] = med3(v[c], F.act_m, F.act_n);
+        }
+#pragma unroll
+        for (int c = 0; c < 16; ++c) v[c] = v[c] * cal[c];
+        if (F.fused) {
+#pragma unroll
+            for (int c = 0; c < 16; ++c) {
+                const float r = rha(v[c]);
+                const unsigned word = (unsigned)ev4[c >> 2];
+                const float e = F.eltw_u8 ? (float)((word >> (8 * (c & 3))) & 255u)
+                                          : (float)(int)(int8_t)(word >> (8 * (c & 3)));
+                v[c] = r + e;
+            }
+            if (F.eltw_relu_folded) {
+#pragma unroll
+                for (int c = 0; c < 16; ++c) v[c] = med3(v[c] * ecal[c], 0.0f, F.hi) + 0.49999997f;
+#pragma unroll
+                for (int d = 0; d < 4; ++d) packed[d] = pack_nonneg(v + d * 4);
+                finished = true;
+            } else if (F.eltw_act == CLDNN_HIP_ACT_RELU) {
+#pragma unroll
+                for (int c = 0; c < 16; ++c) v[c] = relu1(v[c]);
+            } else if (F.eltw_act == CLDNN_HIP_ACT_CLAMP) {
+#pragma unroll
+                for (int c = 0; c < 16; ++c) v[c] = med3(v[c], F.eltw_m, F.eltw_n);
+            }
+            if (!finished && F.has_ecal) {
+#pragma unroll
+                for (int c = 0; c < 16; ++c) v[c] = v[c] * ecal[c];
+            }
+        }
+        if (!finished) {
+#pragma unroll
+            for (int c = 0; c < 16; ++c) {
+                const float y = med3(v[c], F.lo, F.hi);
+                v[c] = y + copysignf(0.49999997f, y);
+            }
+#pragma unroll
+            for (int d = 0; d < 4; ++d) packed[d] = pack_signed(v + d * 4);
+        }
+    }
+    if (valid < 16) {  // partly filled last feature slice: the padding features stay zero
+#pragma unroll
+        for (int d = 0; d < 4; ++d) {
+            unsigned keep = 0;
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+                if (d * 4 + i < valid) keep |= 255u << (8 * i);
+            packed[d] &= (int)keep;
+        }
+    }
+    return packed;
+}
+
+// per-lane requantisation factors of the 16 features a lane finishes
+struct LaneScales {
+    float wq[16], cal[16], ecal[16];
+};
+
+template <int EPI>
+__device__ __forceinline__ void load_scales(const MfmaArgs& a, int f0, LaneScales& sc)
+{
+    if constexpr (EPI == EPI_KIND_RELU || EPI == EPI_KIND_FUSED) {
+        // the host always supplies the vectors these two kinds read (ones where the primitive has none)
+        const Epilogue& e = a.epi;
+#pragma unroll
+        for (int d = 0; d < 4; ++d) {
+            const float4 c4 = *reinterpret_cast<const float4*>(e.calib + f0 + d * 4);
+            sc.cal[d * 4 + 0] = c4.x, sc.cal[d * 4 + 1] = c4.y, sc.cal[d * 4 + 2] = c4.z, sc.cal[d * 4 + 3] = c4.w;
+            if constexpr (EPI == EPI_KIND_FUSED) {
+                const float4 e4 = *reinterpret_cast<const float4*>(e.eltw_calib + f0 + d * 4);
+                sc.ecal[d * 4 + 0] = e4.x, sc.ecal[d * 4 + 1] = e4.y, sc.ecal[d * 4 + 2] = e4.z, sc.ecal[d * 4 + 3] = e4.w;
+            }
+        }
+    } else if constexpr (EPI == EPI_KIND_FAST) {
+        const Epilogue& e = a.epi;
+#pragma unroll
+        for (int d = 0; d < 4; ++d) {
+            float4 c4 = {1.f, 1.f, 1.f, 1.f}, w4 = c4, e4 = c4;
+            if (e.calib) c4 = *reinterpret_cast<const float4*>(e.calib + f0 + d * 4);
+            else if (e.oqf_on) c4 = make_float4(e.oqf, e.oqf, e.oqf, e.oqf);
+            if (a.fe.has_wqf) w4 = *reinterpret_cast<const float4*>(e.wqf + f0 + d * 4);
+            if (a.fe.has_ecal) e4 = *reinterpret_cast<const float4*>(e.eltw_calib + f0 + d * 4);
+            sc.cal[d * 4 + 0] = c4.x, sc.cal[d * 4 + 1] = c4.y, sc.cal[d * 4 + 2] = c4.z, sc.cal[d * 4 + 3] = c4.w;
+            sc.wq[d * 4 + 0] = w4.x, sc.wq[d * 4 + 1] = w4.y, sc.wq[d * 4 + 2] = w4.z, sc.wq[d * 4 + 3] = w4.w;
+            sc.ecal[d * 4 + 0] = e4.x, sc.ecal[d * 4 + 1] = e4.y, sc.ecal[d * 4 + 2] = e4.z, sc.ecal[d * 4 + 3] = e4.w;
+        }
+    }
+}
+
+// Finish the 16 features [f0, f0+16) of one pixel held in acc[.][nt] and store them.
+// obase / ebase: element offsets of (pixel, feature slice) in the output / residual tensor.
+template <int NT, int EPI>
+__device__ __forceinline__ void finish_pixel(const MfmaArgs& a, const v4i (&acc)[4][NT], int nt, int f0, int valid,
+                                             int obase, int ebase, const LaneScales& sc, const v4i& ev4, uint32_t b,
+                                             uint32_t oy, uint32_t ox)
+{
+    const Epilogue& e = a.epi;
+    if constexpr (EPI != EPI_KIND_GENERIC) {
+        const v4i packed = epilogue_fast16<NT, EPI>(a, acc, nt, sc.wq, sc.cal, sc.ecal, ev4, valid);
+        *reinterpret_cast<v4i*>((int8_t*)a.out + obase) = packed;
+    } else {
+        if (a.raw) {
+#pragma unroll
+            for (int c = 0; c < 16; ++c)
+                if (c < valid) a.raw[(((size_t)b * a.OFM + f0 + c) * a.OH + oy) * a.OW + ox] = acc[c >> 2][nt][c & 3];
+        } else {
+            const bool out8 = e.out_dt == CLDNN_HIP_S8 || e.out_dt == CLDNN_HIP_U8;
+            v4i packed = {0, 0, 0, 0};
+#pragma unroll
+            for (int c = 0; c < 16; ++c) {
+                EpiOut o;
+                o.f = 0.f, o.i = 0;
+                if (c < valid) {
+                    float ev = 0.f;
+                    if (e.fused) ev = load_as_float(a.eltw, e.eltw_dt, ebase + c);
+                    o = epilogue_generic(e, acc[c >> 2][nt][c & 3], f0 + c, ev);
+                }
+                if (out8) packed[c >> 2] |= (int)(((unsigned)o.i & 255u) << (8 * (c & 3)));
+                else store_out(a.out, e.out_dt, obase + c, o);
+            }
+            if (out8) *reinterpret_cast<v4i*>((int8_t*)a.out + obase) = packed;
+        }
+    }
+}
+
+struct PixelPos {
+    uint32_t b, oy, ox;
+};
+
+__device__ __forceinline__ PixelPos pixel_pos(const MfmaArgs& a, uint32_t m)
+{
+    PixelPos p;
+    p.b = a.div_ohw.div(m);
+    const uint32_t r = m - p.b * a.OHW;
+    p.oy = a.div_ow.div(r);
+    p.ox = r - p.oy * a.OW;
+    return p;
+}
+
+// =====================================================================================================
+// LDS-staged tile kernel (long K: 3x3 and wide 1x1 layers)
+// =====================================================================================================
+// K-steps of global-load lookahead in the tile kernel, by 16-byte loads per thread and step (even)
+#define MFMA_PREFETCH_DISTANCE(loads) ((loads) <= 2 ? 8 : ((loads) <= 4 ? 4 : 2))
+
+template <int BM, int BN, int WP, bool CHECKED, int EPI>
+__global__ void __launch_bounds__(256) conv_mfma_kernel(MfmaArgs a)
+{
+    constexpr int NT = WP / 16;         // pixel tiles per wave
+    constexpr int WAVES_F = BN / 64;    // waves along features
+    constexpr int A_LOADS = BN / 64;    // 16-byte weight chunks per thread per K-step
+    constexpr int B_LOADS = BM / 64;    // 16-byte activation chunks per thread per K-step
+    constexpr int KC_STRIDE = 256 / BM; // k-chunk distance between a thread's activation loads
+    static_assert((BM / WP) * WAVES_F == 4, "tile must map onto 4 waves");
+
+    const int t = threadIdx.x;
+    const int lane = t & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(t >> 6);
+    const int wave_f = wave % WAVES_F;
+    const int wave_p = wave / WAVES_F;
+    const int kq = lane >> 4;
+    const int l16 = lane & 15;
+
+    // Workgroups that share activation pixels (same pixel tile, different feature tiles) get ids that are
+    // congruent modulo 8 and adjacent in time: they land on the same accelerator die and share its L2.
+    const int xcd = blockIdx.x & 7;
+    const int j = blockIdx.x >> 3;
+    const int ptile = (j / a.ofm_tiles) * 8 + xcd;
+    const int ntile = j % a.ofm_tiles;
+    if (ptile >= a.mtiles) return;
+    const uint32_t m0 = (uint32_t)ptile * BM;
+
+    v4i acc[4][NT];
+    {
+        const int fbase = ntile * BN + wave_f * 64 + kq * 16;
+#pragma unroll
+        for (int mt = 0; mt < 4; ++mt) {
+            const v4i init = *reinterpret_cast<const v4i*>(a.acc_init + fbase + mt * 4);
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt) acc[mt][nt] = init;
+        }
+    }
+    const v4i xm = {(int)a.xor_mask, (int)a.xor_mask, (int)a.xor_mask, (int)a.xor_mask};
+
+    extern __shared__ __align__(16) unsigned char smem[];
+    v4i* ldsA = reinterpret_cast<v4i*>(smem);               // [2][4 * BN]
+    v4i* ldsB = reinterpret_cast<v4i*>(smem) + 2 * 4 * BN;  // [2][4 * BM]
+
+    const int lp = t % BM;
+    const int kc0 = __builtin_amdgcn_readfirstlane(t / BM);
+    const bool ld_valid = m0 + lp < a.M;
+    int iy0, ix0, pix_off;
+    {
+        const PixelPos pp = pixel_pos(a, ld_valid ? m0 + lp : 0);
+        iy0 = (int)pp.oy * a.sy - a.py;
+        ix0 = (int)pp.ox * a.sx - a.px;
+        pix_off = a.in_off + (int)pp.b * a.in_pb + iy0 * a.in_py + ix0 * 16;
+    }
+    const v4i* wsrc = a.wpk + (size_t)ntile * a.ksteps * (4 * BN) + t;
+
+    // Global loads run D K-steps ahead of the multiply: D register sets in rotation.  With one workgroup
+    // per CU (small layers) nothing else hides the memory latency, so the distance has to.  The main loop
+    // is free of branches (the weight stream and the tap table carry D+1 zero steps of slack), which lets
+    // the compiler wait for exactly the oldest set instead of draining the queue.
+    constexpr int D = MFMA_PREFETCH_DISTANCE(A_LOADS + B_LOADS);
+    v4i ra[D][A_LOADS], rb[D][B_LOADS];
+    auto load_global = [&](int ks, v4i (&xa)[A_LOADS], v4i (&xb)[B_LOADS]) {
+#pragma unroll
+        for (int q = 0; q < A_LOADS; ++q) xa[q] = wsrc[(size_t)ks * (4 * BN) + q * 256];
+#pragma unroll
+        for (int q = 0; q < B_LOADS; ++q) {
+            const int e = scalar_table_load(a.ktab, ks * 4 + kc0 + q * KC_STRIDE);
+            if constexpr (!CHECKED) {
+                xb[q] = *reinterpret_cast<const v4i*>(a.in + (pix_off + e));
+            } else {
+                const int iy = iy0 + (e & 1023), ix = ix0 + ((e >> 10) & 1023);
+                const int cb = (e >> 20) & 2047;
+                const bool ok = ld_valid && e >= 0 && iy >= 0 && iy < a.IH && ix >= 0 && ix < a.IW;
+                v4i v = {0, 0, 0, 0};
+                if (ok)
+                    v = *reinterpret_cast<const v4i*>(a.in + (pix_off + cb * a.in_pf + (e & 1023) * a.in_py
+                                                              + ((e >> 10) & 1023) * 16));
+                xb[q] = v;
+            }
+        }
+    };
+    auto store_lds = [&](int buf, const v4i (&xa)[A_LOADS], const v4i (&xb)[B_LOADS]) {
+#pragma unroll
+        for (int q = 0; q < A_LOADS; ++q) ldsA[buf * 4 * BN + t + q * 256] = xa[q];
+#pragma unroll
+        for (int q = 0; q < B_LOADS; ++q) ldsB[buf * 4 * BM + (kc0 + q * KC_STRIDE) * BM + lp] = xb[q];
+    };
+    const int arow = wave_f * 64 + l16;
+    const int bcol = wave_p * WP + l16;
+    auto compute = [&](int buf) {
+        v4i fa[4], fb[NT];
+#pragma unroll
+        for (int mt = 0; mt < 4; ++mt) fa[mt] = ldsA[buf * 4 * BN + kq * BN + arow + mt * 16];
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) fb[nt] = ldsB[buf * 4 * BM + kq * BM + bcol + nt * 16] ^ xm;
+#pragma unroll
+        for (int mt = 0; mt < 4; ++mt)
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt)
+                acc[mt][nt] = __builtin_amdgcn_mfma_i32_16x16x64_i8(fa[mt], fb[nt], acc[mt][nt], 0, 0, 0);
+    };
+
+#pragma unroll
+    for (int d = 0; d < D; ++d) load_global(d, ra[d], rb[d]);
+    store_lds(0, ra[0], rb[0]);
+    load_global(D, ra[0], rb[0]);
+    lds_barrier();
+    const int main_steps = (a.ksteps / D) * D;
+    for (int ks0 = 0; ks0 < main_steps; ks0 += D) {
+#pragma unroll
+        for (int d = 0; d < D; ++d) {
+            const int ks = ks0 + d;
+            compute(d & 1);  // D is even: the LDS buffer of step ks is ks & 1 == d & 1
+            // K-step ks+1 sits in set (d+1)%D, requested D-1 steps ago; refill the set with step ks+1+D
+            store_lds((d & 1) ^ 1, ra[(d + 1) % D], rb[(d + 1) % D]);
+            load_global(ks + 1 + D, ra[(d + 1) % D], rb[(d + 1) % D]);
+            lds_barrier();
+        }
+    }
+    const int rest = a.ksteps - main_steps;  // < D steps left; their operands are already on the way
+#pragma unroll
+    for (int d = 0; d < D - 1; ++d) {
+        if (d < rest) {
+            compute(d & 1);
+            store_lds((d & 1) ^ 1, ra[(d + 1) % D], rb[(d + 1) % D]);
+            lds_barrier();
+        }
+    }
+
+    // ---- epilogue: lane (kq, l16) holds, for each pixel tile, features f0 .. f0+15 of one pixel
+    const int f0 = ntile * BN + wave_f * 64 + kq * 16;
+    if (f0 >= a.OFM) return;
+    const int fs = f0 >> 4;
+    const int valid = a.OFM - f0;  // >= 16 except in the last, partly filled slice
+    LaneScales sc;
+    load_scales<EPI>(a, f0, sc);
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) {
+        const uint32_t m = m0 + wave_p * WP + nt * 16 + l16;
+        if (m < a.M) {
+            const PixelPos pp = pixel_pos(a, m);
+            const int obase = a.out_off + (int)pp.b * a.out_pb + fs * a.out_pf + (int)pp.oy * a.out_py + (int)pp.ox * 16;
+            const int ebase = a.el_off + (int)pp.b * a.el_pb + fs * a.el_pf + (int)(pp.oy * a.esy) * a.el_py
+                              + (int)(pp.ox * a.esx) * 16;
+            v4i ev4 = {0, 0, 0, 0};
+            if constexpr (EPI == EPI_KIND_FUSED) ev4 = *reinterpret_cast<const v4i*>((const int8_t*)a.eltw + ebase);
+            else if constexpr (EPI == EPI_KIND_FAST)
+                if (a.fe.fused) ev4 = *reinterpret_cast<const v4i*>((const int8_t*)a.eltw + ebase);
+            finish_pixel<NT, EPI>(a, acc, nt, f0, valid, obase, ebase, sc, ev4, pp.b, pp.oy, pp.ox);
+        }
+    }
+}
+
+// =====================================================================================================
+// Streaming kernel (short K, bandwidth-bound layers): no LDS, no barriers, no tables.
+// A wave owns ONE span of 64 output features of ONE pixel tile (16*NT pixels).  Its MFMA fragments come
+// straight from global memory (a fragment of lane l IS a contiguous 16-byte piece of fs_b_yx_fsv16
+// memory).  Everything the tile needs - activations of all K-steps, weights, residual, requantisation
+// factors - is requested before anything is waited for, so a wave pays one memory round trip; it uses
+// few registers, so many waves per SIMD overlap their round trips and keep HBM busy.  The four waves
+// of a workgroup take the same pixels and neighbouring spans: the activations reach three of them
+// through L1.  KS = number of K-steps, fixed at compile time (the host pads the weight stream with
+// zero K-chunks).  Needs constant tap offsets (input with a sufficient zero border, or no padding).
+// =====================================================================================================
+template <int NT, int KS, int EPI>
+__global__ void __launch_bounds__(256) conv_stream_kernel(MfmaArgs a)
+{
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int kq = lane >> 4;
+    const int l16 = lane & 15;
+    const uint32_t gw = blockIdx.x * 4u + (uint32_t)wave;
+    const int nspans = a.ofm_tiles;
+    const int span = (int)(gw % (uint32_t)nspans);
+    const uint32_t pt = gw / (uint32_t)nspans;
+    if (pt >= (uint32_t)a.mtiles) return;  // no barriers below: a wave may leave on its own
+
+    const int f0 = span * 64 + kq * 16;
+    const int fs = f0 >> 4;
+    const bool live = f0 < a.OFM;
+    const int valid = a.OFM - f0;
+
+    // tap offsets of this lane's K-chunks, computed instead of looked up (a table load would put a second
+    // memory round trip in front of the activation loads)
+    int koff[KS];
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+        const uint32_t kc = ks * 4 + kq;
+        const uint32_t tap = a.div_cb.div(kc);
+        const uint32_t cb = kc - tap * a.CB;
+        const uint32_t fy = a.div_fx.div(tap);
+        const uint32_t fx = tap - fy * a.FX;
+        koff[ks] = kc < (uint32_t)a.kchunks ? (int)(cb * a.in_pf + fy * a.tap_dy + fx * a.tap_dx) : 0;
+    }
+
+    // ---- requests
+    v4i fb[KS][NT], ev[NT], fa[KS][4], init[4];
+    int ob[NT], eb[NT];
+    PixelPos pos[NT];
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) {
+        const uint32_t m = pt * (16u * NT) + nt * 16 + l16;
+        const uint32_t mm = m < a.M ? m : a.M - 1;
+        int pix, o, e;
+        if (a.linear) {  // dense tensors, 1x1 / stride 1: pixel m sits at m * 16, no division needed
+            pix = a.in_off + (int)mm * 16;
+            o = a.out_off + fs * a.out_pf + (int)mm * 16;
+            e = a.el_off + fs * a.el_pf + (int)mm * 16;
+            pos[nt] = PixelPos{0, 0, 0};
+        } else {
+            const PixelPos pp = pixel_pos(a, mm);
+            pos[nt] = pp;
+            pix = a.in_off + (int)pp.b * a.in_pb + ((int)pp.oy * a.sy - a.py) * a.in_py + ((int)pp.ox * a.sx - a.px) * 16;
+            o = a.out_off + (int)pp.b * a.out_pb + fs * a.out_pf + (int)pp.oy * a.out_py + (int)pp.ox * 16;
+            e = a.el_off + (int)pp.b * a.el_pb + fs * a.el_pf + (int)(pp.oy * a.esy) * a.el_py + (int)(pp.ox * a.esx) * 16;
+        }
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) fb[ks][nt] = *reinterpret_cast<const v4i*>(a.in + (pix + koff[ks]));
+        ob[nt] = m < a.M ? o : -1;
+        eb[nt] = e;
+        ev[nt] = v4i{0, 0, 0, 0};
+        if constexpr (EPI == EPI_KIND_FUSED) {
+            if (live) ev[nt] = *reinterpret_cast<const v4i*>((const int8_t*)a.eltw + e);
+        } else if constexpr (EPI == EPI_KIND_FAST) {
+            if (a.fe.fused && live) ev[nt] = *reinterpret_cast<const v4i*>((const int8_t*)a.eltw + e);
+        }
+    }
+    const v4i* wsrc = a.wpk + (size_t)span * KS * 256 + kq * 64 + l16;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks)
+#pragma unroll
+        for (int mt = 0; mt < 4; ++mt) fa[ks][mt] = wsrc[ks * 256 + mt * 16];
+#pragma unroll
+    for (int mt = 0; mt < 4; ++mt) init[mt] = *reinterpret_cast<const v4i*>(a.acc_init + f0 + mt * 4);
+    LaneScales sc;
+    if (live) load_scales<EPI>(a, f0, sc);
+
+    // ---- multiply
+    const v4i xm = {(int)a.xor_mask, (int)a.xor_mask, (int)a.xor_mask, (int)a.xor_mask};
+    v4i acc[4][NT];
+#pragma unroll
+    for (int mt = 0; mt < 4; ++mt)
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) acc[mt][nt] = init[mt];
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) fb[ks][nt] = fb[ks][nt] ^ xm;
+#pragma unroll
+        for (int mt = 0; mt < 4; ++mt)
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt)
+                acc[mt][nt] = __builtin_amdgcn_mfma_i32_16x16x64_i8(fa[ks][mt], fb[ks][nt], acc[mt][nt], 0, 0, 0);
+    }
+
+    // ---- requantise and store
+    if (live) {
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) {
+            if (ob[nt] >= 0) {
+                PixelPos pp = pos[nt];
+                if constexpr (EPI == EPI_KIND_GENERIC)
+                    if (a.linear) pp = pixel_pos(a, pt * (16u * NT) + nt * 16 + l16);
+                finish_pixel<NT, EPI>(a, acc, nt, f0, valid, ob[nt], eb[nt], sc, ev[nt], pp.b, pp.oy, pp.ox);
+            }
+        }
+    }
+}
+
+template <int BM, int BN, int WP, bool CHECKED>
+void launch_mfma_instance(hipStream_t s, const MfmaArgs& a, int grid, int lds, int epi)
+{
+    const dim3 g(grid), b(256);
+    switch (epi) {
+    case EPI_KIND_RELU: hipLaunchKernelGGL((conv_mfma_kernel<BM, BN, WP, CHECKED, EPI_KIND_RELU>), g, b, lds, s, a); break;
+    case EPI_KIND_FUSED: hipLaunchKernelGGL((conv_mfma_kernel<BM, BN, WP, CHECKED, EPI_KIND_FUSED>), g, b, lds, s, a); break;
+    case EPI_KIND_FAST: hipLaunchKernelGGL((conv_mfma_kernel<BM, BN, WP, CHECKED, EPI_KIND_FAST>), g, b, lds, s, a); break;
+    default: hipLaunchKernelGGL((conv_mfma_kernel<BM, BN, WP, CHECKED, EPI_KIND_GENERIC>), g, b, lds, s, a); break;
+    }
+}
+
+template <int NT, int KS>
+void launch_stream_instance(hipStream_t s, const MfmaArgs& a, int grid, int epi)
+{
+    const dim3 g(grid), b(256);
+    switch (epi) {
+    case EPI_KIND_RELU: hipLaunchKernelGGL((conv_stream_kernel<NT, KS, EPI_KIND_RELU>), g, b, 0, s, a); break;
+    case EPI_KIND_FUSED: hipLaunchKernelGGL((conv_stream_kernel<NT, KS, EPI_KIND_FUSED>), g, b, 0, s, a); break;
+    case EPI_KIND_FAST: hipLaunchKernelGGL((conv_stream_kernel<NT, KS, EPI_KIND_FAST>), g, b, 0, s, a); break;
+    default: hipLaunchKernelGGL((conv_stream_kernel<NT, KS, EPI_KIND_GENERIC>), g, b, 0, s, a); break;
+    }
+}
+
+}  // namespace chip

@@ -18,7 +18,7 @@ void launch_conv_ref(hipStream_t s, const ConvProblem& p, const Epilogue& epi, c
                      const void* eltw, void* out, int* acc_out);
 void launch_reorder(hipStream_t s, const cldnn_hip_tensor& st, const void* src, const cldnn_hip_tensor& dt, void* dst);
 
-// ---- implicit-GEMM int8 MFMA kernel on fs_b_yx_fsv16 (conv_mfma.hip)
+// ---- implicit-GEMM int8 MFMA kernel on fs_b_yx_fsv16 (conv_mfma*.hip)
 struct TileConfig {
     const char* name;
     int tile_pixels;  // BM: output pixels per workgroup
@@ -28,19 +28,24 @@ struct TileConfig {
 int tile_config_count();
 const TileConfig& tile_config(int i);
 
-// Pre-packed weights of one convolution for the MFMA kernel.
+// Pre-packed weights and launch geometry of one convolution for the MFMA kernel.
 struct MfmaPlan {
     int tile;            // row of the tile table
-    int cb;              // input feature slices of 16 (per group)
+    int stream;          // 1: streaming kernel (no LDS), 0: LDS-staged tile kernel
+    int checked;         // 1: taps bounds-checked per load, 0: input carries a sufficient zero border
+    int cb;              // input feature slices of 16
     int kchunks;         // FY*FX*cb
     int ksteps;          // ceil(kchunks / 4)
     int ofm_tiles;       // ceil(OFM / tile_ofm)
+    int mtiles;          // ceil(M / tile_pixels)
     int64_t m_total;     // B*OH*OW
     int grid;
     int lds_bytes;
     size_t packed_bytes; // device bytes of the packed weight stream
     size_t ktab_bytes;
 };
+// table lookup: row of the tile table for a problem
+int mfma_choose(const ConvProblem& p, int cus);
 MfmaPlan mfma_plan(const ConvProblem& p, int tile);
 // host-side packing: weights [OFM][IFM][FY][FX] s8 -> MFMA operand stream, ktab -> per-kchunk tap table
 void mfma_pack_weights(const ConvProblem& p, const MfmaPlan& plan, const int8_t* w, int8_t* packed, int32_t* ktab);
@@ -48,13 +53,28 @@ struct MfmaBuffers {
     const int8_t* packed;
     const int32_t* ktab;
 };
-enum { EPI_GENERIC = 0, EPI_RAW = 1, EPI_FAST = 2 };
-// true when the short epilogue (convert, scale, clamp, round) reproduces the generic one bit for bit
-bool mfma_fast_epilogue_ok(const ConvProblem& p, const Epilogue& e, const float* calib_host, const float* ecal_host,
-                           const float* wqf_host, int ofm);
-// acc_init: per-feature int32 start value of the accumulators, padded to ofm_tiles * tile_ofm
+// parameters of the short epilogue (int8 output, float requantisation)
+struct FastEpi {
+    int32_t has_wqf;      // multiply by wqf[f] and iqf
+    int32_t act;          // CLDNN_HIP_ACT_NONE / RELU / CLAMP
+    float act_m, act_n;
+    int32_t relu_folded;  // relu with non-negative scales: folded into the final clamp
+    int32_t fused;
+    int32_t eltw_act;     // NONE / RELU / CLAMP
+    float eltw_m, eltw_n;
+    int32_t has_ecal;
+    int32_t eltw_relu_folded;  // residual relu with non-negative scales: folded into the final clamp
+    int32_t eltw_u8;
+    float lo, hi;         // saturation bounds of the output type
+    float iqf;
+};
+// true (and *out filled) when the short epilogue reproduces the long one bit for bit
+bool mfma_fast_epilogue(const ConvProblem& p, const Epilogue& e, const float* calib, const float* ecal, const float* wqf,
+                        FastEpi* out);
+// acc_init: per-feature int32 start value of the accumulators, padded to ofm_tiles * tile_ofm.
+// fast == nullptr selects the long epilogue; raw != nullptr dumps the int32 accumulators instead.
 void launch_conv_mfma(hipStream_t s, const ConvProblem& p, const MfmaPlan& plan, const MfmaBuffers& wb,
-                      const int32_t* acc_init, const Epilogue& epi, int epi_kind, const void* in, const void* eltw,
+                      const int32_t* acc_init, const Epilogue& epi, const FastEpi* fast, const void* in, const void* eltw,
                       void* out, int32_t* raw);
 
 // ---- depthwise bandwidth kernel on fs_b_yx_fsv16 (conv_dw.hip)

@@ -195,7 +195,7 @@ typedef struct {
     int32_t second_input_in_output; /* residual is read from the output buffer itself */
     int32_t round_to_even;        /* 0 = reference behaviour (half away from zero) */
     int32_t impl;                 /* CLDNN_HIP_IMPL_* */
-    int32_t tile_override;        /* 0 = table; otherwise index+1 into the tile-config table (tuning / tests) */
+    int32_t tile_override;        /* 0 = table decides; otherwise row + 1 of the tile-config table (tuning / tests) */
 } cldnn_hip_conv_desc;
 
 /* Host pointers: weights [ofm][ifm/groups][fy][fx] dense, bias/wqf/calib/eltw_calib [ofm] or NULL.

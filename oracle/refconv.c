@@ -57,6 +57,26 @@ float rc_round_half_away(float x)
     return roundf(x);
 }
 
+/*
+ * The HIP epilogue rounds with trunc(x + copysign(0.49999997f, x)) (0.49999997f is the largest float
+ * below one half).  Count the finite floats for which that differs from roundf: must be zero.
+ */
+long rc_count_round_trick_mismatches(void)
+{
+    long bad = 0;
+#ifdef _OPENMP
+#pragma omp parallel for reduction(+ : bad) schedule(static)
+#endif
+    for (int64_t u = 0; u < ((int64_t)1 << 32); ++u) {
+        uint32_t b = (uint32_t)u;
+        float x;
+        memcpy(&x, &b, 4);
+        if (!(x == x) || isinf(x)) continue;
+        if (roundf(x) != truncf(x + copysignf(0.49999997f, x))) ++bad;
+    }
+    return bad;
+}
+
 static float rnd(const rc_desc* d, float x)
 {
     return d->round_even ? nearbyintf(x) : roundf(x);

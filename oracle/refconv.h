@@ -19,7 +19,7 @@
  *   tests/test_cases/convolution_gpu_test.cpp:5582-5705                   host loop skeleton
  *
  * Parity pinning: every function here is pinned by the reference's own
- * known-answer tables (tests/golden/*.json, taken from
+ * known-answer tables (tests/golden/conv_kat.json, taken from
  * tests/test_cases/convolution_gpu_test.cpp and
  * tests/test_cases/fused_conv_eltwise_gpu_test.cpp) and by closed-form /
  * brute-force checks in tests/test_oracle.py.  The reference itself cannot be
@@ -101,6 +101,7 @@ double rc_epilogue(const rc_desc* d, int32_t acc, int f, const void* bias, const
 /* Helpers exposed for tests. */
 float rc_round_half_away(float x);
 int   rc_threads_available(void);
+long  rc_count_round_trick_mismatches(void);
 
 #ifdef __cplusplus
 }

@@ -121,34 +121,56 @@ def tiles():
     return list(range(1, hip.lib().cldnn_hip_tile_config_count() + 1))
 
 
+def tile_names():
+    L = hip.lib()
+    return [L.cldnn_hip_tile_config_name(i).decode() for i in range(L.cldnn_hip_tile_config_count())]
+
+
 @pytest.mark.parametrize("shape", SHAPES, ids=lambda s: "x".join(map(str, s[:7])))
 @pytest.mark.parametrize("in_dt", [np.uint8, np.int8], ids=["u8", "s8"])
 def test_mfma_kernel_all_tiles(eng, shape, in_dt):
+    """every row of the tile table (LDS-staged and streaming kernels) x both addressing modes"""
     B, IFM, H, W, OFM, FY, FX, stride, pad = shape
     x, w, bias, wqf, calib = problem(12, B, IFM, H, W, OFM, FY, FX, in_dt)
     ref_o, ref_a = rc.conv(x, w, bias, wqf=wqf, calib=calib, stride=stride, pad=pad, out_dt="s8", act="relu",
                            want_acc=True)
-    for tile in [0] + tiles():
-        go, ga, info = hip.conv_forward(eng, x, w, bias, wqf, calib, stride=stride, pad=pad, out_dt="s8", act="relu",
-                                        fmt="fs_b_yx_fsv16", tile=tile, want_acc=True, want_info=True)
-        assert info.impl == hip.IMPL_MFMA, info.kernel_name
-        assert b"fast" in info.kernel_name
-        np.testing.assert_array_equal(ga, ref_a, err_msg=info.kernel_name.decode())
-        assert_same(ref_o, go)
+    names = tile_names()
+    seen = set()
+    for border in (True, False):
+        in_pad = (pad[0] + (1 if FY > 1 else 0), pad[1]) if border else (0, 0)
+        for tile in [0] + tiles():
+            kw = dict(stride=stride, pad=pad, out_dt="s8", act="relu", fmt="fs_b_yx_fsv16", in_pad=in_pad, tile=tile,
+                      want_acc=True, want_info=True)
+            ksteps = -(-(FY * FX * -(-IFM // 16)) // 4)
+            if tile and names[tile - 1].startswith(("stream", "shot")) and ((not border and pad != (0, 0)) or ksteps > 8):
+                with pytest.raises(hip.HipError):  # needs constant tap offsets (zero border) and K <= 512
+                    hip.conv_forward(eng, x, w, bias, wqf, calib, **kw)
+                continue
+            go, ga, info = hip.conv_forward(eng, x, w, bias, wqf, calib, **kw)
+            name = info.kernel_name.decode()
+            assert info.impl == hip.IMPL_MFMA and "fast" in name, name
+            seen.add(name)
+            np.testing.assert_array_equal(ga, ref_a, err_msg=name)
+            assert_same(ref_o, go)
+    assert any("conv_mfma" in n and "border" in n for n in seen)
+    assert any("stream" in n for n in seen) == (-(-(FY * FX * -(-IFM // 16)) // 4) <= 8)
+    if pad != (0, 0):
+        assert any("checked" in n for n in seen)
 
 
 @pytest.mark.parametrize("out_dt", ["s8", "u8", "f32"])
 @pytest.mark.parametrize("act", [("none", 0, 0), ("relu", 0, 0), ("relu_slope", 0.1, 0), ("clamp", 0.0, 6.0)],
                          ids=lambda a: a[0])
-def test_mfma_generic_epilogue_variants(eng, out_dt, act):
+def test_mfma_epilogue_variants(eng, out_dt, act):
     x, w, bias, wqf, calib = problem(13, 2, 64, 12, 12, 96, 3, 3)
     r = np.random.default_rng(3)
     wqf = (3.0 / (np.sqrt(576) * 147.4 * 73.3) * r.uniform(0.5, 2, 96)).astype(np.float32)
     calib = np.full(96, 127 / 6, np.float32) * r.uniform(0.9, 1.1, 96).astype(np.float32)
-    calib[::7] *= -1  # negative scale: not eligible for the short epilogue
+    calib[::7] *= -1  # negative scales: relu cannot be folded into the final clamp
     kw = dict(stride=(1, 1), pad=(1, 1), out_dt=out_dt, act=act[0], act_m=act[1], act_n=act[2], iqf=0.75)
     (ro, ra), (go, ga, info) = both(eng, x, w, bias, wqf, calib, fmt="fs_b_yx_fsv16", **kw)
-    assert b"generic" in info.kernel_name
+    # the short epilogue covers int8 outputs with none / relu / clamp; everything else takes the long form
+    assert (b"generic" in info.kernel_name) == (out_dt == "f32" or act[0] == "relu_slope")
     np.testing.assert_array_equal(ga, ra)
     assert_same(ro, go)
 
@@ -182,8 +204,11 @@ def test_mfma_fused_eltwise(eng, fast, eltw_dt):
     ecal = r.uniform(0.3, 1.2, 256).astype(np.float32)
     kw = dict(out_dt="s8", act="none", eltw=e, eltw_act="relu", eltw_calib=ecal,
               non_conv_scale=1.0 if fast else 0.5)
-    (ro, ra), (go, ga, info) = both(eng, x, w, bias, wqf, calib, fmt="fs_b_yx_fsv16", **kw)
-    assert (b"fast" in info.kernel_name) == fast
+    for tile in (0, 1, 6, 7, 8):
+        (ro, ra), (go, ga, info) = both(eng, x, w, bias, wqf, calib, fmt="fs_b_yx_fsv16", tile=tile, **kw)
+        assert (b"fast" in info.kernel_name) == fast
+        np.testing.assert_array_equal(ga, ra)
+        assert_same(ro, go)
     np.testing.assert_array_equal(ga, ra)
     assert_same(ro, go)
 

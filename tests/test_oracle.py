@@ -218,6 +218,13 @@ def test_round_half_away():
         assert L.rc_round_half_away(v) == e
 
 
+def test_truncation_rounding_identity_holds_for_every_float():
+    # the HIP epilogue computes round-half-away as trunc(x + copysign(pred(0.5), x)); exhaustive over 2^32 patterns
+    L = rc.lib()
+    L.rc_count_round_trick_mismatches.restype = __import__("ctypes").c_long
+    assert L.rc_count_round_trick_mismatches() == 0
+
+
 def test_output_extent_formula():
     # closed form vs the reference test helper get_expected_output_tensor
     # (tests/test_cases/convolution_gpu_test.cpp:5524-5542)
