@@ -153,6 +153,7 @@ def main():
                     choices=["resnet50_b32_fused", "resnet50_b32", "resnet50_b1", "vgg16_b16", "mobilenet_v2_b32", "c1"])
     ap.add_argument("--tile", type=int, default=0, help="force one row (index+1) of the tile table on every layer")
     ap.add_argument("--per-layer", action="store_true", help="time every layer on its own and print a table to stderr")
+    ap.add_argument("--tune", action="store_true", help="try every row of the tile table on every layer, print the best")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline / full-size check")
     ap.add_argument("--cpu-seconds", type=float, default=15.0)
     args = ap.parse_args()
@@ -197,26 +198,56 @@ def main():
     value = batch * args.steps / t_wall
 
     per_layer = None
-    if args.per_layer:
-        per_layer = []
-        reps = max(5, args.steps // 2)
-        for L in stack:
-            for _ in range(2):
-                L.conv.enqueue(L.xin, L.out, L.ein)
-            with GpuTimer(eng) as lt:
-                for _ in range(reps):
-                    L.conv.enqueue(L.xin, L.out, L.ein)
-            eng.finish()
-            dt = lt.seconds() / reps
-            per_layer.append((L, dt))
-        log("%-18s %-34s %6s %9s %8s %8s %7s" % ("layer", "kernel", "grid", "us", "TOP/s", "GB/s", "bound"))
-        for L, dt in per_layer:
-            tops, gbs = L.info.ops / dt / 1e12, L.info.bytes / dt / 1e9
-            t_m, t_h = L.info.ops / PEAK_INT8_OPS, L.info.bytes / PEAK_HBM
-            log("%-18s %-34s %6d %9.1f %8.1f %8.0f %7s %5.1f%%" % (
-                L.spec["name"], L.info.kernel_name.decode(), L.info.grid, dt * 1e6, tops, gbs,
-                "mfma" if t_m > t_h else "hbm", 100 * max(t_m, t_h) / dt))
-        log("sum of per-layer times: %.1f us" % (sum(dt for _, dt in per_layer) * 1e6))
+    if args.per_layer or args.tune:
+        def time_layers(stk, steps):
+            """per-layer GPU time inside whole steps (so every layer starts with cold caches, as in the real run)"""
+            acc = [0.0] * len(stk)
+            for _ in range(steps):
+                timers = []
+                for L in stk:
+                    tmr = GpuTimer(eng)
+                    with tmr:
+                        L.conv.enqueue(L.xin, L.out, L.ein)
+                    timers.append(tmr)
+                eng.finish()
+                for i, tmr in enumerate(timers):
+                    acc[i] += tmr.seconds()
+            return [v / steps for v in acc]
+
+        def table(stk, times):
+            log("%-18s %-40s %6s %9s %8s %8s %7s" % ("layer", "kernel", "grid", "us", "TOP/s", "GB/s", "bound"))
+            for L, dt in zip(stk, times):
+                tops, gbs = L.info.ops / dt / 1e12, L.info.bytes / dt / 1e9
+                t_m, t_h = L.info.ops / PEAK_INT8_OPS, L.info.bytes / PEAK_HBM
+                log("%-18s %-40s %6d %9.1f %8.1f %8.0f %7s %5.1f%%" % (
+                    L.spec["name"], L.info.kernel_name.decode(), L.info.grid, dt * 1e6, tops, gbs,
+                    "mfma" if t_m > t_h else "hbm", 100 * max(t_m, t_h) / dt))
+            log("sum of per-layer times: %.1f us" % (sum(times) * 1e6))
+
+        per_layer = time_layers(stack, max(3, args.steps // 3))
+        table(stack, per_layer)
+        if args.tune:
+            # every row of the tile table forced on every layer where it applies; report the best row per layer
+            names = [hip.lib().cldnn_hip_tile_config_name(i).decode() for i in range(hip.lib().cldnn_hip_tile_config_count())]
+            best = [(t, "table:" + L.info.kernel_name.decode()) for t, L in zip(per_layer, stack)]
+            for row in range(1, len(names) + 1):
+                alt = build_stack(eng, layers, batch, fuse, tile=row)
+                for _ in range(2):
+                    run_step(alt)
+                times = time_layers(alt, max(3, args.steps // 3))
+                for i, (t, L) in enumerate(zip(times, alt)):
+                    if L.info.tile_index == row - 1 and t < best[i][0]:
+                        best[i] = (t, names[row - 1])
+                for L in alt:
+                    L.conv.close(); L.out.close(); L.xin.close()
+                    if L.ein is not None:
+                        L.ein.close()
+            log("%-18s %6s %6s %5s %3s %9s %9s  %s" % ("layer", "M", "OFM", "K", "k", "table us", "best us", "best row"))
+            for L, t0, (t1, nm) in zip(stack, per_layer, best):
+                l = L.spec
+                log("%-18s %6d %6d %5d %3d %9.1f %9.1f  %s" % (l["name"], batch * l["out_hw"] ** 2, l["ofm"],
+                                                             l["ifm"] * l["k"] ** 2, l["k"], t0 * 1e6, t1 * 1e6, nm))
+            log("sum with the table: %.1f us; sum of per-layer bests: %.1f us" % (sum(per_layer) * 1e6, sum(t for t, _ in best) * 1e6))
 
     res = {
         "metric": "ResNet-50 int8 conv stack images/sec @b32; achieved TOPS vs INT8 MFMA peak"

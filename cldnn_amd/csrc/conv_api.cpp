@@ -351,4 +351,27 @@ cldnn_hip_status cldnn_hip_reorder(cldnn_hip_engine e, const void* src_dev, cons
     });
 }
 
+cldnn_hip_status cldnn_hip_activation(cldnn_hip_engine e, const void* src_dev, const cldnn_hip_tensor* src, void* dst_dev,
+                                      const cldnn_hip_tensor* dst, int32_t activation, float m, float n)
+{
+    return guarded([&] {
+        CHIP_REQUIRE(e && src_dev && src && dst_dev && dst, CLDNN_HIP_INVALID_ARG, "null argument");
+        e->make_current();
+        launch_pointwise(e->stream, *src, src_dev, nullptr, nullptr, *dst, dst_dev, 0, nullptr, 1.0f, activation, m, n);
+    });
+}
+
+cldnn_hip_status cldnn_hip_eltwise_sum(cldnn_hip_engine e, const void* a_dev, const cldnn_hip_tensor* a, const void* b_dev,
+                                       const cldnn_hip_tensor* b, void* dst_dev, const cldnn_hip_tensor* dst,
+                                       int32_t quantized, const float* calib_dev, float output_quantization_factor,
+                                       int32_t activation, float m, float n)
+{
+    return guarded([&] {
+        CHIP_REQUIRE(e && a_dev && a && b_dev && b && dst_dev && dst, CLDNN_HIP_INVALID_ARG, "null argument");
+        e->make_current();
+        launch_pointwise(e->stream, *a, a_dev, b, b_dev, *dst, dst_dev, quantized, calib_dev, output_quantization_factor,
+                         activation, m, n);
+    });
+}
+
 }  // extern "C"

@@ -255,9 +255,10 @@ void launch_conv_mfma(hipStream_t s, const ConvProblem& p, const MfmaPlan& pl, c
     if (fast && !raw) {
         a.fe = *fast;
         kind = EPI_KIND_FAST;
-        // the two branch-free forms (the host keeps vectors of ones where the primitive has no factors)
+        // the branch-free forms
         if (!fast->has_wqf && epi.calib) {
             if (!fast->fused && fast->relu_folded) kind = EPI_KIND_RELU;
+            if (!fast->fused && fast->act == CLDNN_HIP_ACT_NONE) kind = EPI_KIND_LINEAR;
             if (fast->fused && fast->act == CLDNN_HIP_ACT_NONE && fast->eltw_relu_folded && epi.eltw_calib) kind = EPI_KIND_FUSED;
         }
     }

@@ -70,7 +70,8 @@ struct MfmaArgs {
 // VGG stacks consist of, with nothing left to decide at run time:
 //   RELU   clamp(acc * cal, 0, hi)                                    (relu, scales >= 0, unit wqf)
 //   FUSED  clamp((round(acc * cal) + residual) * ecal, 0, hi)         (residual relu, scales >= 0)
-enum { EPI_KIND_GENERIC = 0, EPI_KIND_FAST = 1, EPI_KIND_RELU = 2, EPI_KIND_FUSED = 3 };
+//   LINEAR clamp(acc * cal, lo, hi)                                   (no activation, unit wqf)
+enum { EPI_KIND_GENERIC = 0, EPI_KIND_FAST = 1, EPI_KIND_RELU = 2, EPI_KIND_FUSED = 3, EPI_KIND_LINEAR = 4 };
 template <int EPI> struct epi_is_short { static constexpr bool value = EPI != EPI_KIND_GENERIC; };
 
 // Workgroup barrier that orders LDS traffic only.  __syncthreads() also drains every outstanding
@@ -123,6 +124,27 @@ __device__ __forceinline__ v4i epilogue_fast16(const MfmaArgs& a, const v4i (&ac
     float v[16];
 #pragma unroll
     for (int c = 0; c < 16; ++c) v[c] = (float)acc[c >> 2][nt][c & 3];
+    if constexpr (EPI == EPI_KIND_LINEAR) {
+        v4i packed;
+#pragma unroll
+        for (int c = 0; c < 16; ++c) {
+            const float y = med3(v[c] * cal[c], F.lo, F.hi);
+            v[c] = y + copysignf(0.49999997f, y);
+        }
+#pragma unroll
+        for (int d = 0; d < 4; ++d) packed[d] = pack_signed(v + d * 4);
+        if (valid < 16) {
+#pragma unroll
+            for (int d = 0; d < 4; ++d) {
+                unsigned keep = 0;
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                    if (d * 4 + i < valid) keep |= 255u << (8 * i);
+                packed[d] &= (int)keep;
+            }
+        }
+        return packed;
+    }
     if constexpr (EPI == EPI_KIND_RELU || EPI == EPI_KIND_FUSED) {
         v4i packed;
         if constexpr (EPI == EPI_KIND_RELU) {
@@ -237,8 +259,8 @@ struct LaneScales {
 template <int EPI>
 __device__ __forceinline__ void load_scales(const MfmaArgs& a, int f0, LaneScales& sc)
 {
-    if constexpr (EPI == EPI_KIND_RELU || EPI == EPI_KIND_FUSED) {
-        // the host always supplies the vectors these two kinds read (ones where the primitive has none)
+    if constexpr (EPI == EPI_KIND_RELU || EPI == EPI_KIND_FUSED || EPI == EPI_KIND_LINEAR) {
+        // these kinds are only chosen when the vectors they read exist
         const Epilogue& e = a.epi;
 #pragma unroll
         for (int d = 0; d < 4; ++d) {
@@ -597,6 +619,7 @@ void launch_mfma_instance(hipStream_t s, const MfmaArgs& a, int grid, int lds, i
     switch (epi) {
     case EPI_KIND_RELU: hipLaunchKernelGGL((conv_mfma_kernel<BM, BN, WP, CHECKED, EPI_KIND_RELU>), g, b, lds, s, a); break;
     case EPI_KIND_FUSED: hipLaunchKernelGGL((conv_mfma_kernel<BM, BN, WP, CHECKED, EPI_KIND_FUSED>), g, b, lds, s, a); break;
+    case EPI_KIND_LINEAR: hipLaunchKernelGGL((conv_mfma_kernel<BM, BN, WP, CHECKED, EPI_KIND_LINEAR>), g, b, lds, s, a); break;
     case EPI_KIND_FAST: hipLaunchKernelGGL((conv_mfma_kernel<BM, BN, WP, CHECKED, EPI_KIND_FAST>), g, b, lds, s, a); break;
     default: hipLaunchKernelGGL((conv_mfma_kernel<BM, BN, WP, CHECKED, EPI_KIND_GENERIC>), g, b, lds, s, a); break;
     }
@@ -609,6 +632,7 @@ void launch_stream_instance(hipStream_t s, const MfmaArgs& a, int grid, int epi)
     switch (epi) {
     case EPI_KIND_RELU: hipLaunchKernelGGL((conv_stream_kernel<NT, KS, EPI_KIND_RELU>), g, b, 0, s, a); break;
     case EPI_KIND_FUSED: hipLaunchKernelGGL((conv_stream_kernel<NT, KS, EPI_KIND_FUSED>), g, b, 0, s, a); break;
+    case EPI_KIND_LINEAR: hipLaunchKernelGGL((conv_stream_kernel<NT, KS, EPI_KIND_LINEAR>), g, b, 0, s, a); break;
     case EPI_KIND_FAST: hipLaunchKernelGGL((conv_stream_kernel<NT, KS, EPI_KIND_FAST>), g, b, 0, s, a); break;
     default: hipLaunchKernelGGL((conv_stream_kernel<NT, KS, EPI_KIND_GENERIC>), g, b, 0, s, a); break;
     }

@@ -17,6 +17,10 @@ struct ConvProblem {
 void launch_conv_ref(hipStream_t s, const ConvProblem& p, const Epilogue& epi, const void* in, const void* w,
                      const void* eltw, void* out, int* acc_out);
 void launch_reorder(hipStream_t s, const cldnn_hip_tensor& st, const void* src, const cldnn_hip_tensor& dt, void* dst);
+// dst = act(a [+ b]); quantized: round((a + b) * (calib[f] or oqf)) saturated to char before the activation
+void launch_pointwise(hipStream_t s, const cldnn_hip_tensor& at, const void* a, const cldnn_hip_tensor* bt, const void* b,
+                      const cldnn_hip_tensor& dt, void* dst, int quantized, const float* calib, float oqf, int act, float m,
+                      float n);
 
 // ---- implicit-GEMM int8 MFMA kernel on fs_b_yx_fsv16 (conv_mfma*.hip)
 struct TileConfig {

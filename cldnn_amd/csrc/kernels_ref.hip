@@ -222,6 +222,98 @@ __global__ void __launch_bounds__(256) reorder_kernel(ReorderArgs a, const void*
     }
 }
 
+// ------------------------------------------------------------------------------------------ eltwise / activation
+// Stand-alone forms of what the convolution epilogue fuses (reference
+// kernel_selector/core/cl_kernels/generic_eltwise_ref.cl:311-328 for the sum, activation_ref.cl for the
+// activation).  One work-item per logical element, any layout.
+struct PointwiseArgs {
+    Pitch a, b, dst;
+    int B, F, Y, X;
+    int a_dt, b_dt, dst_dt;
+    int has_b;        // 0: activation only
+    int quantized;    // int sum, then round(sum * factor), saturate to char, then activation
+    const float* calib;
+    float oqf;
+    int act;
+    float m, n;
+};
+
+__global__ void __launch_bounds__(256) pointwise_kernel(PointwiseArgs p, const void* __restrict__ a, const void* __restrict__ b,
+                                                        void* __restrict__ dst)
+{
+    const int64_t total = (int64_t)p.B * p.F * p.Y * p.X;
+    int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= total) return;
+    // destination memory order for the innermost axis keeps the stores coalesced
+    int bi, f, y, x;
+    if (p.dst.fsv > 1 || p.dst.pf == 1) {
+        f = (int)(idx % p.F);
+        int64_t r = idx / p.F;
+        x = (int)(r % p.X);
+        r /= p.X;
+        y = (int)(r % p.Y);
+        bi = (int)(r / p.Y);
+    } else {
+        x = (int)(idx % p.X);
+        int64_t r = idx / p.X;
+        y = (int)(r % p.Y);
+        r /= p.Y;
+        f = (int)(r % p.F);
+        bi = (int)(r / p.F);
+    }
+    const int64_t ai = p.a.at(bi, f, y, x), di = p.dst.at(bi, f, y, x);
+    const bool fp = p.a_dt == CLDNN_HIP_F32;
+    EpiOut o;
+    if (fp) {
+        float v = ((const float*)a)[ai];
+        if (p.has_b) v = v + load_as_float(b, p.b_dt, p.b.at(bi, f, y, x));
+        v = act_f(p.act, p.m, p.n, v);
+        o.f = v;
+        o.i = p.dst_dt == CLDNN_HIP_U8 ? sat_u8(round_half_away(v)) : sat_s8(round_half_away(v));
+    } else {
+        int v = p.a_dt == CLDNN_HIP_U8 ? (int)((const uint8_t*)a)[ai] : (int)((const int8_t*)a)[ai];
+        if (p.has_b) v += (int)load_as_float(b, p.b_dt, p.b.at(bi, f, y, x));
+        if (p.quantized) {
+            const float s = p.calib ? p.calib[f] : p.oqf;
+            v = (int)round_half_away((float)v * s);
+            v = v < -128 ? -128 : (v > 127 ? 127 : v);  // convert_char_sat
+        } else if (p.a_dt == CLDNN_HIP_S8) {
+            v = (int)(signed char)v;  // arithmetic in the unit type wraps
+        } else {
+            v = (int)(unsigned char)v;
+        }
+        v = act_i(p.act, p.m, p.n, v);
+        o.i = v;
+        o.f = (float)v;
+        if (p.dst_dt == CLDNN_HIP_S8) o.i = v < -128 ? -128 : (v > 127 ? 127 : v);
+        else if (p.dst_dt == CLDNN_HIP_U8) o.i = v < 0 ? 0 : (v > 255 ? 255 : v);
+    }
+    store_out(dst, p.dst_dt, di, o);
+}
+
+void launch_pointwise(hipStream_t s, const cldnn_hip_tensor& at, const void* a, const cldnn_hip_tensor* bt, const void* b,
+                      const cldnn_hip_tensor& dt, void* dst, int quantized, const float* calib, float oqf, int act, float m,
+                      float n)
+{
+    CHIP_REQUIRE(at.b == dt.b && at.f == dt.f && at.y == dt.y && at.x == dt.x, CLDNN_HIP_DIMENSION_MISMATCH,
+                 "pointwise: logical sizes differ");
+    PointwiseArgs p{};
+    p.a = make_pitch(at), p.dst = make_pitch(dt);
+    p.B = at.b, p.F = at.f, p.Y = at.y, p.X = at.x;
+    p.a_dt = at.dtype, p.dst_dt = dt.dtype, p.has_b = bt != nullptr;
+    if (bt) {
+        CHIP_REQUIRE(bt->b == at.b && bt->f == at.f && bt->y == at.y && bt->x == at.x, CLDNN_HIP_DIMENSION_MISMATCH,
+                     "eltwise: input sizes differ");
+        p.b = make_pitch(*bt), p.b_dt = bt->dtype;
+    }
+    p.quantized = quantized, p.calib = calib, p.oqf = oqf, p.act = act, p.m = m, p.n = n;
+    const int64_t total = (int64_t)p.B * p.F * p.Y * p.X;
+    const int64_t blocks = (total + 255) / 256;
+    CHIP_REQUIRE(blocks < (1ll << 31), CLDNN_HIP_UNSUPPORTED_SIZE, "tensor too large for the pointwise grid");
+    hipLaunchKernelGGL(pointwise_kernel, dim3((unsigned)blocks), dim3(256), 0, s, p, a, b, dst);
+    CHIP_CHECK(hipGetLastError());
+}
+
 // ------------------------------------------------------------------------------------------ host launchers
 void launch_conv_ref(hipStream_t s, const ConvProblem& p, const Epilogue& epi, const void* in, const void* w,
                      const void* eltw, void* out, int* acc_out)

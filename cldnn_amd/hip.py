@@ -128,6 +128,11 @@ SIGNATURES = {
     "cldnn_hip_tensor_bytes": (C.c_size_t, [C.POINTER(Tensor)]),
     "cldnn_hip_tensor_offset": (C.c_int64, [C.POINTER(Tensor), C.c_int32, C.c_int32, C.c_int32, C.c_int32]),
     "cldnn_hip_reorder": (C.c_int32, [C.c_void_p, C.c_void_p, C.POINTER(Tensor), C.c_void_p, C.POINTER(Tensor)]),
+    "cldnn_hip_activation": (C.c_int32, [C.c_void_p, C.c_void_p, C.POINTER(Tensor), C.c_void_p, C.POINTER(Tensor),
+                                         C.c_int32, C.c_float, C.c_float]),
+    "cldnn_hip_eltwise_sum": (C.c_int32, [C.c_void_p, C.c_void_p, C.POINTER(Tensor), C.c_void_p, C.POINTER(Tensor),
+                                          C.c_void_p, C.POINTER(Tensor), C.c_int32, C.c_void_p, C.c_float, C.c_int32,
+                                          C.c_float, C.c_float]),
     "cldnn_hip_conv_create": (C.c_int32, [C.c_void_p, C.POINTER(ConvDesc), C.c_void_p, C.c_void_p, C.c_void_p,
                                           C.c_void_p, C.c_void_p, C.POINTER(C.c_void_p)]),
     "cldnn_hip_conv_release": (C.c_int32, [C.c_void_p]),

@@ -149,6 +149,21 @@ int64_t cldnn_hip_tensor_offset(const cldnn_hip_tensor* t, int32_t b, int32_t f,
 cldnn_hip_status cldnn_hip_reorder(cldnn_hip_engine e, const void* src_dev, const cldnn_hip_tensor* src,
                                    void* dst_dev, const cldnn_hip_tensor* dst);
 
+enum { CLDNN_HIP_ACT_NONE = 0, CLDNN_HIP_ACT_RELU = 1, CLDNN_HIP_ACT_RELU_SLOPE = 2, CLDNN_HIP_ACT_CLAMP = 3 };
+
+/* stand-alone activation and element-wise sum (what the convolution epilogue fuses when it can);
+ * replace the reference's activation / eltwise kernels for the cases a convolution topology needs
+ * (reference src/gpu/activation_gpu.cpp, src/gpu/eltwise_gpu.cpp,
+ *  kernel_selector/core/cl_kernels/generic_eltwise_ref.cl:311-328).
+ * activation codes: CLDNN_HIP_ACT_*.  quantized != 0: integer sum, round(sum * factor) with the factor
+ * per feature (calib_dev) or per tensor, saturate to int8, then the activation. */
+cldnn_hip_status cldnn_hip_activation(cldnn_hip_engine e, const void* src_dev, const cldnn_hip_tensor* src,
+                                      void* dst_dev, const cldnn_hip_tensor* dst, int32_t activation, float m, float n);
+cldnn_hip_status cldnn_hip_eltwise_sum(cldnn_hip_engine e, const void* a_dev, const cldnn_hip_tensor* a,
+                                       const void* b_dev, const cldnn_hip_tensor* b, void* dst_dev,
+                                       const cldnn_hip_tensor* dst, int32_t quantized, const float* calib_dev,
+                                       float output_quantization_factor, int32_t activation, float m, float n);
+
 /* ------------------------------------------------------------------ convolution
  * One object per convolution / fused_conv_eltwise node; replaces
  * convolution_gpu::create + kernel selection + weight reordering
@@ -157,8 +172,6 @@ cldnn_hip_status cldnn_hip_reorder(cldnn_hip_engine e, const void* src_dev, cons
  * and, at run time, execute_impl (reference src/gpu/primitive_gpu_base.h:117-168).
  * Arithmetic follows the reference semantic kernel
  * (kernel_selector/core/cl_kernels/fused_conv_eltwise_gpu_ref.cl:93-233). */
-enum { CLDNN_HIP_ACT_NONE = 0, CLDNN_HIP_ACT_RELU = 1, CLDNN_HIP_ACT_RELU_SLOPE = 2, CLDNN_HIP_ACT_CLAMP = 3 };
-
 /* which kernel family may be used */
 enum {
     CLDNN_HIP_IMPL_AUTO = 0,      /* tile-config table decides */
