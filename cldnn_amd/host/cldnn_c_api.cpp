@@ -1,0 +1,816 @@
+// The clDNN-compatible C API (include/api/C/cldnn.h) on top of the HIP layer.
+// Counterpart of the reference's src/cldnn.cpp (handle functions, exception -> status translation,
+// thread-local last error), src/engine.cpp, src/memory.cpp, src/network.cpp:40-353 and
+// src/primitive_inst.cpp:42-143 for the primitives of the convolution path.
+#include <cstring>
+#include <functional>
+
+#include "impl.h"
+
+namespace host {
+int hip_dtype(size_t dt);
+int hip_format(int32_t f);
+cldnn_hip_tensor to_hip(const cldnn_layout& l);
+size_t layout_bytes(const cldnn_layout& l);
+cldnn_tensor make_tensor(int b, int f, int x, int y);
+int hip_activation_code(int32_t f);
+void build_program(cldnn_program_impl* prog, cldnn_topology_impl* topo, const std::vector<std::string>& outputs);
+std::string describe_node(const node* n);
+std::string describe_program(const cldnn_program_impl* prog);
+
+static thread_local std::string g_last_error;
+
+// reference src/include/api_impl.h:63-110: exceptions become a status plus a retrievable message
+template <class T, class F>
+T guard(cldnn_status* status, T fallback, F&& f)
+{
+    try {
+        if (status) *status = CLDNN_SUCCESS;
+        return f();
+    } catch (const api_error& e) {
+        g_last_error = e.what();
+        if (status) *status = e.status;
+    } catch (const std::bad_alloc&) {
+        g_last_error = "out of host memory";
+        if (status) *status = CLDNN_OUT_OF_RESOURCES;
+    } catch (const std::exception& e) {
+        g_last_error = e.what();
+        if (status) *status = CLDNN_ERROR;
+    }
+    return fallback;
+}
+template <class F>
+void guard_void(cldnn_status* status, F&& f)
+{
+    guard<int>(status, 0, [&] {
+        f();
+        return 0;
+    });
+}
+
+static size_t copy_names(const std::vector<std::string>& names, char* out, size_t size, size_t* size_ret)
+{
+    // names separated and terminated by '\0', plus one closing '\0' (reference src/cldnn.cpp get_*_names)
+    size_t need = 1;
+    for (auto& n : names) need += n.size() + 1;
+    if (size_ret) *size_ret = need;
+    if (out == nullptr || size < need) throw api_error(CLDNN_INVALID_ARG, "buffer too small");
+    size_t i = 0;
+    for (auto& n : names) {
+        std::memcpy(out + i, n.c_str(), n.size() + 1);
+        i += n.size() + 1;
+    }
+    out[i] = 0;
+    return need;
+}
+
+static std::vector<std::string> ids_of(const cldnn_primitive_id_arr& a)
+{
+    std::vector<std::string> v;
+    for (size_t i = 0; i < a.size; ++i) v.emplace_back(a.data[i] ? a.data[i] : "");
+    return v;
+}
+
+static ref<cldnn_memory_impl> allocate(cldnn_engine_impl* e, const cldnn_layout& l)
+{
+    ref<cldnn_memory_impl> m(new cldnn_memory_impl(), false);
+    m->layout = l;
+    m->engine = ref<cldnn_engine_impl>(e, true);
+    hip_check(cldnn_hip_buffer_alloc(e->h, layout_bytes(l), &m->buf));
+    return m;
+}
+
+static bool same_layout(const cldnn_layout& a, const cldnn_layout& b)
+{
+    if (a.data_type != b.data_type || a.format != b.format) return false;
+    for (int i = 0; i < 4; ++i)
+        if (a.size.sizes[i] != b.size.sizes[i] || a.padding.lower_size.sizes[i] != b.padding.lower_size.sizes[i]
+            || a.padding.upper_size.sizes[i] != b.padding.upper_size.sizes[i])
+            return false;
+    return true;
+}
+
+// memory of another engine / attached host memory is copied into a buffer of this engine
+// (reference src/data.cpp:33-45, src/input_layout.cpp:44-63)
+static ref<cldnn_memory_impl> on_engine(cldnn_engine_impl* e, cldnn_memory_impl* m)
+{
+    if (m->engine.get() == e && m->buf) return ref<cldnn_memory_impl>(m, true);
+    ref<cldnn_memory_impl> c = allocate(e, m->layout);
+    const size_t bytes = layout_bytes(m->layout);
+    if (m->attached) {
+        HOST_REQUIRE(m->attached_bytes >= bytes, CLDNN_INVALID_ARG, "attached memory is smaller than its layout");
+        hip_check(cldnn_hip_buffer_write(c->buf, 0, m->attached, bytes));
+    } else {
+        std::vector<uint8_t> tmp(bytes);
+        hip_check(cldnn_hip_buffer_read(m->buf, 0, tmp.data(), bytes));
+        hip_check(cldnn_hip_buffer_write(c->buf, 0, tmp.data(), bytes));
+    }
+    return c;
+}
+
+static void execute(cldnn_network_impl* net, cldnn_event* deps, size_t ndeps)
+{
+    cldnn_program_impl* prog = net->program.get();
+    cldnn_engine_impl* eng = prog->engine.get();
+    if (ndeps) {
+        std::vector<cldnn_hip_event> hs;
+        for (size_t i = 0; i < ndeps; ++i) {
+            HOST_REQUIRE(deps && deps[i], CLDNN_INVALID_ARG, "null event in the dependency list");
+            hs.push_back(deps[i]->h);
+        }
+        hip_check(cldnn_hip_engine_wait_events(eng->h, hs.data(), hs.size()));
+    }
+    net->executed.clear();
+    net->events.clear();
+    for (auto& u : prog->nodes) {
+        node* n = u.get();
+        prim& p = *n->p;
+        if (n->constant) continue;
+        if (p.type == prim_type::input_layout) {
+            // reference src/primitive_inst.cpp:45 refuses to run with an unset input
+            HOST_REQUIRE(net->input_set[p.id], CLDNN_ERROR, "network input " + p.id + " has not been set");
+            continue;
+        }
+        auto mem_of = [&](node* d) -> cldnn_memory_impl* {
+            auto it = net->mem.find(d);
+            HOST_REQUIRE(it != net->mem.end() && it->second, CLDNN_ERROR, "no memory for primitive " + d->p->id);
+            return it->second.get();
+        };
+        cldnn_memory_impl* out = mem_of(n);
+        cldnn_hip_event pev = nullptr;
+        if (eng->profiling) hip_check(cldnn_hip_event_record_begin(eng->h, &pev));
+        const cldnn_hip_tensor ot = to_hip(n->out);
+        switch (p.type) {
+        case prim_type::reorder: {
+            cldnn_memory_impl* in = mem_of(n->deps[0]);
+            const cldnn_hip_tensor it = to_hip(n->deps[0]->out);
+            hip_check(cldnn_hip_reorder(eng->h, in->device_ptr(), &it, out->device_ptr(), &ot));
+            break;
+        }
+        case prim_type::activation: {
+            cldnn_memory_impl* in = mem_of(n->deps[0]);
+            const cldnn_hip_tensor it = to_hip(n->deps[0]->out);
+            hip_check(cldnn_hip_activation(eng->h, in->device_ptr(), &it, out->device_ptr(), &ot, hip_activation_code(p.act_func),
+                                           p.act_a, p.act_b));
+            break;
+        }
+        case prim_type::eltwise: {
+            HOST_REQUIRE(p.eltw_mode == cldnn_eltwise_sum, CLDNN_INVALID_ARG, "eltwise: only the sum mode is implemented");
+            cldnn_memory_impl* a = mem_of(n->deps[0]);
+            cldnn_memory_impl* b = mem_of(n->deps[1]);
+            const cldnn_hip_tensor at = to_hip(n->deps[0]->out), bt = to_hip(n->deps[1]->out);
+            const float* calib = nullptr;
+            if (!p.eltw_calib.empty()) calib = (const float*)mem_of(n->deps[2])->device_ptr();
+            const bool int_data = n->deps[0]->out.data_type == cldnn_i8 || n->deps[0]->out.data_type == cldnn_u8;
+            const int quantized = int_data && (calib || p.eltw_oqf != 1.0f);
+            int act = CLDNN_HIP_ACT_NONE;
+            if (p.eltw_with_act) act = p.eltw_slope == 0.0f ? CLDNN_HIP_ACT_RELU : CLDNN_HIP_ACT_RELU_SLOPE;
+            hip_check(cldnn_hip_eltwise_sum(eng->h, a->device_ptr(), &at, b->device_ptr(), &bt, out->device_ptr(), &ot, quantized,
+                                            calib, p.eltw_oqf, act, p.eltw_slope, 0.0f));
+            break;
+        }
+        case prim_type::convolution:
+        case prim_type::fused_conv_eltwise: {
+            cldnn_memory_impl* in = mem_of(n->deps[0]);
+            const void* eltw = nullptr;
+            if (p.type == prim_type::fused_conv_eltwise && !p.second_input_in_output) eltw = mem_of(n->deps[1])->device_ptr();
+            hip_check(cldnn_hip_conv_enqueue(n->conv, in->device_ptr(), out->device_ptr(), eltw));
+            break;
+        }
+        default: break;
+        }
+        if (pev) {
+            hip_check(cldnn_hip_event_record_end(pev));
+            ref<cldnn_event_impl> ev(new cldnn_event_impl(), false);
+            ev->engine = ref<cldnn_engine_impl>(eng, true);
+            ev->h = pev;
+            net->events[n] = ev;
+        }
+        net->executed.push_back(p.id);
+    }
+    // one marker for every output that has no event of its own (reference ocl_toolkit.cpp:170-178,197-230)
+    ref<cldnn_event_impl> marker;
+    for (auto& u : prog->nodes) {
+        node* n = u.get();
+        if (!n->is_output || net->events.count(n)) continue;
+        if (!marker) {
+            marker = ref<cldnn_event_impl>(new cldnn_event_impl(), false);
+            marker->engine = ref<cldnn_engine_impl>(eng, true);
+            hip_check(cldnn_hip_event_record(eng->h, &marker->h));
+        }
+        net->events[n] = marker;
+    }
+    hip_check(cldnn_hip_engine_flush(eng->h));
+    net->has_run = true;
+}
+
+}  // namespace host
+
+using namespace host;
+
+cldnn_engine_impl::~cldnn_engine_impl()
+{
+    if (h) cldnn_hip_engine_release(h);
+}
+cldnn_memory_impl::~cldnn_memory_impl()
+{
+    if (buf) cldnn_hip_buffer_release(buf);
+}
+cldnn_event_impl::~cldnn_event_impl()
+{
+    if (h) cldnn_hip_event_release(h);
+}
+cldnn_program_impl::~cldnn_program_impl()
+{
+    for (auto& n : nodes)
+        if (n->conv) cldnn_hip_conv_release(n->conv);
+}
+
+struct cldnn_primitive_type {
+    host::prim_type t;
+    const char* name;
+};
+static const cldnn_primitive_type g_types[] = {
+    {prim_type::input_layout, "input_layout"}, {prim_type::data, "data"},       {prim_type::reorder, "reorder"},
+    {prim_type::activation, "activation"},     {prim_type::eltwise, "eltwise"}, {prim_type::convolution, "convolution"},
+    {prim_type::fused_conv_eltwise, "fused_conv_eltwise"},
+};
+
+extern "C" {
+
+#define TYPE_ID_FN(name, idx)                                                   \
+    cldnn_primitive_type_id cldnn_##name##_type_id(cldnn_status* status)       \
+    {                                                                           \
+        if (status) *status = CLDNN_SUCCESS;                                    \
+        return &g_types[idx];                                                   \
+    }
+TYPE_ID_FN(input_layout, 0)
+TYPE_ID_FN(data, 1)
+TYPE_ID_FN(reorder, 2)
+TYPE_ID_FN(activation, 3)
+TYPE_ID_FN(eltwise, 4)
+TYPE_ID_FN(convolution, 5)
+TYPE_ID_FN(fused_conv_eltwise, 6)
+
+const char* cldnn_get_last_error_message() { return g_last_error.c_str(); }
+
+cldnn_version cldnn_get_version(cldnn_status* status)
+{
+    if (status) *status = CLDNN_SUCCESS;
+    return cldnn_version{1, 4, 25, 0};
+}
+
+// ---------------------------------------------------------------------------------------------- topology
+cldnn_topology cldnn_create_topology(cldnn_status* status)
+{
+    return guard<cldnn_topology>(status, nullptr, [] { return new cldnn_topology_impl(); });
+}
+
+void cldnn_add_primitive(cldnn_topology topology, const struct cldnn_primitive_desc* dto, cldnn_status* status)
+{
+    guard_void(status, [&] {
+        HOST_REQUIRE(topology, CLDNN_INVALID_ARG, "Topology should not be null.");
+        HOST_REQUIRE(dto && dto->id && dto->type, CLDNN_INVALID_ARG, "Invalid primitive descriptor.");
+        auto p = std::make_shared<prim>();
+        p->type = dto->type->t;
+        p->id = dto->id;
+        HOST_REQUIRE(!topology->prims.count(p->id), CLDNN_INVALID_ARG, "Topology already contains primitive with id: " + p->id);
+        p->inputs = ids_of(dto->input);
+        p->output_padding = dto->output_padding;
+        p->out_dt = dto->output_data_type;
+        switch (p->type) {
+        case prim_type::input_layout: p->layout = reinterpret_cast<const cldnn_input_layout_desc*>(dto)->layout; break;
+        case prim_type::data: {
+            cldnn_memory m = reinterpret_cast<const cldnn_data_desc*>(dto)->mem;
+            HOST_REQUIRE(m, CLDNN_INVALID_ARG, "data primitive without memory");
+            p->mem = ref<cldnn_memory_impl>(m, true);
+            break;
+        }
+        case prim_type::reorder: {
+            auto* d = reinterpret_cast<const cldnn_reorder_desc*>(dto);
+            HOST_REQUIRE((!d->mean_subtract || !*d->mean_subtract) && d->subtract_per_feature.size == 0, CLDNN_INVALID_ARG,
+                         "reorder with mean subtraction is not supported by this library");
+            p->reorder_format = d->output_format;
+            break;
+        }
+        case prim_type::activation: {
+            auto* d = reinterpret_cast<const cldnn_activation_desc*>(dto);
+            HOST_REQUIRE(!d->additional_params_input || !*d->additional_params_input, CLDNN_INVALID_ARG,
+                         "activation with a parameter input is not supported by this library");
+            p->act_func = d->activation_func, p->act_a = d->additional_params.a, p->act_b = d->additional_params.b;
+            break;
+        }
+        case prim_type::eltwise: {
+            auto* d = reinterpret_cast<const cldnn_eltwise_desc*>(dto);
+            p->eltw_calib = d->output_calibration_factors ? d->output_calibration_factors : "";
+            p->eltw_oqf = d->output_quantization_factor;
+            p->eltw_mode = d->mode;
+            p->eltw_with_act = d->with_activation != 0;
+            p->eltw_slope = d->activation_negative_slope;
+            for (size_t i = 0; i < d->stride.size; ++i) p->eltw_stride.push_back(d->stride.data[i]);
+            HOST_REQUIRE(d->coefficients.size == 0, CLDNN_INVALID_ARG, "eltwise coefficients are not supported by this library");
+            break;
+        }
+        case prim_type::convolution: {
+            auto* d = reinterpret_cast<const cldnn_convolution_desc*>(dto);
+            p->input_offset = d->input_offset, p->stride = d->stride, p->dilation = d->dilation;
+            p->with_activation = d->with_activation != 0, p->act_slope = d->activation_negative_slope;
+            p->split = d->split, p->groups = d->groups ? d->groups : 1;
+            p->with_output_size = d->with_output_size != 0, p->output_size = d->output_size;
+            p->weights = ids_of(d->weights), p->bias = ids_of(d->bias);
+            p->wqf = ids_of(d->weights_quantization_factors), p->calib = ids_of(d->output_calibration_factors);
+            p->iqf = d->input_quantization_factor, p->oqf = d->output_quantization_factor;
+            p->padding_above = d->padding_above, p->padding_below = d->padding_below;
+            // reference src/convolution.cpp:174-200
+            HOST_REQUIRE(p->weights.size() == p->split, CLDNN_INVALID_ARG, "Weights number does not match the split");
+            HOST_REQUIRE(p->bias.empty() || p->bias.size() == p->weights.size(), CLDNN_INVALID_ARG, "Bias number does not match the weights number");
+            break;
+        }
+        case prim_type::fused_conv_eltwise: {
+            auto* d = reinterpret_cast<const cldnn_fused_conv_eltwise_desc*>(dto);
+            p->input_offset = d->conv.input_offset, p->stride = d->conv.stride, p->dilation = d->conv.dilation;
+            p->with_activation = d->conv.with_activation != 0, p->act_slope = d->conv.activation_negative_slope;
+            p->split = d->conv.split;
+            p->with_output_size = d->conv.with_output_size != 0, p->output_size = d->conv.output_size;
+            p->weights = ids_of(d->conv.weights), p->bias = ids_of(d->conv.bias);
+            p->wqf = ids_of(d->conv.weights_quantization_factors), p->calib = ids_of(d->conv.output_calibration_factors);
+            p->iqf = d->conv.input_quantization_factor, p->oqf = d->conv.output_quantization_factor;
+            p->eltw_calib = d->eltw.output_calibration_factors ? d->eltw.output_calibration_factors : "";
+            p->eltw_oqf = 1.0f;  // the reference leaves this field uninitialised; it is defined as 1 here
+            p->eltw_mode = d->eltw.mode;
+            p->eltw_with_act = d->eltw.with_activation != 0, p->eltw_slope = d->eltw.activation_negative_slope;
+            for (size_t i = 0; i < d->eltw.stride.size; ++i) p->eltw_stride.push_back(d->eltw.stride.data[i]);
+            p->non_conv_scale = d->non_conv_scale;
+            p->second_input_in_output = d->second_input_in_output != 0;
+            p->padding_above = make_tensor(0, 0, 0, 0), p->padding_below = make_tensor(0, 0, 0, 0);
+            HOST_REQUIRE(p->weights.size() == 1 && p->split == 1, CLDNN_INVALID_ARG, "fused_conv_eltwise: split must be 1");
+            break;
+        }
+        }
+        topology->prims[p->id] = p;
+        topology->order.push_back(p->id);
+    });
+}
+
+void cldnn_change_input_layout(cldnn_topology topology, cldnn_primitive_id id, cldnn_layout new_layout, cldnn_status* status)
+{
+    guard_void(status, [&] {
+        HOST_REQUIRE(topology && id, CLDNN_INVALID_ARG, "Topology should not be null.");
+        HOST_REQUIRE(new_layout.format >= cldnn_format_any && new_layout.format < cldnn_format_format_num, CLDNN_INVALID_ARG, "Unknown format of layout.");
+        auto it = topology->prims.find(id);
+        HOST_REQUIRE(it != topology->prims.end() && it->second->type == prim_type::input_layout, CLDNN_INVALID_ARG,
+                     std::string("Primitive ") + id + " is not input layout.");
+        it->second->layout = new_layout;
+    });
+}
+
+void cldnn_get_primitive_ids(cldnn_topology topology, char* ids, size_t size, size_t* size_ret, cldnn_status* status)
+{
+    guard_void(status, [&] {
+        HOST_REQUIRE(topology, CLDNN_INVALID_ARG, "Topology should not be null.");
+        copy_names(topology->order, ids, size, size_ret);
+    });
+}
+
+#define RETAIN_RELEASE(what)                                                                  \
+    void cldnn_retain_##what(cldnn_##what h, cldnn_status* status)                            \
+    {                                                                                         \
+        guard_void(status, [&] {                                                              \
+            HOST_REQUIRE(h, CLDNN_INVALID_ARG, #what " should not be null.");                 \
+            h->retain();                                                                      \
+        });                                                                                   \
+    }                                                                                         \
+    void cldnn_release_##what(cldnn_##what h, cldnn_status* status)                           \
+    {                                                                                         \
+        guard_void(status, [&] {                                                              \
+            HOST_REQUIRE(h, CLDNN_INVALID_ARG, #what " should not be null.");                 \
+            h->release();                                                                     \
+        });                                                                                   \
+    }
+RETAIN_RELEASE(topology)
+RETAIN_RELEASE(engine)
+RETAIN_RELEASE(event)
+RETAIN_RELEASE(program)
+RETAIN_RELEASE(network)
+RETAIN_RELEASE(memory)
+
+// ---------------------------------------------------------------------------------------------- engine
+uint32_t cldnn_get_engine_count(int32_t type, cldnn_status* status)
+{
+    return guard<uint32_t>(status, 0, [&]() -> uint32_t {
+        HOST_REQUIRE(type == cldnn_engine_ocl, CLDNN_DEVICE_ERROR, "Invalid engine type.");
+        return cldnn_hip_device_count();
+    });
+}
+
+void cldnn_release_pending_memory(cldnn_engine engine, cldnn_status* status)
+{
+    guard_void(status, [&] {
+        HOST_REQUIRE(engine, CLDNN_INVALID_ARG, "Engine should not be null.");
+        hip_check(cldnn_hip_engine_finish(engine->h));
+    });
+}
+
+cldnn_engine cldnn_create_engine(int32_t type, uint32_t engine_num, const cldnn_engine_configuration* cfg, cldnn_status* status)
+{
+    return guard<cldnn_engine>(status, nullptr, [&]() -> cldnn_engine {
+        HOST_REQUIRE(type == cldnn_engine_ocl, CLDNN_DEVICE_ERROR, "Invalid engine type.");
+        if (cfg) {
+            HOST_REQUIRE(cfg->context == nullptr, CLDNN_INVALID_ARG, "a user-supplied device context is not supported");
+            HOST_REQUIRE(cfg->priority_mode == cldnn_priority_disabled, CLDNN_INVALID_ARG,
+                         "queue priorities are not supported: the engine's stream runs at the default priority");
+        }
+        ref<cldnn_engine_impl> e(new cldnn_engine_impl(), false);
+        e->profiling = cfg && cfg->enable_profiling;
+        hip_check(cldnn_hip_engine_create(engine_num, e->profiling ? 1 : 0, &e->h));
+        e->retain();
+        return e.get();
+    });
+}
+
+cldnn_engine_info cldnn_get_engine_info(cldnn_engine engine, cldnn_status* status)
+{
+    return guard<cldnn_engine_info>(status, cldnn_engine_info{}, [&] {
+        HOST_REQUIRE(engine, CLDNN_INVALID_ARG, "Engine should not be null.");
+        cldnn_hip_engine_info hi{};
+        hip_check(cldnn_hip_engine_get_info(engine->h, &hi));
+        cldnn_engine_info i{};
+        i.cores_count = hi.cores_count, i.core_frequency = hi.core_frequency;
+        i.max_work_group_size = hi.max_work_group_size, i.max_local_mem_size = hi.max_local_mem_size;
+        i.max_global_mem_size = hi.max_global_mem_size, i.max_alloc_mem_size = hi.max_alloc_mem_size;
+        i.supports_imad = 1, i.supports_immad = 1;
+        return i;
+    });
+}
+
+int32_t cldnn_get_engine_type(cldnn_engine engine, cldnn_status* status)
+{
+    return guard<int32_t>(status, 0, [&] {
+        HOST_REQUIRE(engine, CLDNN_INVALID_ARG, "Engine should not be null.");
+        return (int32_t)cldnn_engine_ocl;
+    });
+}
+
+int64_t cldnn_get_temp_used_device_memory_size(cldnn_engine engine, cldnn_status* status)
+{
+    return guard<int64_t>(status, 0, [&] {
+        HOST_REQUIRE(engine, CLDNN_INVALID_ARG, "Engine should not be null.");
+        return cldnn_hip_engine_used_memory(engine->h);
+    });
+}
+
+int64_t cldnn_get_max_used_device_memory_size(cldnn_engine engine, cldnn_status* status)
+{
+    return guard<int64_t>(status, 0, [&] {
+        HOST_REQUIRE(engine, CLDNN_INVALID_ARG, "Engine should not be null.");
+        return cldnn_hip_engine_max_used_memory(engine->h);
+    });
+}
+
+// ---------------------------------------------------------------------------------------------- events
+cldnn_event cldnn_create_user_event(cldnn_engine engine, cldnn_status* status)
+{
+    return guard<cldnn_event>(status, nullptr, [&]() -> cldnn_event {
+        HOST_REQUIRE(engine, CLDNN_INVALID_ARG, "Engine should not be null.");
+        ref<cldnn_event_impl> ev(new cldnn_event_impl(), false);
+        ev->engine = ref<cldnn_engine_impl>(engine, true);
+        hip_check(cldnn_hip_event_create_user(engine->h, 0, &ev->h));
+        ev->retain();
+        return ev.get();
+    });
+}
+
+int32_t cldnn_is_user_event(cldnn_event event, cldnn_status* status)
+{
+    return guard<int32_t>(status, 0, [&] {
+        HOST_REQUIRE(event, CLDNN_INVALID_ARG, "Event should not be null.");
+        return cldnn_hip_event_is_user(event->h);
+    });
+}
+
+void cldnn_wait_for_event(cldnn_event event, cldnn_status* status)
+{
+    guard_void(status, [&] {
+        HOST_REQUIRE(event, CLDNN_INVALID_ARG, "Event should not be null.");
+        hip_check(cldnn_hip_event_wait(event->h));
+    });
+}
+
+void cldnn_set_event(cldnn_event event, cldnn_status* status)
+{
+    guard_void(status, [&] {
+        HOST_REQUIRE(event, CLDNN_INVALID_ARG, "Event should not be null.");
+        hip_check(cldnn_hip_event_set(event->h));
+    });
+}
+
+void cldnn_add_event_handler(cldnn_event event, cldnn_event_handler handler, void* param, cldnn_status* status)
+{
+    guard_void(status, [&] {
+        HOST_REQUIRE(event && handler, CLDNN_INVALID_ARG, "Event and handler should not be null.");
+        hip_check(cldnn_hip_event_add_handler(event->h, handler, param));
+    });
+}
+
+void cldnn_get_event_profiling_info(cldnn_event event, cldnn_profiling_interval* profiling, size_t size, size_t* size_ret, cldnn_status* status)
+{
+    guard_void(status, [&] {
+        HOST_REQUIRE(event, CLDNN_INVALID_ARG, "Event should not be null.");
+        HOST_REQUIRE(profiling || size == 0, CLDNN_INVALID_ARG, "Profiling should not be null.");
+        // the three intervals of the reference (src/gpu/ocl_base_event.cpp:68-96)
+        if (size_ret) *size_ret = 3;
+        HOST_REQUIRE(size >= 3, CLDNN_INVALID_ARG, "buffer too small");
+        uint64_t ns = 0;
+        hip_check(cldnn_hip_event_elapsed_ns(event->h, &ns));
+        profiling[0] = {"submission", 0};
+        profiling[1] = {"starting", 0};
+        profiling[2] = {"executing", ns};
+    });
+}
+
+// ---------------------------------------------------------------------------------------------- program / network
+static cldnn_program build(cldnn_engine engine, cldnn_topology topology, cldnn_build_option* options, size_t n)
+{
+    HOST_REQUIRE(topology, CLDNN_INVALID_ARG, "Topology should not be null.");
+    ref<cldnn_program_impl> prog(new cldnn_program_impl(), false);
+    if (engine) prog->engine = ref<cldnn_engine_impl>(engine, true);
+    std::vector<std::string> outputs;
+    for (size_t i = 0; i < n; ++i) {
+        switch (options[i].type) {
+        case cldnn_build_option_optimize_data: prog->optimize_data = true; break;
+        case cldnn_build_option_outputs:
+            if (options[i].data) outputs = ids_of(*reinterpret_cast<const cldnn_primitive_id_arr*>(options[i].data));
+            break;
+        default: break;  // fusing, debug, tuning_config, graph_dumps_dir, learning_config: accepted, no effect here
+        }
+    }
+    build_program(prog.get(), topology, outputs);
+    prog->retain();
+    return prog.get();
+}
+
+cldnn_program cldnn_build_program(cldnn_engine engine, cldnn_topology topology, cldnn_build_option* options, size_t options_num, cldnn_status* status)
+{
+    return guard<cldnn_program>(status, nullptr, [&] {
+        HOST_REQUIRE(engine, CLDNN_INVALID_ARG, "Engine should not be null.");
+        return build(engine, topology, options, options_num);
+    });
+}
+
+void cldnn_plan_topology(cldnn_topology topology, cldnn_build_option* options, size_t options_num, char* json, size_t size, size_t* size_ret,
+                         cldnn_status* status)
+{
+    guard_void(status, [&] {
+        cldnn_program p = build(nullptr, topology, options, options_num);
+        const std::string s = describe_program(p);
+        p->release();
+        if (size_ret) *size_ret = s.size() + 1;
+        HOST_REQUIRE(json && size >= s.size() + 1, CLDNN_INVALID_ARG, "buffer too small");
+        std::memcpy(json, s.c_str(), s.size() + 1);
+    });
+}
+
+cldnn_network cldnn_allocate_network(cldnn_program program, cldnn_status* status)
+{
+    return guard<cldnn_network>(status, nullptr, [&]() -> cldnn_network {
+        HOST_REQUIRE(program, CLDNN_INVALID_ARG, "Program should not be null.");
+        ref<cldnn_network_impl> net(new cldnn_network_impl(), false);
+        net->program = ref<cldnn_program_impl>(program, true);
+        cldnn_engine_impl* e = program->engine.get();
+        for (auto& u : program->nodes) {
+            node* n = u.get();
+            if (n->constant) net->mem[n] = on_engine(e, n->p->mem.get());
+            else if (n->p->type == prim_type::input_layout) net->input_set[n->p->id] = false;
+            else if (n->p->type == prim_type::fused_conv_eltwise && n->p->second_input_in_output) net->mem[n] = net->mem[n->deps[1]];
+            else net->mem[n] = allocate(e, n->out);
+        }
+        net->retain();
+        return net.get();
+    });
+}
+
+cldnn_network cldnn_build_network(cldnn_engine engine, cldnn_topology topology, cldnn_build_option* options, size_t options_num, cldnn_status* status)
+{
+    return guard<cldnn_network>(status, nullptr, [&]() -> cldnn_network {
+        HOST_REQUIRE(engine, CLDNN_INVALID_ARG, "Engine should not be null.");
+        cldnn_program p = build(engine, topology, options, options_num);
+        cldnn_status st = CLDNN_SUCCESS;
+        cldnn_network n = cldnn_allocate_network(p, &st);
+        p->release();
+        if (st != CLDNN_SUCCESS) throw api_error(st, g_last_error);
+        return n;
+    });
+}
+
+void cldnn_set_network_input(cldnn_network network, cldnn_primitive_id id, cldnn_memory mem, cldnn_status* status)
+{
+    guard_void(status, [&] {
+        HOST_REQUIRE(network, CLDNN_INVALID_ARG, "Network should not be null.");
+        HOST_REQUIRE(id && mem, CLDNN_INVALID_ARG, "Id and memory should not be null.");
+        cldnn_program_impl* prog = network->program.get();
+        auto it = prog->by_id.find(id);
+        HOST_REQUIRE(it != prog->by_id.end() && it->second->p->type == prim_type::input_layout, CLDNN_INVALID_ARG,
+                     std::string("primitive ") + id + " is not an input");
+        // the previous run must be over before its input is replaced (reference network.cpp:112-113)
+        hip_check(cldnn_hip_engine_finish(prog->engine->h));
+        HOST_REQUIRE(same_layout(mem->layout, it->second->out), CLDNN_INVALID_ARG, "set_network_input: memory layout differs from the input's layout");
+        network->mem[it->second] = on_engine(prog->engine.get(), mem);
+        network->input_set[id] = true;
+    });
+}
+
+void cldnn_get_primitive_info(cldnn_network network, cldnn_primitive_id id, char* info, size_t size, size_t* size_ret, cldnn_status* status)
+{
+    guard_void(status, [&] {
+        HOST_REQUIRE(network && id, CLDNN_INVALID_ARG, "Network should not be null.");
+        auto it = network->program->by_id.find(id);
+        HOST_REQUIRE(it != network->program->by_id.end(), CLDNN_INVALID_ARG, std::string("unknown primitive ") + id);
+        const std::string s = describe_node(it->second);
+        if (size_ret) *size_ret = s.size() + 1;
+        HOST_REQUIRE(info && size >= s.size() + 1, CLDNN_INVALID_ARG, "buffer too small");
+        std::memcpy(info, s.c_str(), s.size() + 1);
+    });
+}
+
+cldnn_engine cldnn_get_network_engine(cldnn_network network, cldnn_status* status)
+{
+    return guard<cldnn_engine>(status, nullptr, [&] {
+        HOST_REQUIRE(network, CLDNN_INVALID_ARG, "Network should not be null.");
+        network->program->engine->retain();
+        return network->program->engine.get();
+    });
+}
+
+cldnn_program cldnn_get_network_program(cldnn_network network, cldnn_status* status)
+{
+    return guard<cldnn_program>(status, nullptr, [&] {
+        HOST_REQUIRE(network, CLDNN_INVALID_ARG, "Network should not be null.");
+        network->program->retain();
+        return network->program.get();
+    });
+}
+
+static std::vector<std::string> names_if(cldnn_network net, const std::function<bool(node*)>& pred)
+{
+    std::vector<std::string> v;
+    for (auto& u : net->program->nodes)
+        if (pred(u.get())) v.push_back(u->p->id);
+    return v;
+}
+
+void cldnn_get_network_output_names(cldnn_network network, char* names, size_t size, size_t* size_ret, cldnn_status* status)
+{
+    guard_void(status, [&] {
+        HOST_REQUIRE(network, CLDNN_INVALID_ARG, "Network should not be null.");
+        copy_names(names_if(network, [](node* n) { return n->is_output; }), names, size, size_ret);
+    });
+}
+
+void cldnn_get_network_executed_primitive_names(cldnn_network network, char* names, size_t size, size_t* size_ret, cldnn_status* status)
+{
+    guard_void(status, [&] {
+        HOST_REQUIRE(network, CLDNN_INVALID_ARG, "Network should not be null.");
+        copy_names(network->executed, names, size, size_ret);
+    });
+}
+
+void cldnn_get_network_all_primitive_names(cldnn_network network, char* names, size_t size, size_t* size_ret, cldnn_status* status)
+{
+    guard_void(status, [&] {
+        HOST_REQUIRE(network, CLDNN_INVALID_ARG, "Network should not be null.");
+        copy_names(names_if(network, [](node*) { return true; }), names, size, size_ret);
+    });
+}
+
+void cldnn_get_network_all_primitive_org_names(cldnn_network network, char* names, size_t size, size_t* size_ret, cldnn_status* status)
+{
+    guard_void(status, [&] {
+        HOST_REQUIRE(network, CLDNN_INVALID_ARG, "Network should not be null.");
+        copy_names(network->program->all_org_ids, names, size, size_ret);
+    });
+}
+
+void cldnn_execute_network(cldnn_network network, cldnn_event* dependencies, size_t deps_num, cldnn_status* status)
+{
+    guard_void(status, [&] {
+        HOST_REQUIRE(network, CLDNN_INVALID_ARG, "Network should not be null.");
+        execute(network, dependencies, deps_num);
+    });
+}
+
+static node* output_node(cldnn_network network, const char* name)
+{
+    HOST_REQUIRE(network && name && *name, CLDNN_INVALID_ARG, "ID of primitive should not be null or empty.");
+    auto it = network->program->by_id.find(name);
+    HOST_REQUIRE(it != network->program->by_id.end() && it->second->is_output, CLDNN_INVALID_ARG,
+                 std::string("primitive ") + name + " is not an output of the network");
+    HOST_REQUIRE(network->has_run, CLDNN_ERROR, "the network has not been executed");
+    return it->second;
+}
+
+cldnn_network_output cldnn_get_network_output(cldnn_network network, const char* name, cldnn_status* status)
+{
+    return guard<cldnn_network_output>(status, cldnn_network_output{nullptr, nullptr}, [&] {
+        node* n = output_node(network, name);
+        cldnn_network_output o{network->events.at(n).get(), network->mem.at(n).get()};
+        o.event->retain();
+        o.memory->retain();
+        return o;
+    });
+}
+
+cldnn_memory cldnn_get_network_output_memory(cldnn_network network, const char* name, cldnn_status* status)
+{
+    return guard<cldnn_memory>(status, nullptr, [&] {
+        node* n = output_node(network, name);
+        cldnn_memory m = network->mem.at(n).get();
+        m->retain();
+        return m;
+    });
+}
+
+cldnn_event cldnn_get_network_output_event(cldnn_network network, const char* name, cldnn_status* status)
+{
+    return guard<cldnn_event>(status, nullptr, [&] {
+        node* n = output_node(network, name);
+        cldnn_event e = network->events.at(n).get();
+        e->retain();
+        return e;
+    });
+}
+
+// ---------------------------------------------------------------------------------------------- memory
+cldnn_memory cldnn_allocate_memory(cldnn_engine engine, cldnn_layout layout, cldnn_status* status)
+{
+    return guard<cldnn_memory>(status, nullptr, [&]() -> cldnn_memory {
+        HOST_REQUIRE(engine, CLDNN_INVALID_ARG, "Engine should not be null.");
+        HOST_REQUIRE(layout.format >= cldnn_format_any && layout.format < cldnn_format_format_num, CLDNN_INVALID_ARG, "Unknown format of layout.");
+        ref<cldnn_memory_impl> m = allocate(engine, layout);
+        m->retain();
+        return m.get();
+    });
+}
+
+cldnn_memory cldnn_attach_memory(cldnn_layout layout, void* pointer, size_t size, cldnn_status* status)
+{
+    return guard<cldnn_memory>(status, nullptr, [&]() -> cldnn_memory {
+        HOST_REQUIRE(pointer, CLDNN_INVALID_ARG, "pointer should not be null");
+        HOST_REQUIRE(size >= layout_bytes(layout), CLDNN_INVALID_ARG, "buffer size does not match layout size");
+        ref<cldnn_memory_impl> m(new cldnn_memory_impl(), false);
+        m->layout = layout;
+        m->attached = pointer;
+        m->attached_bytes = size;
+        m->retain();
+        return m.get();
+    });
+}
+
+int32_t cldnn_is_the_same_buffer(cldnn_memory mem1, cldnn_memory mem2, cldnn_status* status)
+{
+    return guard<int32_t>(status, 0, [&]() -> int32_t {
+        HOST_REQUIRE(mem1 && mem2, CLDNN_INVALID_ARG, "Memory should not be null.");
+        if (mem1 == mem2) return 1;
+        if (mem1->buf && mem2->buf) return cldnn_hip_buffer_device_ptr(mem1->buf) == cldnn_hip_buffer_device_ptr(mem2->buf);
+        if (mem1->attached && mem2->attached) return mem1->attached == mem2->attached;
+        return 0;
+    });
+}
+
+void* cldnn_lock_memory(cldnn_memory memory, cldnn_status* status)
+{
+    return guard<void*>(status, nullptr, [&]() -> void* {
+        HOST_REQUIRE(memory, CLDNN_INVALID_ARG, "Memory should not be null.");
+        if (memory->attached) return memory->attached;
+        void* p = cldnn_hip_buffer_lock(memory->buf);
+        if (!p) throw api_error(CLDNN_DEVICE_ERROR, cldnn_hip_last_error());
+        return p;
+    });
+}
+
+void cldnn_unlock_memory(cldnn_memory memory, cldnn_status* status)
+{
+    guard_void(status, [&] {
+        HOST_REQUIRE(memory, CLDNN_INVALID_ARG, "Memory should not be null.");
+        if (!memory->attached) hip_check(cldnn_hip_buffer_unlock(memory->buf));
+    });
+}
+
+cldnn_layout cldnn_get_memory_layout(cldnn_memory memory, cldnn_status* status)
+{
+    return guard<cldnn_layout>(status, cldnn_layout{}, [&] {
+        HOST_REQUIRE(memory, CLDNN_INVALID_ARG, "Memory should not be null.");
+        return memory->layout;
+    });
+}
+
+cldnn_engine cldnn_get_memory_engine(cldnn_memory memory, cldnn_status* status)
+{
+    return guard<cldnn_engine>(status, nullptr, [&]() -> cldnn_engine {
+        HOST_REQUIRE(memory, CLDNN_INVALID_ARG, "Memory should not be null.");
+        if (!memory->engine) return nullptr;
+        memory->engine->retain();
+        return memory->engine.get();
+    });
+}
+
+}  // extern "C"

@@ -1,0 +1,173 @@
+// Internal objects behind the handles of the clDNN-compatible C API (include/api/C/cldnn.h).
+// Small counterpart of the reference's core runtime (src/include/{engine,memory,event,topology,
+// program,network}_impl.h, refcounted_obj.h) for the one path this library serves.
+#pragma once
+#include <atomic>
+#include <map>
+#include <memory>
+#include <stdexcept>
+#include <string>
+#include <vector>
+
+#include "../../include/api/C/primitives.h"
+#include "../../include/cldnn_hip.h"
+
+namespace host {
+
+struct api_error : std::runtime_error {
+    cldnn_status status;
+    api_error(cldnn_status s, const std::string& m) : std::runtime_error(m), status(s) {}
+};
+#define HOST_REQUIRE(cond, status, msg)                     \
+    do {                                                    \
+        if (!(cond)) throw ::host::api_error((status), (msg)); \
+    } while (0)
+void hip_check(cldnn_hip_status s);  // throws api_error carrying the HIP layer's message
+
+// intrusive reference counting (reference src/include/refcounted_obj.h:33-66)
+struct refcounted {
+    std::atomic<int> refs{1};
+    virtual ~refcounted() {}
+    void retain() { refs.fetch_add(1); }
+    void release()
+    {
+        if (refs.fetch_sub(1) == 1) delete this;
+    }
+};
+template <class T>
+struct ref {  // owning smart pointer for refcounted objects
+    T* p = nullptr;
+    ref() {}
+    explicit ref(T* q, bool add_ref) : p(q)
+    {
+        if (p && add_ref) p->retain();
+    }
+    ref(const ref& o) : p(o.p)
+    {
+        if (p) p->retain();
+    }
+    ref& operator=(const ref& o)
+    {
+        if (o.p) o.p->retain();
+        if (p) p->release();
+        p = o.p;
+        return *this;
+    }
+    ~ref()
+    {
+        if (p) p->release();
+    }
+    T* operator->() const { return p; }
+    T* get() const { return p; }
+    explicit operator bool() const { return p != nullptr; }
+};
+
+enum class prim_type { input_layout, data, reorder, activation, eltwise, convolution, fused_conv_eltwise };
+
+}  // namespace host
+
+struct cldnn_engine_impl : host::refcounted {
+    cldnn_hip_engine h = nullptr;
+    bool profiling = false;
+    ~cldnn_engine_impl() override;
+};
+
+struct cldnn_memory_impl : host::refcounted {
+    cldnn_layout layout{};
+    host::ref<cldnn_engine_impl> engine;  // empty for attached host memory
+    cldnn_hip_buffer buf = nullptr;
+    void* attached = nullptr;
+    size_t attached_bytes = 0;
+    ~cldnn_memory_impl() override;
+    void* device_ptr() const { return buf ? cldnn_hip_buffer_device_ptr(buf) : nullptr; }
+};
+
+struct cldnn_event_impl : host::refcounted {
+    host::ref<cldnn_engine_impl> engine;
+    cldnn_hip_event h = nullptr;
+    ~cldnn_event_impl() override;
+};
+
+namespace host {
+
+// deep copy of a primitive descriptor
+struct prim {
+    prim_type type;
+    std::string id;
+    std::vector<std::string> inputs;
+    cldnn_padding output_padding{};
+    cldnn_optional_data_type out_dt{};
+    // input_layout
+    cldnn_layout layout{};
+    // data
+    ref<cldnn_memory_impl> mem;
+    // reorder
+    int32_t reorder_format = cldnn_format_any;
+    // activation
+    int32_t act_func = activation_none;
+    float act_a = 0.f, act_b = 0.f;
+    // eltwise / fused eltw part
+    std::string eltw_calib;
+    float eltw_oqf = 1.f;
+    int32_t eltw_mode = cldnn_eltwise_sum;
+    bool eltw_with_act = false;
+    float eltw_slope = 0.f;
+    std::vector<cldnn_tensor> eltw_stride;
+    // convolution / fused conv part
+    cldnn_tensor input_offset{}, stride{}, dilation{}, output_size{}, padding_above{}, padding_below{};
+    bool with_activation = false;
+    float act_slope = 0.f;
+    uint32_t split = 1, groups = 1;
+    bool with_output_size = false;
+    std::vector<std::string> weights, bias, wqf, calib;
+    float iqf = 1.f, oqf = 1.f;
+    float non_conv_scale = 1.f;
+    bool second_input_in_output = false;
+};
+
+}  // namespace host
+
+struct cldnn_topology_impl : host::refcounted {
+    std::map<std::string, std::shared_ptr<host::prim>> prims;
+    std::vector<std::string> order;
+};
+
+namespace host {
+
+struct node {
+    std::shared_ptr<prim> p;        // possibly rewritten by the graph passes
+    std::string org_id;             // id in the user's topology ("" for inserted nodes)
+    std::vector<node*> deps;        // data dependencies in primitive order (input, [input2], weights, bias, wqf, calib, [eltw calib])
+    std::vector<node*> users;
+    cldnn_layout out{};             // output layout incl. physical padding
+    int32_t user_format = cldnn_format_any;  // output format before the layout pass (what the topology implies)
+    bool is_output = false;
+    bool constant = false;          // data primitive
+    // activation folded into a convolution (reference prepare_primitive_fusing.cpp:396-433)
+    int32_t fused_act = activation_none;
+    float fused_a = 0.f, fused_b = 0.f;
+    // compiled convolution
+    cldnn_hip_conv conv = nullptr;
+    cldnn_hip_conv_info conv_info{};
+    ref<cldnn_memory_impl> eltw_calib_dev;  // device copy of eltwise calibration (stand-alone eltwise)
+};
+
+}  // namespace host
+
+struct cldnn_program_impl : host::refcounted {
+    host::ref<cldnn_engine_impl> engine;
+    std::vector<std::unique_ptr<host::node>> nodes;  // execution order
+    std::map<std::string, host::node*> by_id;
+    bool optimize_data = false;
+    std::vector<std::string> all_org_ids;
+    ~cldnn_program_impl() override;
+};
+
+struct cldnn_network_impl : host::refcounted {
+    host::ref<cldnn_program_impl> program;
+    std::map<host::node*, host::ref<cldnn_memory_impl>> mem;
+    std::map<host::node*, host::ref<cldnn_event_impl>> events;
+    std::map<std::string, bool> input_set;
+    std::vector<std::string> executed;
+    bool has_run = false;
+};

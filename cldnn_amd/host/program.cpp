@@ -1,0 +1,688 @@
+// Program build: topology -> ordered graph, the three graph passes the convolution path uses
+// (activation fusing, conv+eltwise fusing, layout selection with reorder insertion and border
+// preparation), output-layout calculation and compilation of the convolution objects.
+//
+// Reference counterparts: src/program.cpp:312-451 (pipeline), src/convolution.cpp:32-130 and
+// src/fused_conv_eltwise.cpp:32-122 (output layout + validation), src/include/sliding_window_utils.h:90-129,
+// src/graph_optimizer/prepare_primitive_fusing.cpp:181-337,396-433, src/layout_optimizer.cpp:187-291,
+// src/graph_optimizer/{reorder_inputs,prepare_padding,handle_input_padding,compile_graph}.cpp,
+// src/gpu/convolution_gpu.cpp:71-162, src/gpu/fused_conv_eltwise_gpu.cpp:70-200.
+#include <algorithm>
+#include <cstring>
+#include <functional>
+#include <set>
+
+#include "impl.h"
+
+namespace host {
+
+void hip_check(cldnn_hip_status s)
+{
+    if (s != CLDNN_HIP_SUCCESS) throw api_error((cldnn_status)s, cldnn_hip_last_error());
+}
+
+// ------------------------------------------------------------------------------------------ layouts
+int hip_dtype(size_t dt)
+{
+    switch (dt) {
+    case cldnn_i8: return CLDNN_HIP_S8;
+    case cldnn_u8: return CLDNN_HIP_U8;
+    case cldnn_i32: return CLDNN_HIP_I32;
+    case cldnn_f32: return CLDNN_HIP_F32;
+    default: throw api_error(CLDNN_UNSUPPORTED_FORMAT, "data type not supported by this library (i8, u8, i32, f32 only)");
+    }
+}
+
+int hip_format(int32_t f)
+{
+    switch (f) {
+    case cldnn_format_bfyx: return CLDNN_HIP_FMT_BFYX;
+    case cldnn_format_yxfb: return CLDNN_HIP_FMT_YXFB;
+    case cldnn_format_byxf: return CLDNN_HIP_FMT_BYXF;
+    case cldnn_format_fs_b_yx_fsv16: return CLDNN_HIP_FMT_FS_B_YX_FSV16;
+    case cldnn_format_b_fs_yx_fsv4: return CLDNN_HIP_FMT_B_FS_YX_FSV4;
+    default: throw api_error(CLDNN_UNSUPPORTED_FORMAT, "memory format not supported by this library");
+    }
+}
+
+cldnn_hip_tensor to_hip(const cldnn_layout& l)
+{
+    cldnn_hip_tensor t{};
+    t.dtype = hip_dtype(l.data_type);
+    t.format = hip_format(l.format);
+    t.b = l.size.sizes[0], t.f = l.size.sizes[1], t.x = l.size.sizes[2], t.y = l.size.sizes[3];
+    const int32_t* lo = l.padding.lower_size.sizes;
+    const int32_t* hi = l.padding.upper_size.sizes;
+    t.pad_lo_b = lo[0], t.pad_lo_f = lo[1], t.pad_lo_x = lo[2], t.pad_lo_y = lo[3];
+    t.pad_hi_b = hi[0], t.pad_hi_f = hi[1], t.pad_hi_x = hi[2], t.pad_hi_y = hi[3];
+    return t;
+}
+
+size_t layout_bytes(const cldnn_layout& l)
+{
+    cldnn_hip_tensor t = to_hip(l);
+    size_t b = cldnn_hip_tensor_bytes(&t);
+    HOST_REQUIRE(b > 0, CLDNN_INVALID_ARG, std::string("bad layout: ") + cldnn_hip_last_error());
+    return b;
+}
+
+cldnn_tensor make_tensor(int b, int f, int x, int y)
+{
+    cldnn_tensor t{};
+    t.batch_num = 1, t.feature_num = 1, t.spatial_num = 3, t.local_num = 2;
+    for (int i = 0; i < CLDNN_TENSOR_DIM_MAX; ++i) t.sizes[i] = 1;
+    t.sizes[0] = b, t.sizes[1] = f, t.sizes[2] = x, t.sizes[3] = y;
+    return t;
+}
+
+static cldnn_padding no_padding()
+{
+    cldnn_padding p{};
+    p.lower_size = make_tensor(0, 0, 0, 0);
+    p.upper_size = make_tensor(0, 0, 0, 0);
+    for (int i = 4; i < CLDNN_TENSOR_DIM_MAX; ++i) p.lower_size.sizes[i] = p.upper_size.sizes[i] = 0;
+    return p;
+}
+
+static bool is_int8(size_t dt) { return dt == cldnn_i8 || dt == cldnn_u8; }
+
+// ------------------------------------------------------------------------------------------ constants
+// host copy of a data primitive's memory, element count checked
+static std::vector<uint8_t> read_constant(node* n, size_t expect_elems, const char* what)
+{
+    HOST_REQUIRE(n && n->constant && n->p->mem, CLDNN_INVALID_ARG, std::string(what) + " must be a data primitive");
+    cldnn_memory_impl* m = n->p->mem.get();
+    const cldnn_layout& l = m->layout;
+    size_t elems = (size_t)l.size.sizes[0] * l.size.sizes[1] * l.size.sizes[2] * l.size.sizes[3];
+    HOST_REQUIRE(elems == expect_elems, CLDNN_DIMENSION_MISMATCH,
+                 std::string(what) + ": " + std::to_string(elems) + " elements, expected " + std::to_string(expect_elems));
+    cldnn_hip_tensor t = to_hip(l);
+    HOST_REQUIRE(t.pad_lo_x == 0 && t.pad_lo_y == 0 && t.pad_hi_x == 0 && t.pad_hi_y == 0 && t.pad_lo_f == 0 && t.pad_hi_f == 0,
+                 CLDNN_UNSUPPORTED_FORMAT, std::string(what) + ": padded constants are not supported");
+    size_t bytes = layout_bytes(l);
+    std::vector<uint8_t> out(bytes);
+    if (m->attached) {
+        std::memcpy(out.data(), m->attached, bytes);
+    } else {
+        hip_check(cldnn_hip_buffer_read(m->buf, 0, out.data(), bytes));
+    }
+    return out;
+}
+
+// ------------------------------------------------------------------------------------------ output layouts
+static int spatial(const cldnn_tensor& t, int i) { return t.sizes[2 + i]; }
+
+struct conv_geom {
+    int B, IFM, IH, IW, OFM, FY, FX, sy, sx, dy, dx, py, px, OH, OW, groups;
+};
+
+static conv_geom conv_geometry(const prim& p, const cldnn_layout& in, const cldnn_layout& w)
+{
+    conv_geom g{};
+    g.B = in.size.sizes[0], g.IFM = in.size.sizes[1], g.IW = in.size.sizes[2], g.IH = in.size.sizes[3];
+    g.groups = p.groups ? (int)p.groups : 1;
+    HOST_REQUIRE(p.split == 1, CLDNN_INVALID_ARG, "convolution split > 1 is not supported (use groups)");
+    HOST_REQUIRE(w.format == cldnn_format_bfyx, CLDNN_UNSUPPORTED_FORMAT, "convolution weights must be given in bfyx (o, i, y, x)");
+    g.OFM = w.size.sizes[0];
+    g.FX = w.size.sizes[2], g.FY = w.size.sizes[3];
+    HOST_REQUIRE(w.size.sizes[1] * g.groups == g.IFM, CLDNN_DIMENSION_MISMATCH,
+                 "weights input feature count (x groups) differs from the input's feature count");
+    HOST_REQUIRE(g.OFM % g.groups == 0, CLDNN_DIMENSION_MISMATCH, "output features do not divide into groups");
+    g.sx = spatial(p.stride, 0), g.sy = spatial(p.stride, 1);
+    g.dx = spatial(p.dilation, 0), g.dy = spatial(p.dilation, 1);
+    // reference src/convolution.cpp:54-61
+    HOST_REQUIRE(g.sx > 0 && g.sy > 0, CLDNN_INVALID_ARG, "stride spatial X/Y must be positive");
+    HOST_REQUIRE(g.dx > 0 && g.dy > 0, CLDNN_INVALID_ARG, "dilation spatial X/Y must be positive");
+    HOST_REQUIRE(p.input_offset.sizes[0] == 0 && p.input_offset.sizes[1] == 0, CLDNN_INVALID_ARG,
+                 "input offset in batch / feature is not supported");
+    int ox = spatial(p.input_offset, 0), oy = spatial(p.input_offset, 1);
+    HOST_REQUIRE(ox <= 0 && oy <= 0, CLDNN_INVALID_ARG, "positive input offsets are not supported");
+    // symmetric padding_above / padding_below fold into the offset (reference handle_input_padding.cpp:27-92)
+    int pax = spatial(p.padding_above, 0), pay = spatial(p.padding_above, 1);
+    int pbx = spatial(p.padding_below, 0), pby = spatial(p.padding_below, 1);
+    HOST_REQUIRE(pax == pbx && pay == pby, CLDNN_INVALID_ARG, "asymmetric padding_above / padding_below is not supported");
+    g.px = -ox + pax, g.py = -oy + pay;
+    if (p.with_output_size) {
+        g.OW = spatial(p.output_size, 0), g.OH = spatial(p.output_size, 1);
+        HOST_REQUIRE(g.OW > 0 && g.OH > 0, CLDNN_INVALID_ARG, "user-defined output size must be positive");
+        HOST_REQUIRE(g.OW == cldnn_hip_conv_out_extent(g.IW, g.px, g.FX, g.dx, g.sx)
+                         && g.OH == cldnn_hip_conv_out_extent(g.IH, g.py, g.FY, g.dy, g.sy),
+                     CLDNN_INVALID_ARG, "user-defined output size differs from the computed one");
+    } else {
+        g.OW = cldnn_hip_conv_out_extent(g.IW, g.px, g.FX, g.dx, g.sx);
+        g.OH = cldnn_hip_conv_out_extent(g.IH, g.py, g.FY, g.dy, g.sy);
+    }
+    return g;
+}
+
+static node* dep_named(node* n, const std::string& id)
+{
+    for (node* d : n->deps)
+        if (d->p->id == id) return d;
+    throw api_error(CLDNN_ERROR, "internal: dependency " + id + " of " + n->p->id + " not found");
+}
+
+static void calc_layout(node* n)
+{
+    prim& p = *n->p;
+    cldnn_padding pad = p.output_padding;
+    switch (p.type) {
+    case prim_type::input_layout: n->out = p.layout; return;
+    case prim_type::data: n->out = p.mem->layout; return;
+    case prim_type::reorder: {
+        n->out = n->deps[0]->out;
+        n->out.format = p.reorder_format;
+        if (p.out_dt.enabled) n->out.data_type = p.out_dt.data_type;
+        break;
+    }
+    case prim_type::activation: {
+        n->out = n->deps[0]->out;
+        if (p.out_dt.enabled) n->out.data_type = p.out_dt.data_type;
+        break;
+    }
+    case prim_type::eltwise: {
+        HOST_REQUIRE(n->deps.size() >= 2, CLDNN_INVALID_ARG, "eltwise needs two inputs");
+        const cldnn_layout &a = n->deps[0]->out, &b = n->deps[1]->out;
+        n->out = a;
+        if (!p.eltw_stride.empty()) {
+            // strided inputs: the first input's size divided by its stride (reference src/eltwise.cpp:59-66)
+            HOST_REQUIRE(p.eltw_stride.size() == 2, CLDNN_INVALID_ARG, "eltwise needs one stride per input");
+            for (int i = 2; i < 4; ++i) {
+                HOST_REQUIRE(p.eltw_stride[0].sizes[i] > 0 && p.eltw_stride[1].sizes[i] > 0, CLDNN_INVALID_ARG, "eltwise stride must be positive");
+                n->out.size.sizes[i] = a.size.sizes[i] / p.eltw_stride[0].sizes[i];
+                HOST_REQUIRE(n->out.size.sizes[i] == b.size.sizes[i] / p.eltw_stride[1].sizes[i], CLDNN_DIMENSION_MISMATCH,
+                             "eltwise inputs differ in size after striding");
+            }
+        } else {
+            for (int i = 0; i < 4; ++i)
+                HOST_REQUIRE(a.size.sizes[i] == b.size.sizes[i], CLDNN_DIMENSION_MISMATCH,
+                             "eltwise inputs differ in size (broadcast is not supported)");
+        }
+        if (p.out_dt.enabled) n->out.data_type = p.out_dt.data_type;
+        break;
+    }
+    case prim_type::convolution:
+    case prim_type::fused_conv_eltwise: {
+        const cldnn_layout& in = n->deps[0]->out;
+        node* w = dep_named(n, p.weights.at(0));
+        conv_geom g = conv_geometry(p, in, w->out);
+        n->out = in;  // format follows the input (reference src/convolution.cpp:129)
+        n->out.size = make_tensor(g.B, g.OFM, g.OW, g.OH);
+        if (p.out_dt.enabled) n->out.data_type = p.out_dt.data_type;
+        break;
+    }
+    }
+    n->out.padding = pad;  // explicit output padding of the primitive; the border pass may widen it
+}
+
+// ------------------------------------------------------------------------------------------ graph helpers
+static node* add_node(cldnn_program_impl* prog, std::shared_ptr<prim> p, const std::string& org)
+{
+    auto n = std::unique_ptr<node>(new node());
+    n->p = std::move(p);
+    n->org_id = org;
+    n->constant = n->p->type == prim_type::data;
+    node* raw = n.get();
+    HOST_REQUIRE(!prog->by_id.count(raw->p->id), CLDNN_INVALID_ARG, "duplicate primitive id: " + raw->p->id);
+    prog->by_id[raw->p->id] = raw;
+    prog->nodes.push_back(std::move(n));
+    return raw;
+}
+
+static void replace_dep(node* user, node* from, node* to)
+{
+    for (auto& d : user->deps)
+        if (d == from) d = to;
+    for (auto& s : user->p->inputs)
+        if (s == from->p->id) s = to->p->id;
+    from->users.erase(std::remove(from->users.begin(), from->users.end(), user), from->users.end());
+    to->users.push_back(user);
+}
+
+static void remove_node(cldnn_program_impl* prog, node* n)
+{
+    for (node* d : n->deps) d->users.erase(std::remove(d->users.begin(), d->users.end(), n), d->users.end());
+    prog->by_id.erase(n->p->id);
+    prog->nodes.erase(std::remove_if(prog->nodes.begin(), prog->nodes.end(), [n](const std::unique_ptr<node>& u) { return u.get() == n; }),
+                      prog->nodes.end());
+}
+
+static void sort_nodes(cldnn_program_impl* prog)
+{
+    std::vector<std::unique_ptr<node>> sorted;
+    std::set<node*> done;
+    std::map<node*, std::unique_ptr<node>> owned;
+    std::vector<node*> order;
+    for (auto& u : prog->nodes) order.push_back(u.get());
+    for (auto& u : prog->nodes) owned[u.get()] = std::move(u);
+    std::function<void(node*, int)> visit = [&](node* n, int depth) {
+        if (done.count(n)) return;
+        HOST_REQUIRE(depth < 100000, CLDNN_INVALID_ARG, "topology contains a cycle");
+        done.insert(n);
+        for (node* d : n->deps) visit(d, depth + 1);
+        sorted.push_back(std::move(owned[n]));
+    };
+    for (node* n : order) visit(n, 0);
+    prog->nodes = std::move(sorted);
+}
+
+static size_t position(cldnn_program_impl* prog, node* n)
+{
+    for (size_t i = 0; i < prog->nodes.size(); ++i)
+        if (prog->nodes[i].get() == n) return i;
+    return (size_t)-1;
+}
+
+static std::shared_ptr<prim> make_reorder(const std::string& id, const std::string& input, int32_t format)
+{
+    auto r = std::make_shared<prim>();
+    r->type = prim_type::reorder;
+    r->id = id;
+    r->inputs = {input};
+    r->output_padding = no_padding();
+    r->reorder_format = format;
+    return r;
+}
+
+// ------------------------------------------------------------------------------------------ passes
+// activation -> fused into the producing convolution (reference prepare_primitive_fusing.cpp:396-433)
+static void fuse_activations(cldnn_program_impl* prog)
+{
+    std::vector<node*> acts;
+    for (auto& u : prog->nodes)
+        if (u->p->type == prim_type::activation) acts.push_back(u.get());
+    for (node* a : acts) {
+        node* in = a->deps[0];
+        if (a->is_output || in->is_output || a->deps.size() != 1) continue;
+        if (in->users.size() != 1 || in->fused_act != activation_none) continue;
+        if (in->p->type != prim_type::convolution) continue;
+        const int f = a->p->act_func;
+        if (!(f == activation_relu || f == activation_relu_negative_slope || f == activation_clamp || f == activation_none)) continue;
+        in->fused_act = f, in->fused_a = a->p->act_a, in->fused_b = a->p->act_b;
+        in->p->output_padding = a->p->output_padding;
+        for (node* u : std::vector<node*>(a->users)) replace_dep(u, a, in);
+        remove_node(prog, a);
+    }
+}
+
+// convolution (1x1, stride 1) + eltwise sum with relu -> fused_conv_eltwise (reference :181-337)
+static void fuse_conv_eltwise(cldnn_program_impl* prog)
+{
+    std::vector<node*> convs;
+    for (auto& u : prog->nodes)
+        if (u->p->type == prim_type::convolution) convs.push_back(u.get());
+    for (node* c : convs) {
+        if (c->users.size() != 1 || c->is_output) continue;
+        node* e = c->users[0];
+        if (e->p->type != prim_type::eltwise || e->is_output || e->p->inputs.size() != 2) continue;
+        if (e->p->eltw_mode != cldnn_eltwise_sum || !e->p->eltw_with_act) continue;
+        const cldnn_layout& cl = c->out;
+        const bool ok_type = (is_int8(cl.data_type) && (cl.format == cldnn_format_b_fs_yx_fsv4 || cl.format == cldnn_format_fs_b_yx_fsv16
+                                                        || cl.format == cldnn_format_bfyx || cl.format == cldnn_format_byxf))
+                             || (cl.format == cldnn_format_bfyx && cl.data_type == cldnn_f32);
+        if (!ok_type) continue;
+        node* w = dep_named(c, c->p->weights.at(0));
+        if (w->out.size.sizes[2] != 1 || w->out.size.sizes[3] != 1) continue;
+        if (spatial(c->p->stride, 0) != 1 || spatial(c->p->stride, 1) != 1) continue;
+        if (c->fused_act != activation_none) continue;
+        // the convolution must be the later-executed input of the eltwise
+        node* in0 = e->deps[0];
+        node* in1 = e->deps[1];
+        const int fused_idx = position(prog, in0) < position(prog, in1) ? 1 : 0;
+        if (e->deps[fused_idx] != c) continue;
+        node* other = e->deps[1 - fused_idx];
+
+        auto f = std::make_shared<prim>(*c->p);
+        f->type = prim_type::fused_conv_eltwise;
+        f->id = c->p->id + "_fused_" + e->p->id;
+        f->inputs = {c->p->inputs[0], other->p->id};
+        f->eltw_calib = e->p->eltw_calib;
+        f->eltw_oqf = e->p->eltw_oqf;
+        f->eltw_mode = e->p->eltw_mode;
+        f->eltw_with_act = true;
+        f->eltw_slope = e->p->eltw_slope;
+        f->non_conv_scale = 1.0f;
+        f->output_padding = e->p->output_padding;
+        f->out_dt.data_type = (cldnn_data_type)e->out.data_type;  // the fused primitive produces what the eltwise produced
+        f->out_dt.enabled = 1;
+        if (e->p->eltw_stride.size() == 2) {
+            f->stride.sizes[2] *= e->p->eltw_stride[fused_idx].sizes[2];
+            f->stride.sizes[3] *= e->p->eltw_stride[fused_idx].sizes[3];
+            f->eltw_stride = {e->p->eltw_stride[1 - fused_idx]};
+        } else {
+            f->eltw_stride.clear();
+        }
+        node* nf = add_node(prog, f, e->org_id);
+        nf->user_format = e->user_format;
+        // dependencies: input, input2, weights, bias, wqf, calib, eltw calib
+        nf->deps.push_back(c->deps[0]);
+        nf->deps.push_back(other);
+        for (size_t i = 1; i < c->deps.size(); ++i) nf->deps.push_back(c->deps[i]);
+        for (size_t i = 2; i < e->deps.size(); ++i) nf->deps.push_back(e->deps[i]);
+        for (node* d : nf->deps) d->users.push_back(nf);
+        for (node* u : std::vector<node*>(e->users)) replace_dep(u, e, nf);
+        remove_node(prog, e);
+        remove_node(prog, c);
+    }
+}
+
+static bool quantized(const prim& p)
+{
+    if (p.type == prim_type::fused_conv_eltwise) return !p.wqf.empty();
+    return !p.wqf.empty() || !p.calib.empty() || p.oqf != 1.0f;
+}
+
+// does this convolution run on the int8 matrix-core / depthwise kernels if its tensors are blocked?
+static bool wants_blocked(node* n)
+{
+    const prim& p = *n->p;
+    if (p.type != prim_type::convolution && p.type != prim_type::fused_conv_eltwise) return false;
+    const cldnn_layout& in = n->deps[0]->out;
+    node* w = dep_named(n, p.weights.at(0));
+    if (!is_int8(in.data_type) || w->out.data_type != cldnn_i8) return false;
+    const bool int_mode = quantized(p) || (p.type == prim_type::fused_conv_eltwise);
+    if (!int_mode) return false;
+    const int groups = p.groups ? (int)p.groups : 1;
+    const bool depthwise = groups > 1 && groups == in.size.sizes[1] && groups == w->out.size.sizes[0];
+    return groups == 1 || depthwise;
+}
+
+// The layout rule that stands where the reference has byxf_af32 / fs_bs_yx_bsv4_fsv32 (which its own
+// layout_optimizer never selects, src/layout_optimizer.cpp:245-250): quantized int8 convolutions run in
+// fs_b_yx_fsv16; reorders are inserted where a tensor enters or leaves that format.
+static void select_layouts(cldnn_program_impl* prog)
+{
+    std::map<node*, node*> blocked_copy;  // producer -> its reorder into fs_b_yx_fsv16
+    int counter = 0;
+    auto blocked_version = [&](node* src, node* before) -> node* {
+        if (src->out.format == cldnn_format_fs_b_yx_fsv16) return src;
+        auto it = blocked_copy.find(src);
+        if (it != blocked_copy.end()) return it->second;
+        auto r = make_reorder(src->p->id + "_to_fsv16_" + std::to_string(counter++), src->p->id, cldnn_format_fs_b_yx_fsv16);
+        node* rn = add_node(prog, r, "");
+        rn->deps = {src};
+        src->users.push_back(rn);
+        calc_layout(rn);
+        // keep execution order: place the reorder right before its first consumer
+        auto self = std::move(prog->nodes.back());
+        prog->nodes.pop_back();
+        prog->nodes.insert(prog->nodes.begin() + position(prog, before), std::move(self));
+        blocked_copy[src] = rn;
+        return rn;
+    };
+    for (size_t i = 0; i < prog->nodes.size(); ++i) {
+        node* n = prog->nodes[i].get();
+        if (n->constant) continue;
+        for (node* d : n->deps)
+            if (!d->constant && d->out.format == cldnn_format_any) calc_layout(d);
+        if (wants_blocked(n)) {
+            const int32_t user_format = n->user_format;
+            node* a = blocked_version(n->deps[0], n);
+            if (a != n->deps[0]) replace_dep(n, n->deps[0], a);
+            if (n->p->type == prim_type::fused_conv_eltwise && !n->p->second_input_in_output) {
+                node* b = blocked_version(n->deps[1], n);
+                if (b != n->deps[1]) replace_dep(n, n->deps[1], b);
+            }
+            calc_layout(n);
+            i = position(prog, n);
+            if (n->is_output && user_format != cldnn_format_fs_b_yx_fsv16) {
+                // the user sees the result under the same id in the format the topology implies
+                const std::string id = n->p->id;
+                prog->by_id.erase(id);
+                n->p = std::make_shared<prim>(*n->p);
+                n->p->id = id + "_fsv16";
+                prog->by_id[n->p->id] = n;
+                auto r = make_reorder(id, n->p->id, user_format);
+                node* rn = add_node(prog, r, n->org_id);
+                rn->deps = {n};
+                for (node* u : n->users)  // other consumers keep reading the blocked tensor
+                    for (auto& s : u->p->inputs)
+                        if (s == id) s = n->p->id;
+                n->users.push_back(rn);
+                rn->is_output = true;
+                n->is_output = false;
+                auto self = std::move(prog->nodes.back());
+                prog->nodes.pop_back();
+                prog->nodes.insert(prog->nodes.begin() + i + 1, std::move(self));
+                calc_layout(rn);
+            }
+        } else {
+            calc_layout(n);
+            if (n->is_output && n->out.format == cldnn_format_fs_b_yx_fsv16 && n->p->type != prim_type::reorder) {
+                // an elementwise node that inherited the blocked format from its producer
+                const bool user_blocked = n->user_format == cldnn_format_fs_b_yx_fsv16;
+                if (!user_blocked) {
+                    const std::string id = n->p->id;
+                    prog->by_id.erase(id);
+                    n->p = std::make_shared<prim>(*n->p);
+                    n->p->id = id + "_fsv16";
+                    prog->by_id[n->p->id] = n;
+                    auto r = make_reorder(id, n->p->id, n->user_format);
+                    node* rn = add_node(prog, r, n->org_id);
+                    rn->deps = {n};
+                    n->users.push_back(rn);
+                    rn->is_output = true;
+                    n->is_output = false;
+                    auto self = std::move(prog->nodes.back());
+                    prog->nodes.pop_back();
+                    prog->nodes.insert(prog->nodes.begin() + i + 1, std::move(self));
+                    calc_layout(rn);
+                }
+            }
+        }
+    }
+}
+
+// Give the input of every padded blocked convolution a physical zero border, so the kernels address taps
+// with constant offsets (reference prepare_padding.cpp does the same for its optimised kernels).
+static void prepare_borders(cldnn_program_impl* prog)
+{
+    for (auto& u : prog->nodes) {
+        node* n = u.get();
+        if (!wants_blocked(n) || n->deps[0]->out.format != cldnn_format_fs_b_yx_fsv16) continue;
+        node* w = dep_named(n, n->p->weights.at(0));
+        conv_geom g = conv_geometry(*n->p, n->deps[0]->out, w->out);
+        if (g.px == 0 && g.py == 0 && g.FX == 1 && g.FY == 1) continue;
+        node* src = n->deps[0];
+        if (src->p->type == prim_type::input_layout || src->p->type == prim_type::data) continue;  // user memory: checked kernel
+        const int hi_x = std::max(0, (g.OW - 1) * g.sx - g.px + (g.FX - 1) * g.dx - (g.IW - 1));
+        const int hi_y = std::max(0, (g.OH - 1) * g.sy - g.py + (g.FY - 1) * g.dy - (g.IH - 1));
+        cldnn_padding& pad = src->out.padding;
+        pad.lower_size.sizes[2] = std::max(pad.lower_size.sizes[2], g.px);
+        pad.lower_size.sizes[3] = std::max(pad.lower_size.sizes[3], g.py);
+        pad.upper_size.sizes[2] = std::max(pad.upper_size.sizes[2], hi_x);
+        pad.upper_size.sizes[3] = std::max(pad.upper_size.sizes[3], hi_y);
+    }
+}
+
+// ------------------------------------------------------------------------------------------ compile
+static int hip_act(int32_t f)
+{
+    switch (f) {
+    case activation_none: return CLDNN_HIP_ACT_NONE;
+    case activation_relu: return CLDNN_HIP_ACT_RELU;
+    case activation_relu_negative_slope: return CLDNN_HIP_ACT_RELU_SLOPE;
+    case activation_clamp: return CLDNN_HIP_ACT_CLAMP;
+    default: throw api_error(CLDNN_INVALID_ARG, "activation function not supported by this library (none, relu, relu_negative_slope, clamp)");
+    }
+}
+int hip_activation_code(int32_t f) { return hip_act(f); }
+
+// convolution / fused_conv_eltwise -> one cldnn_hip_conv object (reference convolution_gpu.cpp:71-162)
+static void compile_conv(cldnn_program_impl* prog, node* n)
+{
+    prim& p = *n->p;
+    const bool fused = p.type == prim_type::fused_conv_eltwise;
+    node* in = n->deps[0];
+    node* w = dep_named(n, p.weights.at(0));
+    conv_geom g = conv_geometry(p, in->out, w->out);
+    const int ifm_g = g.IFM / g.groups;
+
+    cldnn_hip_conv_desc d{};
+    d.input = to_hip(in->out);
+    d.output = to_hip(n->out);
+    d.weights_dtype = hip_dtype(w->out.data_type);
+    HOST_REQUIRE(d.weights_dtype == CLDNN_HIP_S8 || d.weights_dtype == CLDNN_HIP_F32, CLDNN_INVALID_ARG, "weights must be i8 or f32");
+    d.ofm = g.OFM, d.ifm = g.IFM, d.fy = g.FY, d.fx = g.FX;
+    d.stride_y = g.sy, d.stride_x = g.sx, d.dilation_y = g.dy, d.dilation_x = g.dx;
+    d.pad_y = g.py, d.pad_x = g.px, d.groups = g.groups;
+    d.input_quantization_factor = p.iqf;
+    d.output_quantization_factor = p.oqf;
+    d.bias_dtype = CLDNN_HIP_NO_TYPE;
+
+    const size_t wcount = (size_t)g.OFM * ifm_g * g.FY * g.FX;
+    std::vector<uint8_t> wv = read_constant(w, wcount, "weights"), bv, qv, cv, ev;
+    if (!p.bias.empty()) {
+        node* b = dep_named(n, p.bias[0]);
+        bv = read_constant(b, g.OFM, "bias");
+        d.bias_dtype = hip_dtype(b->out.data_type);
+        HOST_REQUIRE(d.bias_dtype == CLDNN_HIP_I32 || d.bias_dtype == CLDNN_HIP_F32, CLDNN_INVALID_ARG, "bias must be i32 or f32");
+    }
+    if (!p.wqf.empty()) {
+        node* q = dep_named(n, p.wqf[0]);
+        HOST_REQUIRE(q->out.data_type == cldnn_f32, CLDNN_INVALID_ARG, "weights_quantization_factors must be f32");
+        qv = read_constant(q, g.OFM, "weights_quantization_factors");
+        d.has_wqf = 1;
+    }
+    if (!p.calib.empty()) {
+        // the API requires quantization factors whenever calibration factors are given (reference api/CPP/convolution.hpp:462-463)
+        HOST_REQUIRE(!p.wqf.empty() || fused, CLDNN_INVALID_ARG, "output_calibration_factors need weights_quantization_factors");
+        node* c = dep_named(n, p.calib[0]);
+        HOST_REQUIRE(c->out.data_type == cldnn_f32, CLDNN_INVALID_ARG, "output_calibration_factors must be f32");
+        cv = read_constant(c, g.OFM, "output_calibration_factors");
+        d.has_calib = 1;
+    }
+    // with_activation overrides whatever activation was folded in (reference convolution_gpu.cpp:100-101)
+    if (p.with_activation) {
+        d.activation = p.act_slope == 0.0f ? CLDNN_HIP_ACT_RELU : CLDNN_HIP_ACT_RELU_SLOPE;
+        d.activation_m = p.act_slope;
+    } else {
+        d.activation = hip_act(n->fused_act);
+        d.activation_m = n->fused_a, d.activation_n = n->fused_b;
+    }
+    const void* eltw_calib = nullptr;
+    if (fused) {
+        HOST_REQUIRE(p.eltw_mode == cldnn_eltwise_sum, CLDNN_INVALID_ARG, "fused_conv_eltwise supports the sum mode only");
+        d.fused = 1;
+        d.non_conv_scale = p.non_conv_scale;
+        d.second_input_in_output = p.second_input_in_output ? 1 : 0;
+        if (!p.second_input_in_output) d.eltw = to_hip(n->deps[1]->out);
+        if (p.eltw_with_act) {
+            d.eltw_activation = p.eltw_slope == 0.0f ? CLDNN_HIP_ACT_RELU : CLDNN_HIP_ACT_RELU_SLOPE;
+            d.eltw_activation_m = p.eltw_slope;
+        }
+        d.eltw_stride_x = d.eltw_stride_y = 1;
+        if (!p.eltw_stride.empty()) d.eltw_stride_x = p.eltw_stride[0].sizes[2], d.eltw_stride_y = p.eltw_stride[0].sizes[3];
+        if (!p.eltw_calib.empty()) {
+            node* c = dep_named(n, p.eltw_calib);
+            ev = read_constant(c, g.OFM, "eltwise output_calibration_factors");
+            d.has_eltw_calib = 1;
+            eltw_calib = ev.data();
+        }
+    }
+    d.impl = CLDNN_HIP_IMPL_AUTO;
+    hip_check(cldnn_hip_conv_create(prog->engine->h, &d, wv.data(), bv.empty() ? nullptr : bv.data(),
+                                    qv.empty() ? nullptr : (const float*)qv.data(), cv.empty() ? nullptr : (const float*)cv.data(),
+                                    (const float*)eltw_calib, &n->conv));
+    hip_check(cldnn_hip_conv_get_info(n->conv, &n->conv_info));
+}
+
+// ------------------------------------------------------------------------------------------ build
+void build_program(cldnn_program_impl* prog, cldnn_topology_impl* topo, const std::vector<std::string>& outputs)
+{
+    // nodes + dependencies
+    for (const std::string& id : topo->order) add_node(prog, std::make_shared<prim>(*topo->prims.at(id)), id);
+    prog->all_org_ids = topo->order;
+    auto link = [&](node* n, const std::string& id) {
+        auto it = prog->by_id.find(id);
+        HOST_REQUIRE(it != prog->by_id.end(), CLDNN_INVALID_ARG, "primitive " + n->p->id + " refers to unknown primitive " + id);
+        n->deps.push_back(it->second);
+        it->second->users.push_back(n);
+    };
+    for (auto& u : prog->nodes) {
+        node* n = u.get();
+        prim& p = *n->p;
+        for (auto& s : p.inputs) link(n, s);
+        for (auto* v : {&p.weights, &p.bias, &p.wqf, &p.calib})
+            for (auto& s : *v) link(n, s);
+        if (!p.eltw_calib.empty()) link(n, p.eltw_calib);
+        const size_t need = (p.type == prim_type::input_layout || p.type == prim_type::data) ? 0
+                            : (p.type == prim_type::eltwise || p.type == prim_type::fused_conv_eltwise) ? 2 : 1;
+        HOST_REQUIRE(p.inputs.size() >= need, CLDNN_INVALID_ARG, "primitive " + p.id + " has too few inputs");
+    }
+    // outputs: the build option's list, else every primitive nobody consumes (reference program.cpp mark_outputs)
+    if (!outputs.empty()) {
+        for (auto& id : outputs) {
+            auto it = prog->by_id.find(id);
+            HOST_REQUIRE(it != prog->by_id.end(), CLDNN_INVALID_ARG, "unknown output primitive " + id);
+            it->second->is_output = true;
+        }
+    } else {
+        for (auto& u : prog->nodes)
+            if (u->users.empty() && !u->constant) u->is_output = true;
+    }
+    sort_nodes(prog);
+    for (auto& u : prog->nodes) u->out.format = cldnn_format_any;
+    for (auto& u : prog->nodes) calc_layout(u.get());  // layouts in the user's formats (also validates)
+    for (auto& u : prog->nodes) u->user_format = u->out.format;
+
+    if (prog->optimize_data) {
+        fuse_activations(prog);
+        fuse_conv_eltwise(prog);
+        sort_nodes(prog);
+        for (auto& u : prog->nodes) u->out.format = cldnn_format_any;
+        for (auto& u : prog->nodes)
+            if (u->constant || u->p->type == prim_type::input_layout) calc_layout(u.get());
+        select_layouts(prog);
+    }
+    for (auto& u : prog->nodes) calc_layout(u.get());
+    prepare_borders(prog);
+    for (auto& u : prog->nodes)
+        HOST_REQUIRE(u->p->type != prim_type::eltwise || u->p->eltw_stride.empty(), CLDNN_INVALID_ARG,
+                     "eltwise " + u->p->id + ": strides are only supported when the eltwise is fused into a convolution");
+    if (!prog->engine) return;  // planning only: the graph is inspected, nothing is compiled
+    for (auto& u : prog->nodes) {
+        node* n = u.get();
+        if (n->p->type == prim_type::convolution || n->p->type == prim_type::fused_conv_eltwise) compile_conv(prog, n);
+    }
+}
+
+// ------------------------------------------------------------------------------------------ inspection
+static std::string four(const int32_t* s)
+{
+    return "[" + std::to_string(s[0]) + "," + std::to_string(s[1]) + "," + std::to_string(s[2]) + "," + std::to_string(s[3]) + "]";
+}
+
+// one node as JSON; sizes and paddings are [b, f, x, y] like cldnn_tensor::sizes
+std::string describe_node(const node* n)
+{
+    static const char* tn[] = {"input_layout", "data", "reorder", "activation", "eltwise", "convolution", "fused_conv_eltwise"};
+    const prim& p = *n->p;
+    std::string s = "{\"id\":\"" + p.id + "\",\"type\":\"" + tn[(int)p.type] + "\",\"org_id\":\"" + n->org_id + "\",\"deps\":[";
+    for (size_t i = 0; i < n->deps.size(); ++i) s += std::string(i ? "," : "") + "\"" + n->deps[i]->p->id + "\"";
+    s += "],\"is_output\":" + std::string(n->is_output ? "true" : "false");
+    s += ",\"format\":" + std::to_string(n->out.format) + ",\"data_type\":" + std::to_string(n->out.data_type);
+    s += ",\"size\":" + four(n->out.size.sizes) + ",\"pad_lower\":" + four(n->out.padding.lower_size.sizes) + ",\"pad_upper\":"
+         + four(n->out.padding.upper_size.sizes);
+    if (p.type == prim_type::convolution || p.type == prim_type::fused_conv_eltwise) {
+        s += ",\"stride\":" + four(p.stride.sizes) + ",\"fused_activation\":" + std::to_string(n->fused_act);
+        s += ",\"fused_activation_params\":[" + std::to_string(n->fused_a) + "," + std::to_string(n->fused_b) + "]";
+    }
+    if (p.type == prim_type::fused_conv_eltwise) {
+        s += ",\"eltw_stride\":" + (p.eltw_stride.empty() ? std::string("null") : four(p.eltw_stride[0].sizes));
+        s += ",\"eltw_slope\":" + std::to_string(p.eltw_slope) + ",\"eltw_calib\":\"" + p.eltw_calib + "\"";
+    }
+    if (n->conv)
+        s += std::string(",\"kernel\":\"") + n->conv_info.kernel_name + "\",\"grid\":" + std::to_string(n->conv_info.grid)
+             + ",\"ops\":" + std::to_string(n->conv_info.ops) + ",\"bytes\":" + std::to_string(n->conv_info.bytes);
+    return s + "}";
+}
+
+std::string describe_program(const cldnn_program_impl* prog)
+{
+    std::string s = "[";
+    for (size_t i = 0; i < prog->nodes.size(); ++i) s += (i ? "," : "") + describe_node(prog->nodes[i].get());
+    return s + "]";
+}
+
+}  // namespace host

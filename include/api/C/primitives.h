@@ -1,0 +1,112 @@
+/*
+ * Descriptor structures ("dto") of the primitives a convolution topology needs.  Field order and
+ * meaning follow the reference headers: api/C/input_layout.h, data.h, reorder.h, activation.h,
+ * eltwise.h, convolution.h:36-74 and api_extension/C/fused_conv_eltwise.h:35-97.
+ */
+#ifndef CLDNN_PRIMITIVES_H
+#define CLDNN_PRIMITIVES_H
+#include "cldnn.h"
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+CLDNN_BEGIN_PRIMITIVE_DESC(input_layout)
+cldnn_layout layout;
+CLDNN_END_PRIMITIVE_DESC(input_layout)
+CLDNN_DECLARE_PRIMITIVE_TYPE_ID(input_layout);
+
+CLDNN_BEGIN_PRIMITIVE_DESC(data)
+cldnn_memory mem;
+CLDNN_END_PRIMITIVE_DESC(data)
+CLDNN_DECLARE_PRIMITIVE_TYPE_ID(data);
+
+CLDNN_BEGIN_PRIMITIVE_DESC(reorder)
+cldnn_format_type output_format;
+cldnn_primitive_id mean_subtract;          /* not supported: must be empty */
+cldnn_float_arr subtract_per_feature;      /* not supported: must be empty */
+cldnn_reorder_mean_mode mean_mode;
+CLDNN_END_PRIMITIVE_DESC(reorder)
+CLDNN_DECLARE_PRIMITIVE_TYPE_ID(reorder);
+
+CLDNN_BEGIN_PRIMITIVE_DESC(activation)
+cldnn_activation_func activation_func;
+cldnn_activation_additional_params additional_params;
+cldnn_primitive_id additional_params_input; /* not supported: must be empty */
+CLDNN_END_PRIMITIVE_DESC(activation)
+CLDNN_DECLARE_PRIMITIVE_TYPE_ID(activation);
+
+typedef enum {
+    cldnn_eltwise_sum,
+    cldnn_eltwise_sub,
+    cldnn_eltwise_max,
+    cldnn_eltwise_prod
+} cldnn_eltwise_mode; /* only cldnn_eltwise_sum is implemented */
+
+CLDNN_BEGIN_PRIMITIVE_DESC(eltwise)
+cldnn_primitive_id output_calibration_factors;
+float output_quantization_factor;
+int32_t mode; /* cldnn_eltwise_mode */
+cldnn_float_arr coefficients;
+uint32_t with_activation;
+float activation_negative_slope;
+cldnn_tensor_arr stride;
+CLDNN_END_PRIMITIVE_DESC(eltwise)
+CLDNN_DECLARE_PRIMITIVE_TYPE_ID(eltwise);
+
+CLDNN_BEGIN_PRIMITIVE_DESC(convolution)
+cldnn_tensor input_offset;   /* negative spatial values = zero padding */
+cldnn_tensor stride;
+cldnn_tensor dilation;
+uint32_t with_activation;
+float activation_negative_slope;
+uint32_t split;              /* must be 1 (use groups) */
+uint32_t with_output_size;
+cldnn_tensor output_size;
+cldnn_primitive_id_arr weights;
+cldnn_primitive_id_arr bias;
+cldnn_primitive_id_arr weights_quantization_factors;
+cldnn_primitive_id_arr output_calibration_factors;
+float input_quantization_factor;
+float output_quantization_factor;
+uint32_t groups;
+cldnn_tensor padding_above;  /* symmetric use only */
+cldnn_tensor padding_below;
+CLDNN_END_PRIMITIVE_DESC(convolution)
+CLDNN_DECLARE_PRIMITIVE_TYPE_ID(convolution);
+
+CLDNN_BEGIN_PRIMITIVE_DESC(fused_conv_eltwise)
+struct conv_data {
+    cldnn_tensor input_offset;
+    cldnn_tensor stride;
+    cldnn_tensor dilation;
+    uint32_t with_activation;
+    float activation_negative_slope;
+    uint32_t split;
+    uint32_t with_output_size;
+    cldnn_tensor output_size;
+    cldnn_primitive_id_arr weights;
+    cldnn_primitive_id_arr bias;
+    cldnn_primitive_id_arr weights_quantization_factors;
+    cldnn_primitive_id_arr output_calibration_factors;
+    float input_quantization_factor;
+    float output_quantization_factor;
+} conv;
+struct eltw_data {
+    cldnn_primitive_id output_calibration_factors;
+    float output_quantization_factor;
+    int32_t mode;
+    cldnn_float_arr coefficients;
+    uint32_t with_activation;
+    float activation_negative_slope;
+    cldnn_tensor_arr stride;
+} eltw;
+float non_conv_scale;
+uint8_t second_input_in_output;
+CLDNN_END_PRIMITIVE_DESC(fused_conv_eltwise)
+CLDNN_DECLARE_PRIMITIVE_TYPE_ID(fused_conv_eltwise);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

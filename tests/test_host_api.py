@@ -1,0 +1,371 @@
+"""Host side of the clDNN-compatible API on the CPU: symbol coverage, object handling, error behaviour
+and the graph passes (output layout, dependency order, activation fusing, conv+eltwise fusing, the
+fs_b_yx_fsv16 layout rule, border preparation), observed through the engine-less planning call.
+
+The checks follow what the reference asserts in tests/test_cases/topology_test.cpp,
+tests/test_cases/fused_conv_eltwise_gpu_test.cpp:31-100 (graph shape after fusing) and
+src/convolution.cpp:32-130 (output layout, argument validation).
+"""
+import ctypes as C
+import os
+import re
+
+import numpy as np
+import pytest
+
+from cldnn_amd import api as cl
+from oracle import refconv as rc
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+F = cl.format
+DT = cl.data_types
+
+
+def header_functions():
+    names = []
+    for h in ("include/api/C/cldnn.h", "include/api/C/primitives.h"):
+        src = open(os.path.join(ROOT, h)).read()
+        names += re.findall(r"^CLDNN_API[^;(]*?\b(cldnn_\w+)\s*\(", src, re.M)
+        names += [f"cldnn_{t}_type_id" for t in re.findall(r"^CLDNN_DECLARE_PRIMITIVE_TYPE_ID\((\w+)\);", src, re.M)]
+    return names
+
+
+def test_library_exports_every_declared_function():
+    names = header_functions()
+    assert len(names) > 60
+    l = C.CDLL(cl.LIB_PATH)
+    for n in names:
+        assert hasattr(l, n), n
+
+
+def test_binding_covers_header():
+    assert sorted(header_functions()) == sorted(cl.SIGNATURES)
+
+
+def test_headers_compile_as_c_and_cpp(tmp_path):
+    """The public headers stand alone: C99 and C++14 translation units that include all of them build."""
+    incs = ["api/C/cldnn.h", "api/C/input_layout.h", "api/C/data.h", "api/C/reorder.h", "api/C/activation.h",
+            "api/C/eltwise.h", "api/C/convolution.h", "api_extension/C/fused_conv_eltwise.h"]
+    body = "".join(f'#include "{i}"\n' for i in incs) + "int main(void) { struct cldnn_convolution_desc d; (void)d; return 0; }\n"
+    for name, cc, std in (("a.c", "gcc", "-std=c99"), ("a.cpp", "g++", "-std=c++14")):
+        p = tmp_path / name
+        p.write_text(body)
+        rc_ = os.system(f"{cc} {std} -Wall -Werror -fsyntax-only -I{ROOT}/include {p}")
+        assert rc_ == 0, name
+
+
+def test_version():
+    v = cl._call("cldnn_get_version")
+    assert (v.major, v.minor) == (1, 4)
+
+
+def test_engine_needs_a_gpu_or_works():
+    import torch
+    if torch.cuda.is_available():
+        assert cl.engine.engine_count() >= 1
+    else:
+        assert cl.engine.engine_count() == 0
+        with pytest.raises(cl.error) as e:
+            cl.engine()
+        assert e.value.status == cl.DEVICE_ERROR and "no host fallback" in str(e.value)
+
+
+def test_null_handles_are_invalid_arg():
+    st = C.c_int32(0)
+    cl.lib().cldnn_retain_engine(None, C.byref(st))
+    assert st.value == cl.INVALID_ARG
+    cl.lib().cldnn_execute_network(None, None, 0, C.byref(st))
+    assert st.value == cl.INVALID_ARG
+    assert b"null" in cl.lib().cldnn_get_last_error_message()
+
+
+def attach(arr, shape_bfxy=None, fmt=F.bfyx):
+    a = np.ascontiguousarray(arr)
+    if shape_bfxy is None:
+        b, f, y, x = a.shape
+        shape_bfxy = (b, f, x, y)
+    return cl.memory.attach(cl.layout(cl.DT_OF[a.dtype], fmt, cl.tensor(*shape_bfxy)), a)
+
+
+def vec(n, dtype=np.float32, value=1):
+    return attach(np.full(n, value, dtype), (1, 1, n, 1))
+
+
+def test_attached_memory():
+    a = np.arange(24, dtype=np.int8).reshape(1, 2, 3, 4)
+    m = attach(a)
+    l = m.get_layout()
+    assert (l.data_type, l.format, list(l.size.sizes[:4])) == (DT.i8, F.bfyx, [1, 2, 4, 3])
+    assert m.is_the_same_buffer(m)
+    np.testing.assert_array_equal(m.read(), a)
+    with pytest.raises(cl.error):  # buffer smaller than the layout
+        cl._call("cldnn_attach_memory", cl.layout(DT.i8, F.bfyx, cl.tensor(1, 2, 4, 4)), a.ctypes.data_as(C.c_void_p), a.nbytes)
+
+
+def conv_topology(B=2, IFM=16, H=12, W=10, OFM=8, FY=3, FX=3, in_fmt=F.bfyx, in_dt=DT.i8, quant=True, **kw):
+    w = np.ones((OFM, IFM // kw.get("groups", 1), FY, FX), np.int8)
+    t = cl.topology(cl.input_layout("in", cl.layout(in_dt, in_fmt, cl.tensor(B, IFM, W, H))), cl.data("w", attach(w)),
+                    cl.data("q", vec(OFM)), cl.data("c", vec(OFM)))
+    q = dict(w_quantization_factor=["q"], output_calibration_factors=["c"]) if quant else {}
+    t.add(cl.convolution("conv", "in", ["w"], **q, **kw))
+    return t
+
+
+def by_id(nodes):
+    return {n["id"]: n for n in nodes}
+
+
+# ------------------------------------------------------------------------------------------ topology object
+def test_topology_ids_and_errors():
+    t = conv_topology()
+    assert t.get_primitive_ids() == ["in", "w", "q", "c", "conv"]
+    with pytest.raises(cl.error) as e:
+        t.add(cl.activation("conv", "in", cl.activation_func.relu))
+    assert e.value.status == cl.INVALID_ARG and "already contains" in str(e.value)
+    with pytest.raises(cl.error):
+        t.change_input_layout("conv", cl.layout(DT.i8, F.bfyx, cl.tensor(1, 1, 1, 1)))
+    t.change_input_layout("in", cl.layout(DT.i8, F.bfyx, cl.tensor(1, 16, 20, 20)))
+    assert by_id(cl.plan(t))["conv"]["size"] == [1, 8, 18, 18]
+
+
+def test_unknown_dependency_is_reported():
+    t = cl.topology(cl.input_layout("in", cl.layout(DT.i8, F.bfyx, cl.tensor(1, 16, 4, 4))),
+                    cl.activation("a", "nope", cl.activation_func.relu))
+    with pytest.raises(cl.error) as e:
+        cl.plan(t)
+    assert "unknown primitive nope" in str(e.value)
+
+
+def test_weights_count_must_match_split():
+    x = cl.input_layout("in", cl.layout(DT.i8, F.bfyx, cl.tensor(1, 16, 4, 4)))
+    with pytest.raises(cl.error):
+        cl.topology(x, cl.convolution("conv", "in", ["w"], bias=["b0", "b1"]))
+
+
+# ------------------------------------------------------------------------------------------ output layout
+@pytest.mark.parametrize("H,W,FY,FX,sy,sx,py,px,dy,dx", [
+    (12, 10, 3, 3, 1, 1, 0, 0, 1, 1), (12, 10, 3, 3, 1, 1, 1, 1, 1, 1), (224, 224, 7, 7, 2, 2, 3, 3, 1, 1),
+    (56, 56, 1, 1, 2, 2, 0, 0, 1, 1), (9, 11, 5, 3, 2, 1, 2, 1, 1, 1), (15, 15, 3, 3, 1, 1, 2, 2, 2, 2),
+    (7, 9, 3, 3, 3, 2, 0, 1, 1, 1)])
+def test_conv_output_layout(H, W, FY, FX, sy, sx, py, px, dy, dx):
+    t = conv_topology(H=H, W=W, FY=FY, FX=FX, stride=cl.tensor(1, 1, sx, sy), input_offset=cl.tensor(0, 0, -px, -py, 0),
+                      dilation=cl.tensor(1, 1, dx, dy))
+    n = by_id(cl.plan(t))["conv"]
+    # format and data type follow the input, the feature count the weights (reference src/convolution.cpp:113-129)
+    assert n["format"] == F.bfyx and n["data_type"] == DT.i8
+    assert n["size"] == [2, 8, rc.out_extent(W, px, FX, dx, sx), rc.out_extent(H, py, FY, dy, sy)]
+    # closed form for the cases without a partial last window
+    if (W + 2 * px - ((FX - 1) * dx + 1)) % sx == 0:
+        assert n["size"][2] == (W + 2 * px - ((FX - 1) * dx + 1)) // sx + 1
+
+
+def test_conv_output_type_override_and_padding():
+    t = conv_topology(output_data_type=DT.u8, output_padding=cl.padding((0, 0, 2, 1)))
+    n = by_id(cl.plan(t))["conv"]
+    assert n["data_type"] == DT.u8
+    assert n["pad_lower"] == [0, 0, 1, 2] and n["pad_upper"] == [0, 0, 1, 2]
+
+
+def test_user_output_size_must_agree():
+    ok = conv_topology(output_size=cl.tensor(2, 8, 8, 10))
+    assert by_id(cl.plan(ok))["conv"]["size"] == [2, 8, 8, 10]
+    with pytest.raises(cl.error):
+        cl.plan(conv_topology(output_size=cl.tensor(2, 8, 9, 10)))
+
+
+@pytest.mark.parametrize("kw,msg", [
+    (dict(stride=cl.tensor(1, 1, 0, 1)), "stride"),
+    (dict(dilation=cl.tensor(1, 1, 1, 0)), "dilation"),
+    (dict(input_offset=cl.tensor(0, 1, 0, 0, 0)), "input offset"),
+    (dict(groups=3), "feature count"),
+    (dict(padding_above=cl.tensor(0, 0, 1, 1, 0)), "asymmetric"),
+])
+def test_conv_argument_validation(kw, msg):
+    with pytest.raises(cl.error) as e:
+        cl.plan(conv_topology(**kw))
+    assert msg in str(e.value)
+
+
+def test_weights_feature_mismatch():
+    t = cl.topology(cl.input_layout("in", cl.layout(DT.i8, F.bfyx, cl.tensor(1, 16, 4, 4))),
+                    cl.data("w", attach(np.ones((8, 12, 1, 1), np.int8))), cl.convolution("conv", "in", ["w"]))
+    with pytest.raises(cl.error) as e:
+        cl.plan(t)
+    assert e.value.status == cl.DIMENSION_MISMATCH
+
+
+# ------------------------------------------------------------------------------------------ dependency order
+def test_dependency_order_of_convolution():
+    """input, weights, bias, quantization factors, calibration factors (reference src/gpu/convolution_gpu.cpp:37-69)."""
+    t = cl.topology(cl.input_layout("in", cl.layout(DT.i8, F.bfyx, cl.tensor(1, 16, 4, 4))),
+                    cl.data("calib", vec(8)), cl.data("bias", vec(8, np.int32)), cl.data("wq", vec(8)),
+                    cl.data("weights", attach(np.ones((8, 16, 1, 1), np.int8))),
+                    cl.convolution("conv", "in", ["weights"], ["bias"], ["wq"], ["calib"]))
+    nodes = cl.plan(t)
+    assert by_id(nodes)["conv"]["deps"] == ["in", "weights", "bias", "wq", "calib"]
+    order = [n["id"] for n in nodes]
+    assert all(order.index(d) < order.index("conv") for d in by_id(nodes)["conv"]["deps"])
+    assert [n["id"] for n in nodes if n["is_output"]] == ["conv"]
+
+
+def test_outputs_option():
+    t = conv_topology()
+    t.add(cl.activation("relu", "conv", cl.activation_func.relu))
+    assert [n["id"] for n in cl.plan(t) if n["is_output"]] == ["relu"]
+    assert [n["id"] for n in cl.plan(t, cl.build_options(outputs=["conv", "relu"])) if n["is_output"]] == ["conv", "relu"]
+    with pytest.raises(cl.error):
+        cl.plan(t, cl.build_options(outputs=["nope"]))
+
+
+# ------------------------------------------------------------------------------------------ fusing passes
+def two_convs(second_fy=3, act=cl.activation_func.relu, params=(0.0, 0.0)):
+    t = conv_topology(input_offset=cl.tensor(0, 0, -1, -1, 0))
+    t.add(cl.activation("relu", "conv", act, params),
+          cl.data("w2", attach(np.ones((8, 8, second_fy, second_fy), np.int8))),
+          cl.convolution("conv2", "relu", ["w2"], w_quantization_factor=["q"], output_calibration_factors=["c"],
+                         input_offset=cl.tensor(0, 0, -(second_fy // 2), -(second_fy // 2), 0)))
+    return t
+
+
+def test_activation_is_folded_into_convolution():
+    plain = by_id(cl.plan(two_convs()))
+    assert "relu" in plain and plain["conv"]["fused_activation"] == cl.activation_func.none
+    opt = by_id(cl.plan(two_convs(), cl.build_options(optimize_data=True)))
+    assert "relu" not in opt
+    assert opt["conv"]["fused_activation"] == cl.activation_func.relu
+    assert opt["conv2_fsv16"]["deps"][0] == "conv"
+
+
+def test_clamp_parameters_survive_folding():
+    opt = by_id(cl.plan(two_convs(act=cl.activation_func.clamp, params=(-3.0, 5.0)), cl.build_options(optimize_data=True)))
+    assert opt["conv"]["fused_activation"] == cl.activation_func.clamp
+    assert opt["conv"]["fused_activation_params"] == [-3.0, 5.0]
+
+
+def test_activation_with_two_consumers_of_the_conv_is_kept():
+    t = two_convs()
+    t.add(cl.activation("other", "conv", cl.activation_func.relu))
+    opt = by_id(cl.plan(t, cl.build_options(optimize_data=True)))
+    assert "relu" in opt and opt["conv"]["fused_activation"] == cl.activation_func.none
+
+
+def test_unsupported_activation_is_not_folded():
+    opt = by_id(cl.plan(two_convs(act=cl.activation_func.logistic), cl.build_options(optimize_data=True)))
+    assert "relu" in opt and opt["conv"]["fused_activation"] == cl.activation_func.none
+
+
+def residual_block(fy=1, stride=1, with_activation=True, eltw_strides=None, in_fmt=F.bfyx):
+    """conv(3x3) -> [conv 1x1 | 3x3] + shortcut -> eltwise sum (+relu): the tail of a ResNet block."""
+    B, Cn, H, W = 2, 16, 8, 8
+    w1 = attach(np.ones((Cn, Cn, 3, 3), np.int8))
+    w2 = attach(np.ones((Cn, Cn, fy, fy), np.int8))
+    t = cl.topology(cl.input_layout("in", cl.layout(DT.i8, in_fmt, cl.tensor(B, Cn, W, H))),
+                    cl.data("w1", w1), cl.data("w2", w2), cl.data("q", vec(Cn)), cl.data("c", vec(Cn)),
+                    cl.convolution("conv1", "in", ["w1"], w_quantization_factor=["q"], output_calibration_factors=["c"],
+                                   input_offset=cl.tensor(0, 0, -1, -1, 0), with_activation=True),
+                    cl.convolution("conv2", "conv1", ["w2"], w_quantization_factor=["q"], output_calibration_factors=["c"],
+                                   input_offset=cl.tensor(0, 0, -(fy // 2), -(fy // 2), 0), stride=cl.tensor(1, 1, stride, stride)),
+                    cl.eltwise("sum", "in", "conv2", cl.eltwise_mode.sum, with_activation, 0.0, output_calibration_factors="c",
+                               stride=eltw_strides),
+                    cl.activation("out", "sum", cl.activation_func.none))
+    return t
+
+
+def test_conv_eltwise_fusing():
+    opt = cl.plan(residual_block(), cl.build_options(optimize_data=True))
+    ids = [n["id"] for n in opt]
+    assert "conv2" not in ids and "sum" not in ids
+    f = by_id(opt)["conv2_fused_sum"]
+    assert f["type"] == "fused_conv_eltwise"
+    # input, second input, then the convolution's constants, then the eltwise calibration
+    assert f["deps"][2:] == ["w2", "q", "c", "c"]
+    assert f["eltw_calib"] == "c"
+    # both data inputs were moved into the blocked layout
+    assert f["deps"][0] == "conv1" and f["deps"][1].startswith("in_to_fsv16")
+    assert f["format"] == F.fs_b_yx_fsv16
+
+
+@pytest.mark.parametrize("kw", [dict(fy=3), dict(with_activation=False)], ids=["3x3", "no_activation"])
+def test_conv_eltwise_not_fused(kw):
+    ids = [n["id"] for n in cl.plan(residual_block(**kw), cl.build_options(optimize_data=True))]
+    assert "conv2" in ids and "sum" in ids
+
+
+def test_conv_eltwise_fusing_moves_eltwise_stride_into_the_conv():
+    """A strided eltwise after a 1x1 convolution: the convolution takes the stride, the shortcut keeps its own
+    (reference src/graph_optimizer/prepare_primitive_fusing.cpp:300-318)."""
+    B, Cn, H, W = 1, 16, 8, 8
+    t = cl.topology(cl.input_layout("in", cl.layout(DT.i8, F.bfyx, cl.tensor(B, Cn, W, H))),
+                    cl.input_layout("short", cl.layout(DT.i8, F.bfyx, cl.tensor(B, Cn, W, H))),
+                    cl.data("w", attach(np.ones((Cn, Cn, 1, 1), np.int8))), cl.data("q", vec(Cn)),
+                    cl.convolution("conv", "in", ["w"], w_quantization_factor=["q"], output_calibration_factors=["q"]))
+    # both inputs subsampled by 2 -> output 4x4
+    t.add(cl.eltwise("sum", "short", "conv", cl.eltwise_mode.sum, True, 0.0, stride=[cl.tensor(1, 1, 2, 2), cl.tensor(1, 1, 2, 2)]))
+    t.add(cl.activation("out", "sum", cl.activation_func.none))
+    nodes = cl.plan(t, cl.build_options(optimize_data=True))
+    f = by_id(nodes)["conv_fused_sum"]
+    assert f["stride"][2:] == [2, 2] and f["eltw_stride"][2:] == [2, 2]
+    assert f["size"] == [1, 16, 4, 4]
+    with pytest.raises(cl.error) as e:  # left unfused, a strided eltwise is refused: only the fused form is served
+        cl.plan(t)
+    assert "fused into a convolution" in str(e.value)
+
+
+# ------------------------------------------------------------------------------------------ layout rule
+def test_layout_rule_blocks_quantized_int8_convolutions():
+    plain = by_id(cl.plan(conv_topology()))
+    assert plain["conv"]["format"] == F.bfyx and not any("fsv16" in k for k in plain)
+    opt = cl.plan(conv_topology(), cl.build_options(optimize_data=True))
+    ids = [n["id"] for n in opt]
+    # reorder in, convolution under an internal id, reorder back under the user's id
+    assert ids[-3:] == ["in_to_fsv16_0", "conv_fsv16", "conv"]
+    o = by_id(opt)
+    assert o["in_to_fsv16_0"]["format"] == F.fs_b_yx_fsv16 and o["conv_fsv16"]["format"] == F.fs_b_yx_fsv16
+    assert o["conv"]["type"] == "reorder" and o["conv"]["format"] == F.bfyx and o["conv"]["is_output"]
+    assert not o["conv_fsv16"]["is_output"] and o["conv"]["org_id"] == "conv"
+
+
+def test_layout_rule_keeps_user_blocked_tensors():
+    opt = cl.plan(conv_topology(in_fmt=F.fs_b_yx_fsv16), cl.build_options(optimize_data=True))
+    assert [n["id"] for n in opt][-1] == "conv" and by_id(opt)["conv"]["type"] == "convolution"
+    assert by_id(opt)["conv"]["format"] == F.fs_b_yx_fsv16
+
+
+@pytest.mark.parametrize("kw", [dict(quant=False), dict(in_dt=DT.f32), dict(IFM=16, OFM=8, groups=2)])
+def test_layout_rule_leaves_other_convolutions_alone(kw):
+    if kw.get("in_dt") == DT.f32:
+        kw = dict(kw, quant=False)
+    opt = cl.plan(conv_topology(**kw), cl.build_options(optimize_data=True))
+    assert not any("fsv16" in n["id"] for n in opt)
+    assert by_id(opt)["conv"]["format"] == F.bfyx
+
+
+def test_layout_rule_takes_depthwise():
+    opt = cl.plan(conv_topology(IFM=16, OFM=16, groups=16), cl.build_options(optimize_data=True))
+    assert by_id(opt)["conv_fsv16"]["format"] == F.fs_b_yx_fsv16
+
+
+def test_one_reorder_serves_all_blocked_consumers():
+    opt = cl.plan(residual_block(), cl.build_options(optimize_data=True))
+    assert sum(n["id"].startswith("in_to_fsv16") for n in opt) == 1
+    o = by_id(opt)
+    assert o["conv1"]["deps"][0] == o["conv2_fused_sum"]["deps"][1]
+
+
+def test_border_preparation():
+    """The producer of a padded blocked convolution's input carries the zero border physically
+    (reference src/graph_optimizer/prepare_padding.cpp:26-124)."""
+    o = by_id(cl.plan(two_convs(), cl.build_options(optimize_data=True)))
+    assert o["in_to_fsv16_0"]["pad_lower"] == [0, 0, 1, 1] and o["in_to_fsv16_0"]["pad_upper"] == [0, 0, 1, 1]
+    assert o["conv"]["pad_lower"] == [0, 0, 1, 1]          # conv2 is 3x3 with offset -1
+    o = by_id(cl.plan(two_convs(second_fy=1), cl.build_options(optimize_data=True)))
+    assert o["conv"]["pad_lower"] == [0, 0, 0, 0]          # a 1x1 consumer needs no border
+
+
+def test_border_for_strided_window_covers_the_last_tap():
+    t = conv_topology(H=9, W=9, FY=3, FX=3, stride=cl.tensor(1, 1, 2, 2), input_offset=cl.tensor(0, 0, -1, -1, 0))
+    o = by_id(cl.plan(t, cl.build_options(optimize_data=True)))
+    r = o["in_to_fsv16_0"]
+    OW = o["conv_fsv16"]["size"][2]
+    last = (OW - 1) * 2 - 1 + 2  # leftmost tap of the last window + filter reach
+    assert r["pad_lower"][2] == 1 and r["pad_upper"][2] == max(0, last - 8)

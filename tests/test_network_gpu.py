@@ -1,0 +1,326 @@
+"""The convolution path through the clDNN-compatible API on the GPU: topology -> network -> execute,
+checked against the reference's known-answer tables and the CPU oracle.
+
+The tests are shaped like the reference's (tests/test_cases/convolution_gpu_test.cpp:4006-4200,
+tests/test_cases/fused_conv_eltwise_gpu_test.cpp:31-236, tests/test_cases/memory_test.cpp,
+tests/test_cases/topology_test.cpp): build a topology from input_layout / data / convolution primitives,
+run a network, read the output memory.
+"""
+import numpy as np
+import pytest
+
+import kat
+from cldnn_amd import api as cl
+from oracle import refconv as rc
+
+pytestmark = pytest.mark.gpu
+K = kat.load()
+F = cl.format
+DT = cl.data_types
+CL_DT = {"s8": DT.i8, "u8": DT.u8, "f32": DT.f32, "i32": DT.i32}
+OPT = [False, True]
+
+
+@pytest.fixture(scope="module")
+def eng():
+    return cl.engine()
+
+
+def vec_mem(eng, values):
+    a = np.ascontiguousarray(values).reshape(1, 1, 1, -1)
+    return cl.make_memory(eng, a)
+
+
+def run(eng, topo, inputs, optimize):
+    net = cl.network(eng, topo, cl.build_options(optimize_data=optimize))
+    for k, v in inputs.items():
+        net.set_input_data(k, v)
+    return net, net.execute()
+
+
+def check(out, expected, out_dt, tol=0.0):
+    if out_dt == "f32":
+        np.testing.assert_allclose(out, expected, atol=max(tol, 1e-5), rtol=1e-5)
+    else:
+        np.testing.assert_array_equal(out.astype(np.int64), np.asarray(expected).astype(np.int64))
+
+
+# ------------------------------------------------------------------------------------------ known answers
+@pytest.mark.parametrize("optimize", OPT, ids=["plain", "optimize_data"])
+@pytest.mark.parametrize("case", K["conv_quantized"], ids=lambda c: c["name"])
+def test_kat_conv_quantized(eng, case, optimize):
+    p = kat.diag_problem(case)
+    topo = cl.topology(
+        cl.input_layout("input", cl.layout(CL_DT[case["in_dt"]], F.bfyx, cl.tensor(1, len(case["features"]), 4, 1))),
+        cl.data("weights", cl.make_memory(eng, p["w"])), cl.data("biases", vec_mem(eng, p["bias"])),
+        cl.data("quantizations", vec_mem(eng, p["wqf"])),
+        cl.convolution("conv", "input", ["weights"], ["biases"], ["quantizations"], with_activation=True,
+                       output_data_type=CL_DT[case["out_dt"]]))
+    net, outs = run(eng, topo, {"input": cl.make_memory(eng, p["x"])}, optimize)
+    assert list(outs) == ["conv"]
+    check(outs["conv"].get_memory().read(), p["expected"], case["out_dt"], case.get("tol", 0.0))
+
+
+@pytest.mark.parametrize("optimize", OPT, ids=["plain", "optimize_data"])
+@pytest.mark.parametrize("case", K["fused"], ids=lambda c: c["name"])
+def test_kat_fused_conv_eltwise(eng, case, optimize):
+    p = kat.diag_problem(case, fused=True)
+    n = len(case["features"])
+    topo = cl.topology(
+        cl.input_layout("input", cl.layout(CL_DT[case["in_dt"]], F.bfyx, cl.tensor(1, n, 4, 1))),
+        cl.input_layout("non_conv_input", cl.layout(CL_DT[case["in_dt"]], F.bfyx, cl.tensor(1, n, 2, 1))),
+        cl.data("weights", cl.make_memory(eng, p["w"])), cl.data("biases", vec_mem(eng, p["bias"])),
+        cl.data("wqf", vec_mem(eng, p["wqf"])), cl.data("conv_calib", vec_mem(eng, p["conv_calib"])),
+        cl.data("eltw_calib", vec_mem(eng, p["eltw_calib"])),
+        cl.fused_conv_eltwise("fused_conv", "input", "non_conv_input", cl.eltwise_mode.sum, ["weights"], ["biases"],
+                              ["wqf"] if case["pass_wqf"] else None, ["conv_calib"] if case["pass_conv_calib"] else None, 1.0,
+                              float(p["non_conv_scale"]), "eltw_calib" if case["pass_eltw_calib"] else "",
+                              eltw_with_activation=True,
+                              output_data_type=CL_DT[case["out_dt"]] if case.get("out_dt_explicit", True) else None))
+    net, outs = run(eng, topo, {"input": cl.make_memory(eng, p["x"]), "non_conv_input": cl.make_memory(eng, p["nci"])}, optimize)
+    check(outs["fused_conv"].get_memory().read(), p["expected"], case["out_dt"], case.get("tol", 0.0))
+
+
+@pytest.mark.parametrize("case", K["indexing"], ids=lambda c: c["name"])
+def test_kat_indexing(eng, case):
+    p = kat.indexing_problem(case, K["indexing"])
+    b, f, h, w = p["x"].shape
+    prims = [cl.input_layout("input", cl.layout(cl.DT_OF[p["x"].dtype], F.bfyx, cl.tensor(b, f, w, h))),
+             cl.data("weights", cl.make_memory(eng, p["w"]))]
+    if p["bias"] is not None:
+        prims.append(cl.data("biases", vec_mem(eng, p["bias"])))
+    prims.append(cl.convolution("conv", "input", ["weights"], ["biases"] if p["bias"] is not None else None,
+                                stride=cl.tensor(1, 1, p["stride"][1], p["stride"][0]),
+                                input_offset=cl.tensor(0, 0, -p["pad"][1], -p["pad"][0], 0), groups=p["groups"],
+                                with_activation=p["act"] == "relu"))
+    net, outs = run(eng, cl.topology(*prims), {"input": cl.make_memory(eng, p["x"])}, False)
+    out = outs["conv"].get_memory().read()
+    assert out.shape == p["expected"].shape
+    np.testing.assert_allclose(out.astype(np.float64), p["expected"], atol=max(p["tol"], 1e-5), rtol=0)
+
+
+# ------------------------------------------------------------------------------------------ networks vs the oracle
+def rand_layer(r, ofm, ifm, k, in_u8=True):
+    w = r.integers(-127, 128, (ofm, ifm, k, k)).astype(np.int8)
+    bias = r.integers(-1000, 1001, ofm).astype(np.int32)
+    sigma = np.sqrt(ifm * k * k) * (147.4 if in_u8 else 73.9) * 73.3
+    calib = (40.0 / sigma * r.uniform(0.5, 2.0, ofm)).astype(np.float32)
+    return w, bias, np.ones(ofm, np.float32), calib
+
+
+def bottleneck(eng, seed, B=2, C=64, M=32, H=14, W=14, unsigned=False):
+    """1x1 reduce -> 3x3 -> 1x1 expand + shortcut, relu: one ResNet bottleneck block.
+
+    Signed activations by default: the reference's stand-alone quantized eltwise saturates to the signed range
+    (generic_eltwise_ref.cl:318-330, convert_char_sat), so only then do the fused and the two-primitive graph agree."""
+    r = np.random.default_rng(seed)
+    np_dt, dt, name = (np.uint8, DT.u8, "u8") if unsigned else (np.int8, DT.i8, "s8")
+    x = (r.integers(0, 256, (B, C, H, W)) if unsigned else r.integers(-128, 128, (B, C, H, W))).astype(np_dt)
+    L = [rand_layer(r, M, C, 1, unsigned), rand_layer(r, M, M, 3, unsigned), rand_layer(r, C, M, 1, unsigned)]
+    ecal = r.uniform(0.4, 0.9, C).astype(np.float32)
+    prims = [cl.input_layout("input", cl.layout(dt, F.bfyx, cl.tensor(B, C, W, H)))]
+    for i, (w, b, q, c) in enumerate(L):
+        prims += [cl.data(f"w{i}", cl.make_memory(eng, w)), cl.data(f"b{i}", vec_mem(eng, b)), cl.data(f"q{i}", vec_mem(eng, q)),
+                  cl.data(f"c{i}", vec_mem(eng, c))]
+    prims += [cl.data("ecal", vec_mem(eng, ecal)),
+              cl.convolution("reduce", "input", ["w0"], ["b0"], ["q0"], ["c0"]),
+              cl.activation("reduce_relu", "reduce", cl.activation_func.relu),
+              cl.convolution("mid", "reduce_relu", ["w1"], ["b1"], ["q1"], ["c1"], input_offset=cl.tensor(0, 0, -1, -1, 0),
+                             with_activation=True),
+              cl.convolution("expand", "mid", ["w2"], ["b2"], ["q2"], ["c2"], output_data_type=DT.i8),
+              cl.eltwise("sum", "input", "expand", cl.eltwise_mode.sum, True, 0.0, output_calibration_factors="ecal"),
+              cl.reorder("out", "sum", F.bfyx)]
+
+    def oracle():
+        a = rc.conv(x, L[0][0], L[0][1], wqf=L[0][2], calib=L[0][3], out_dt=name, act="relu")
+        a = rc.conv(a, L[1][0], L[1][1], wqf=L[1][2], calib=L[1][3], pad=(1, 1), out_dt=name, act="relu")
+        return rc.conv(a, L[2][0], L[2][1], wqf=L[2][2], calib=L[2][3], out_dt=name, eltw=x, eltw_act="relu", eltw_calib=ecal)
+
+    return cl.topology(*prims), x, oracle
+
+
+@pytest.mark.parametrize("optimize", OPT, ids=["plain", "optimize_data"])
+def test_bottleneck_block(eng, optimize):
+    topo, x, oracle = bottleneck(eng, 7)
+    net, outs = run(eng, topo, {"input": cl.make_memory(eng, x)}, optimize)
+    out = outs["out"].get_memory().read()
+    expected = oracle()
+    assert out.dtype == np.int8 and out.shape == expected.shape
+    np.testing.assert_array_equal(out, expected)
+    executed = net.get_executed_primitive_ids()
+    if optimize:
+        # the graph the layout rule and the fusing passes produce: blocked int8 matrix-core kernels throughout
+        assert "reduce_relu" not in executed and "sum" not in executed and "expand_fused_sum" in executed
+        for pid in ("reduce", "mid", "expand_fused_sum"):
+            info = net.get_primitive_info(pid)
+            assert info["format"] == F.fs_b_yx_fsv16 and info["kernel"].startswith(("conv_mfma", "conv_stream")), info
+        assert "border" in net.get_primitive_info("mid")["kernel"]
+    else:
+        assert {"reduce", "reduce_relu", "mid", "expand", "sum", "out"} <= set(executed)
+        assert net.get_primitive_info("mid")["kernel"].startswith("conv_ref")
+    assert net.get_all_primitive_org_ids()[0] == "input"
+
+
+def test_unsigned_bottleneck_block(eng):
+    """Unsigned activations with a signed expand convolution: the data types of the benchmark's residual blocks."""
+    topo, x, oracle = bottleneck(eng, 8, unsigned=True)
+    net, outs = run(eng, topo, {"input": cl.make_memory(eng, x)}, True)
+    out = outs["out"].get_memory().read()
+    assert out.dtype == np.uint8 and out.max() > 127
+    np.testing.assert_array_equal(out, oracle())
+
+
+def test_fused_and_unfused_graphs_agree(eng):
+    """conv + eltwise executed as two primitives equals the fused primitive (the property the reference's fusing pass
+    relies on, src/graph_optimizer/prepare_primitive_fusing.cpp:181-337)."""
+    topo, x, _ = bottleneck(eng, 11, B=3, C=48, M=16, H=9, W=11)
+    outs = []
+    for optimize in OPT:
+        net, o = run(eng, topo, {"input": cl.make_memory(eng, x)}, optimize)
+        outs.append(o["out"].get_memory().read())
+    np.testing.assert_array_equal(outs[0], outs[1])
+
+
+def test_network_runs_again_with_new_input(eng):
+    topo, x, _ = bottleneck(eng, 3)
+    net = cl.network(eng, topo, cl.build_options(optimize_data=True))
+    net.set_input_data("input", cl.make_memory(eng, x))
+    first = net.execute()["out"].get_memory().read()
+    net.set_input_data("input", cl.make_memory(eng, np.zeros_like(x)))
+    second = net.execute()["out"].get_memory().read()
+    net.set_input_data("input", cl.make_memory(eng, x))
+    third = net.execute()["out"].get_memory().read()
+    assert not np.array_equal(first, second)
+    np.testing.assert_array_equal(first, third)
+
+
+def test_user_blocked_input_and_padded_input(eng):
+    """An input the user already holds in fs_b_yx_fsv16 is consumed in place; a bfyx input with physical padding is read
+    through its pitches (reference tests: input padding variants of convolution_gpu_test.cpp)."""
+    r = np.random.default_rng(5)
+    x = r.integers(-128, 128, (2, 32, 6, 7)).astype(np.int8)
+    w, b, q, c = rand_layer(r, 32, 32, 3, in_u8=False)
+    expected = rc.conv(x, w, b, wqf=q, calib=c, pad=(1, 1), out_dt="s8", act="relu")
+    consts = [cl.data("w", cl.make_memory(eng, w)), cl.data("b", vec_mem(eng, b)), cl.data("q", vec_mem(eng, q)),
+              cl.data("c", vec_mem(eng, c))]
+    conv = cl.convolution("conv", "input", ["w"], ["b"], ["q"], ["c"], input_offset=cl.tensor(0, 0, -1, -1, 0), with_activation=True)
+    pad = cl.padding((0, 0, 2, 3), (0, 0, 1, 0))
+    lay = cl.layout(DT.i8, F.bfyx, cl.tensor(2, 32, 7, 6), pad)
+    m = cl.memory.allocate(eng, lay)
+    m.write(x)
+    for optimize in OPT:
+        net, outs = run(eng, cl.topology(cl.input_layout("input", lay), conv, *consts), {"input": m}, optimize)
+        np.testing.assert_array_equal(outs["conv"].get_memory().read(), expected)
+    # blocked by the user: stage it with a reorder network first
+    stage = cl.topology(cl.input_layout("input", cl.layout(DT.i8, F.bfyx, cl.tensor(2, 32, 7, 6))),
+                        cl.reorder("blocked", "input", F.fs_b_yx_fsv16))
+    _, so = run(eng, stage, {"input": cl.make_memory(eng, x)}, False)
+    xb = so["blocked"].get_memory()
+    assert xb.get_layout().format == F.fs_b_yx_fsv16
+    topo = cl.topology(cl.input_layout("input", xb.get_layout()), conv, *consts, cl.reorder("plain", "conv", F.bfyx))
+    net, outs = run(eng, topo, {"input": xb}, True)
+    assert "input_to_fsv16_0" not in net.get_all_primitive_ids()
+    np.testing.assert_array_equal(outs["plain"].get_memory().read(), expected)
+
+
+def test_depthwise_through_network(eng):
+    r = np.random.default_rng(9)
+    C = 32
+    x = r.integers(0, 256, (2, C, 10, 10)).astype(np.uint8)
+    w = r.integers(-127, 128, (C, 1, 3, 3)).astype(np.int8)
+    b = r.integers(-500, 500, C).astype(np.int32)
+    q = np.ones(C, np.float32)
+    c = (40.0 / (3 * 147.4 * 73.3) * r.uniform(0.5, 2, C)).astype(np.float32)
+    expected = rc.conv(x, w, b, wqf=q, calib=c, pad=(1, 1), stride=(2, 2), groups=C, out_dt="u8", act="relu")
+    topo = cl.topology(cl.input_layout("input", cl.layout(DT.u8, F.bfyx, cl.tensor(2, C, 10, 10))),
+                       cl.data("w", cl.make_memory(eng, w)), cl.data("b", vec_mem(eng, b)), cl.data("q", vec_mem(eng, q)),
+                       cl.data("c", vec_mem(eng, c)),
+                       cl.convolution("dw", "input", ["w"], ["b"], ["q"], ["c"], stride=cl.tensor(1, 1, 2, 2),
+                                      input_offset=cl.tensor(0, 0, -1, -1, 0), with_activation=True, groups=C))
+    for optimize in OPT:
+        net, outs = run(eng, topo, {"input": cl.make_memory(eng, x)}, optimize)
+        np.testing.assert_array_equal(outs["dw"].get_memory().read(), expected)
+    assert net.get_primitive_info("dw_fsv16")["kernel"].startswith("conv_dw")
+
+
+def test_attached_constants_and_input(eng):
+    """Host memory attached with cldnn_attach_memory serves as constants and as network input."""
+    r = np.random.default_rng(2)
+    x = r.integers(-128, 128, (1, 16, 5, 5)).astype(np.int8)
+    w, b, q, c = rand_layer(r, 16, 16, 1, in_u8=False)
+
+    def att(a, shape):
+        a = np.ascontiguousarray(a)
+        return cl.memory.attach(cl.layout(cl.DT_OF[a.dtype], F.bfyx, cl.tensor(*shape)), a)
+
+    topo = cl.topology(cl.input_layout("input", cl.layout(DT.i8, F.bfyx, cl.tensor(1, 16, 5, 5))),
+                       cl.data("w", att(w, (16, 16, 1, 1))), cl.data("b", att(b, (1, 1, 16, 1))),
+                       cl.data("q", att(q, (1, 1, 16, 1))), cl.data("c", att(c, (1, 1, 16, 1))),
+                       cl.convolution("conv", "input", ["w"], ["b"], ["q"], ["c"]))
+    net, outs = run(eng, topo, {"input": att(x, (1, 16, 5, 5))}, True)
+    np.testing.assert_array_equal(outs["conv"].get_memory().read(), rc.conv(x, w, b, wqf=q, calib=c, out_dt="s8"))
+
+
+# ------------------------------------------------------------------------------------------ runtime objects
+def test_memory_lock_roundtrip_and_identity(eng):
+    a = np.arange(2 * 3 * 4 * 5, dtype=np.float32).reshape(2, 3, 4, 5)
+    for fmt in (F.bfyx, F.yxfb, F.byxf):
+        m = cl.make_memory(eng, a, fmt)
+        np.testing.assert_array_equal(m.read(), a)
+    m2 = cl.memory.allocate(eng, m.get_layout())
+    assert m.is_the_same_buffer(m) and not m.is_the_same_buffer(m2)
+    assert np.count_nonzero(m2.read()) == 0  # fresh memory is zero-filled
+    assert eng.get_temp_used_device_memory_size() > 0
+    assert eng.get_max_used_device_memory_size() >= eng.get_temp_used_device_memory_size()
+    info = eng.get_info()
+    assert info.cores_count >= 64 and info.supports_immad == 1 and info.max_global_mem_size > (1 << 34)
+
+
+def test_set_input_errors(eng):
+    topo, x, _ = bottleneck(eng, 1)
+    net = cl.network(eng, topo)
+    with pytest.raises(cl.error) as e:
+        net.execute()
+    assert "has not been set" in str(e.value)
+    with pytest.raises(cl.error) as e:
+        net.set_input_data("input", cl.make_memory(eng, x[:1]))
+    assert "layout" in str(e.value)
+    with pytest.raises(cl.error):
+        net.set_input_data("mid", cl.make_memory(eng, x))
+    with pytest.raises(cl.error):
+        cl._call("cldnn_get_network_output_memory", net.h, b"out")  # not executed yet
+
+
+def test_events_and_profiling():
+    eng = cl.engine(enable_profiling=True)
+    topo, x, oracle = bottleneck(eng, 4)
+    net = cl.network(eng, topo, cl.build_options(optimize_data=True))
+    net.set_input_data("input", cl.make_memory(eng, x))
+    gate = cl.event.create_user_event(eng)
+    assert gate.is_user_event()
+    gate.set()
+    outs = net.execute([gate])
+    ev = outs["out"].get_event()
+    ev.wait()
+    prof = ev.get_profiling_info()
+    assert set(prof) == {"submission", "starting", "executing"}
+    assert 0 < prof["executing"] < 50_000_000
+    np.testing.assert_array_equal(outs["out"].get_memory().read(), oracle())
+    fired = []
+    cb = cl.EVENT_HANDLER(lambda p: fired.append(1))
+    cl._call("cldnn_add_event_handler", ev.h, cb, None)
+    assert fired == [1]  # the event is complete: the handler runs at once
+
+
+def test_unsupported_requests_fail_loudly(eng):
+    lay = cl.layout(DT.f16, F.bfyx, cl.tensor(1, 16, 4, 4))
+    with pytest.raises(cl.error) as e:
+        cl.memory.allocate(eng, lay)
+    assert e.value.status == cl.UNSUPPORTED_FORMAT
+    topo = cl.topology(cl.input_layout("input", cl.layout(DT.i8, F.bfyx, cl.tensor(1, 16, 4, 4))),
+                       cl.activation("act", "input", cl.activation_func.logistic))
+    net = cl.network(eng, topo)
+    net.set_input_data("input", cl.make_memory(eng, np.zeros((1, 16, 4, 4), np.int8)))
+    with pytest.raises(cl.error) as e:
+        net.execute()
+    assert "not supported" in str(e.value)
