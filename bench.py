@@ -106,10 +106,12 @@ class GpuTimer:
         hip.check(hip.lib().cldnn_hip_event_record_end(self.ev))
 
     def seconds(self):
-        ns = C.c_uint64()
-        hip.check(hip.lib().cldnn_hip_event_elapsed_ns(self.ev, C.byref(ns)))
-        hip.check(hip.lib().cldnn_hip_event_release(self.ev))
-        return ns.value * 1e-9
+        if self.ev is not None:  # read once, then give the event back
+            ns = C.c_uint64()
+            hip.check(hip.lib().cldnn_hip_event_elapsed_ns(self.ev, C.byref(ns)))
+            hip.check(hip.lib().cldnn_hip_event_release(self.ev))
+            self.ev, self.value = None, ns.value * 1e-9
+        return self.value
 
 
 def cpu_pass(eng, stack, images, verify):
@@ -144,17 +146,53 @@ def cpu_baseline_and_check(eng, stack, batch, budget_seconds):
     return dict(images=n, seconds=tn, threads=threads, checked=checked, mismatches=mism)
 
 
+def copy_calibration(args):
+    """A plain device copy of known size (256 MiB read + 256 MiB written per step): the yardstick that the
+    FETCH_SIZE / WRITE_SIZE counter readings of the convolution kernels are scaled by."""
+    eng = hip.Engine(0, profiling=True)
+    t = hip.Tensor.make(hip.F32, hip.BFYX, 1, 64, 1024, 1024)
+    src, dst = hip.Buffer(eng, t), hip.Buffer(eng, t)
+    for _ in range(args.warmup):
+        hip.reorder(eng, src, dst)
+    eng.finish()
+    with GpuTimer(eng) as tm:
+        for _ in range(args.steps):
+            hip.reorder(eng, src, dst)
+    eng.finish()
+    nbytes = 2 * src.nbytes
+    print(json.dumps({"metric": "device copy", "value": nbytes * args.steps / tm.seconds() / 1e9, "unit": "GB/s", "n_gpus": 1,
+                      "steps": args.steps, "warmup": args.warmup, "ms_per_step": tm.seconds() / args.steps * 1e3,
+                      "higher_is_better": True, "config": {"workload": "copy_256m", "read_bytes": src.nbytes,
+                                                           "written_bytes": src.nbytes}}), flush=True)
+
+
+def measured_traffic(workload):
+    """HBM bytes per launch from the committed counter summary of this workload (None when there is none)."""
+    path = os.path.join(ROOT, "profiles", "conv_stack_%s_hbm_traffic.txt" % workload)
+    if not os.path.exists(path):
+        return None
+    with open(path) as f:
+        for line in f:
+            if line.startswith("traffic_bytes_per_launch:"):
+                return int(line.split(":")[1])
+    return None
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=30)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="resnet50_b32_fused",
-                    choices=["resnet50_b32_fused", "resnet50_b32", "resnet50_b1", "vgg16_b16", "mobilenet_v2_b32", "c1"])
+                    choices=["resnet50_b32_fused", "resnet50_b32", "resnet50_b1", "vgg16_b16", "mobilenet_v2_b32", "c1",
+                             "copy_256m"])
     ap.add_argument("--tile", type=int, default=0, help="force one row (index+1) of the tile table on every layer")
     ap.add_argument("--per-layer", action="store_true", help="time every layer on its own and print a table to stderr")
     ap.add_argument("--tune", action="store_true", help="try every row of the tile table on every layer, print the best")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline / full-size check")
+    ap.add_argument("--host-io", action="store_true",
+                    help="also report the rate with the first layer's input crossing PCIe into the device and the last "
+                         "layer's output crossing back, every step (never the headline value)")
     ap.add_argument("--cpu-seconds", type=float, default=15.0)
     args = ap.parse_args()
     if args.gpus != 1:
@@ -163,6 +201,8 @@ def main():
         sys.exit(2)
 
     wl = args.workload
+    if wl == "copy_256m":
+        return copy_calibration(args)
     if wl.startswith("resnet50"):
         layers, batch, fuse = workloads.resnet50(), (1 if wl.endswith("b1") else 32), wl.endswith("fused")
     elif wl == "vgg16_b16":
@@ -196,6 +236,25 @@ def main():
     launches = len(stack) * args.steps
     ms_per_step = t_wall / args.steps * 1e3
     value = batch * args.steps / t_wall
+
+    host_io = None
+    if args.host_io:
+        # what a caller holding host tensors pays: bfyx input host -> device, device reorder into the blocked layout
+        # with its border, the stack, blocked output device -> host
+        first, last_l = stack[0], stack[-1]
+        plain = hip.Buffer(eng, hip.Tensor.make(first.xin.tensor.dtype, hip.BFYX, *first.x.shape))
+        for _ in range(2):
+            plain.write_raw(first.x); hip.reorder(eng, plain, first.xin); run_step(stack); last_l.out.read_raw()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            plain.write_raw(first.x)
+            hip.reorder(eng, plain, first.xin)
+            run_step(stack)
+            last_l.out.read_raw()
+        dt = time.perf_counter() - t0
+        host_io = {"images_per_s": batch * args.steps / dt, "ms_per_step": dt / args.steps * 1e3,
+                   "host_to_device_bytes": int(first.x.nbytes), "device_to_host_bytes": int(last_l.out.nbytes)}
+        plain.close()
 
     per_layer = None
     if args.per_layer or args.tune:
@@ -273,7 +332,7 @@ def main():
             "peak": PEAK_INT8_OPS / 1e12,
             "unit": "TOP/s",
             "frac": ops * args.steps / t_gpu / PEAK_INT8_OPS,
-            "traffic": None,
+            "traffic": measured_traffic(wl),
             "kernel": "conv_mfma_kernel (all tile instances)",
             "launches": launches,
             "avg_launch_us": t_gpu / launches * 1e6,
@@ -290,6 +349,8 @@ def main():
         "gpu_seconds_events": t_gpu,
         "wall_seconds": t_wall,
     }
+    if host_io:
+        res["pcie_inclusive"] = host_io
 
     if not args.no_cpu:
         cb = cpu_baseline_and_check(eng, stack, batch, args.cpu_seconds)
