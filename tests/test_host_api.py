@@ -54,6 +54,18 @@ def test_headers_compile_as_c_and_cpp(tmp_path):
         assert rc_ == 0, name
 
 
+def test_cpp_api_program_builds_and_needs_a_gpu():
+    """The C++ wrappers (include/api/CPP) compile into the reference-style test program; without a GPU it stops at
+    engine creation with the library's message instead of computing anything on the host."""
+    import subprocess
+    import torch
+    r = subprocess.run(["make", "-C", os.path.join(ROOT, "tests", "cpp"), "conv_network_test"], capture_output=True, text=True)
+    assert r.returncode == 0, r.stdout + r.stderr
+    if not torch.cuda.is_available():
+        r = subprocess.run([os.path.join(ROOT, "tests", "cpp", "conv_network_test")], capture_output=True, text=True)
+        assert r.returncode == 2 and "no HIP device" in r.stdout, r.stdout + r.stderr
+
+
 def test_version():
     v = cl._call("cldnn_get_version")
     assert (v.major, v.minor) == (1, 4)

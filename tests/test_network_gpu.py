@@ -261,6 +261,18 @@ def test_attached_constants_and_input(eng):
     np.testing.assert_array_equal(outs["conv"].get_memory().read(), rc.conv(x, w, b, wqf=q, calib=c, out_dt="s8"))
 
 
+def test_cpp_api_program():
+    """The same path through the C++ wrappers: tests/cpp/conv_network_test.cpp compares five networks with the oracle."""
+    import os
+    import subprocess
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    exe = os.path.join(root, "tests", "cpp", "conv_network_test")
+    if not os.path.exists(exe):
+        subprocess.run(["make", "-C", os.path.dirname(exe), "conv_network_test"], check=True)
+    r = subprocess.run([exe], capture_output=True, text=True, timeout=100)
+    assert r.returncode == 0 and "all cases passed" in r.stdout, r.stdout + r.stderr
+
+
 # ------------------------------------------------------------------------------------------ runtime objects
 def test_memory_lock_roundtrip_and_identity(eng):
     a = np.arange(2 * 3 * 4 * 5, dtype=np.float32).reshape(2, 3, 4, 5)
