@@ -189,6 +189,8 @@ def main():
     ap.add_argument("--tile", type=int, default=0, help="force one row (index+1) of the tile table on every layer")
     ap.add_argument("--per-layer", action="store_true", help="time every layer on its own and print a table to stderr")
     ap.add_argument("--tune", action="store_true", help="try every row of the tile table on every layer, print the best")
+    ap.add_argument("--only", default="", help="comma-separated layer names: run just these layers of the workload "
+                                               "(same buffers every step, so their tensors stay cache-resident)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline / full-size check")
     ap.add_argument("--host-io", action="store_true",
                     help="also report the rate with the first layer's input crossing PCIe into the device and the last "
@@ -211,6 +213,13 @@ def main():
         layers, batch, fuse = workloads.mobilenet_v2(), 32, False
     else:
         layers, batch, fuse = [workloads._layer("c1", 64, 64, 3, 1, 1, 56)], 1, False
+
+    if args.only:
+        keep = set(args.only.split(","))
+        layers = [l for l in layers if l["name"] in keep]
+        if not layers:
+            log("bench.py: no layer of %s is named in --only" % wl)
+            sys.exit(2)
 
     eng = hip.Engine(0, profiling=True)
     info = eng.info()

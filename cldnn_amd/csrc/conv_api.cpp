@@ -217,7 +217,7 @@ void build(cldnn_hip_conv c, const void* weights, const void* bias, const float*
     if (impl == CLDNN_HIP_IMPL_MFMA) {
         int tile = d.tile_override > 0 ? d.tile_override - 1 : mfma_choose(p, c->engine->props.multiProcessorCount);
         CHIP_REQUIRE(tile >= 0 && tile < tile_config_count(), CLDNN_HIP_INVALID_ARG, "tile_override out of range");
-        c->mplan = mfma_plan(p, tile);
+        c->mplan = mfma_plan(p, tile, c->engine->props.multiProcessorCount);
         std::vector<int8_t> packed(c->mplan.packed_bytes);
         std::vector<int32_t> ktab(c->mplan.ktab_bytes / sizeof(int32_t));
         mfma_pack_weights(p, c->mplan, w8, packed.data(), ktab.data());
@@ -227,7 +227,7 @@ void build(cldnn_hip_conv c, const void* weights, const void* bias, const float*
         const TileConfig& tc = tile_config(tile);
         inf.tile_index = tile, inf.tile_pixels = tc.tile_pixels, inf.tile_ofm = tc.tile_ofm;
         inf.grid = c->mplan.grid, inf.block = 256, inf.lds_bytes = c->mplan.lds_bytes;
-        std::snprintf(inf.kernel_name, sizeof(inf.kernel_name), "conv_%s<%s,%s,%s>", c->mplan.stream ? "stream" : "mfma",
+        std::snprintf(inf.kernel_name, sizeof(inf.kernel_name), "conv_%s<%s,%s,%s>", c->mplan.stream ? "stream" : (c->mplan.bdir ? "bdir" : (c->mplan.wsl ? "wsl" : "mfma")),
                       tc.name, c->mplan.checked ? "checked" : "border", c->fast ? "fast" : "generic");
     } else {
         c->dplan = dw_plan(p);

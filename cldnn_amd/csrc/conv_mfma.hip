@@ -1,5 +1,6 @@
 // Host side of the int8 MFMA convolution: the gfx950 tile-config table, plans, weight
 // pre-packing, eligibility of the short epilogue and the launch.
+#include <algorithm>
 #include <cmath>
 #include <cstring>
 
@@ -11,6 +12,13 @@ namespace chip {
 DECL_TILE(0) DECL_TILE(1) DECL_TILE(2) DECL_TILE(3) DECL_TILE(4) DECL_TILE(5)
 #undef DECL_TILE
 void launch_stream(hipStream_t s, const MfmaArgs& a, int nt, int grid, int epi);
+void launch_bdir_f64(hipStream_t s, const MfmaArgs& a, int nt, int grid, int lds, int epi);
+void launch_bdir_f128(hipStream_t s, const MfmaArgs& a, int nt, int grid, int lds, int epi);
+void launch_bdir_k2(hipStream_t s, const MfmaArgs& a, int nt, int grid, int lds, int epi);
+void launch_bdir_k4(hipStream_t s, const MfmaArgs& a, int nt, int grid, int lds, int epi);
+#define DECL_WSL(d) void launch_wsl_d##d(hipStream_t s, const MfmaArgs& a, int nt, int grid, int lds, int epi);
+DECL_WSL(1) DECL_WSL(2) DECL_WSL(3) DECL_WSL(4) DECL_WSL(6) DECL_WSL(8)
+#undef DECL_WSL
 
 typedef void (*tile_launcher)(hipStream_t, const MfmaArgs&, int, int, bool, int);
 
@@ -24,9 +32,26 @@ static const TileConfig g_tiles[] = {
     // rows of the streaming kernel: a wave owns one span of 64 features of one tile of wave_pixels pixels
     {"stream_p16", 16, 64, 16},
     {"stream_p32", 32, 64, 32},
+    // rows of the direct-activation kernel: weights through LDS, activations straight into registers;
+    // a wave owns wave_pixels pixels and all tile_ofm features
+    {"bdir_p64_f64", 64, 64, 16},
+    {"bdir_p128_f64", 128, 64, 32},
+    {"bdir_p256_f64", 256, 64, 64},
+    {"bdir_p64_f128", 64, 128, 16},
+    {"bdir_p128_f128", 128, 128, 32},
+    {"bdir_p256_f128", 256, 128, 64},
+    // rows of the weights-stationary kernel: persistent workgroups, the 64-feature weight tile resident in LDS
+    {"wsl_p64", 64, 64, 16},
+    {"wsl_p128", 128, 64, 32},
+    {"wsl_p256", 256, 64, 64},
+    // direct-activation kernel with K split over 2 or 4 groups of four waves inside the workgroup
+    {"bdir_k2_p64_f64", 64, 64, 16, 2},
+    {"bdir_k4_p64_f64", 64, 64, 16, 4},
+    {"bdir_k2_p128_f64", 128, 64, 32, 2},
 };
-enum { FIRST_STREAM_ROW = 6 };
-enum { MFMA_SLACK_STEPS = 10 };  // >= largest prefetch distance + 1
+enum { FIRST_STREAM_ROW = 6, FIRST_BDIR_ROW = 8, FIRST_WSL_ROW = 14, FIRST_BDIRK_ROW = 17 };
+enum { WSL_MAX_LDS = 160 * 1024 };
+enum { MFMA_SLACK_STEPS = 40 };  // >= weight look-ahead + activation look-ahead + 3
 static const tile_launcher g_launch[] = {launch_mfma_tile_0, launch_mfma_tile_1, launch_mfma_tile_2, launch_mfma_tile_3,
                                          launch_mfma_tile_4, launch_mfma_tile_5};
 
@@ -57,19 +82,21 @@ static bool border_covers(const ConvProblem& p)
     return t.pad_lo_y >= p.py && t.pad_lo_x >= p.px && t.pad_hi_y >= hi_y && t.pad_hi_x >= hi_x;
 }
 
-// ---- the gfx950 tile-config table lookup.  Key: (pixels M, OFM, K-steps, border available); value: table row.
-int mfma_choose(const ConvProblem& p, int cus)
+// ---- the gfx950 tile-config table lookup.  Key: (pixels M, OFM, K-steps, border available, slices in fours);
+// value: table row.  The entries come from sweeps of every row over every layer shape of the ResNet-50,
+// VGG-16 and MobileNet-v2 stacks (bench.py --tune); they stand where the reference keeps a tuned cache file.
+enum {
+    ROW_P128_F128 = 0, ROW_P256_F64 = 1, ROW_P64_F128 = 2, ROW_P128_F64 = 3, ROW_P64_F64 = 4, ROW_P256_F128 = 5,
+    ROW_STREAM_P16 = 6, ROW_STREAM_P32 = 7,
+    ROW_BDIR_P64_F64 = 8, ROW_BDIR_P128_F64 = 9, ROW_BDIR_P256_F64 = 10, ROW_BDIR_P64_F128 = 11, ROW_BDIR_P128_F128 = 12,
+    ROW_BDIR_P256_F128 = 13, ROW_WSL_P64 = 14, ROW_WSL_P128 = 15, ROW_WSL_P256 = 16,
+    ROW_BDIR_K2_P64_F64 = 17, ROW_BDIR_K4_P64_F64 = 18, ROW_BDIR_K2_P128_F64 = 19
+};
+
+static int choose_lds_tile(const ConvProblem& p, int64_t m, int cus)
 {
-    const int64_t m = (int64_t)p.B * p.OH * p.OW;
-    const int ksteps = (p.FY * p.FX * ((p.IFM + 15) / 16) + 3) / 4;
-    if (ksteps <= 8 && border_covers(p)) {
-        // short K: bound by HBM bandwidth.  Stream unless there are too few pixels to occupy the chip
-        const int64_t waves = ((m + 31) / 32) * ((p.OFM + 63) / 64);
-        if (waves >= 4ll * cus) return FIRST_STREAM_ROW + 1;
-        if (waves * 2 >= 4ll * cus) return FIRST_STREAM_ROW;
-    }
-    static const int order_f128[] = {5, 0, 2, 1, 3, 4};
-    static const int order_f64[] = {1, 3, 4};
+    static const int order_f128[] = {ROW_P256_F128, ROW_P128_F128, ROW_P64_F128, ROW_P256_F64, ROW_P128_F64, ROW_P64_F64};
+    static const int order_f64[] = {ROW_P256_F64, ROW_P128_F64, ROW_P64_F64};
     const int* order = p.OFM > 64 ? order_f128 : order_f64;
     const int n = p.OFM > 64 ? 6 : 3;
     int best = order[n - 1];
@@ -83,16 +110,76 @@ int mfma_choose(const ConvProblem& p, int cus)
     return best;
 }
 
-MfmaPlan mfma_plan(const ConvProblem& p, int tile)
+int mfma_choose(const ConvProblem& p, int cus)
+{
+    const int64_t m = (int64_t)p.B * p.OH * p.OW;
+    const int cb = (p.IFM + 15) / 16;
+    const int ksteps = (p.FY * p.FX * cb + 3) / 4;
+    const bool border = border_covers(p);
+    const bool direct = border && cb % 4 == 0;  // the direct-activation and weights-stationary kernels apply
+    const int64_t stream_waves = ((m + 31) / 32) * ((p.OFM + 63) / 64);
+    const bool stream_fits = border && ksteps <= 8 && stream_waves * 2 >= 4ll * cus;
+    const int stream_row = stream_waves >= 4ll * cus ? ROW_STREAM_P32 : ROW_STREAM_P16;
+
+    if (ksteps <= 2 || !direct) {
+        // one or two K-steps: bound by HBM bandwidth, one memory round trip per wave
+        if (stream_fits) return stream_row;
+        return choose_lds_tile(p, m, cus);
+    }
+    if (ksteps <= 8) {
+        if (m >= 16384) return ROW_WSL_P64;                       // 1x1 reductions at 56x56 and 28x28
+        if (m >= 4096) {
+            if (p.OFM >= 512) return ksteps <= 4 ? ROW_WSL_P128 : ROW_BDIR_P128_F128;  // 14x14 expansions / projections
+            return stream_fits ? stream_row : ROW_BDIR_P64_F64;
+        }
+        if (p.OFM >= 1024) return ROW_P64_F128;                   // 7x7 expansions
+        return stream_fits ? stream_row : ROW_BDIR_P64_F64;
+    }
+    // long K
+    if (ksteps <= 40 && m >= 50000 && p.OFM <= 64) return ROW_WSL_P128;          // 3x3 at 56x56, 64 features
+    if (m >= 100000 && p.OFM >= 128) return ROW_BDIR_P256_F128;                  // VGG-sized layers
+    if (m >= 16384) return p.OFM > 64 || m >= 50000 ? ROW_BDIR_P128_F64 : ROW_BDIR_P64_F64;
+    if (m >= 4096) return ROW_BDIR_P64_F64;                                      // 14x14
+    if (ksteps >= 32) return ROW_BDIR_K2_P64_F64;                                // 7x7 with K >= 2048: split K in the workgroup
+    if (p.OFM >= 1024) return ROW_P128_F128;
+    return ROW_BDIR_P64_F64;
+}
+
+// look-ahead D of the weights-stationary kernel and the K-step count padded to a multiple of it:
+// least padding first, then the deepest look-ahead
+static void wsl_depth(int ksteps, int* depth, int* padded)
+{
+    static const int depths[] = {8, 6, 4, 3, 2, 1};
+    int best_d = 1, best_pad = ksteps;
+    for (int d : depths) {
+        const int pad = (ksteps + d - 1) / d * d;
+        if (pad < best_pad || (pad == best_pad && d > best_d)) best_pad = pad, best_d = d;
+    }
+    // one padded step in sixteen is cheaper than a shallow look-ahead
+    for (int d : depths) {
+        const int pad = (ksteps + d - 1) / d * d;
+        if (d > best_d && (pad - ksteps) * 16 <= ksteps) {
+            best_d = d, best_pad = pad;
+            break;
+        }
+    }
+    *depth = best_d, *padded = best_pad;
+}
+
+MfmaPlan mfma_plan(const ConvProblem& p, int tile, int cus)
 {
     const TileConfig& tc = g_tiles[tile];
     MfmaPlan pl{};
     pl.tile = tile;
     pl.checked = border_covers(p) ? 0 : 1;
-    pl.stream = tile >= FIRST_STREAM_ROW ? 1 : 0;
+    pl.stream = tile >= FIRST_STREAM_ROW && tile < FIRST_BDIR_ROW ? 1 : 0;
+    pl.bdir = (tile >= FIRST_BDIR_ROW && tile < FIRST_WSL_ROW) || tile >= FIRST_BDIRK_ROW ? 1 : 0;
+    pl.wsl = tile >= FIRST_WSL_ROW && tile < FIRST_BDIRK_ROW ? 1 : 0;
     CHIP_REQUIRE(!(pl.stream && pl.checked), CLDNN_HIP_INVALID_ARG,
                  "the streaming kernel needs an input whose physical zero border covers the convolution's padding");
     pl.cb = (p.IFM + 15) / 16;
+    CHIP_REQUIRE(!(pl.bdir || pl.wsl) || (!pl.checked && pl.cb % 4 == 0), CLDNN_HIP_INVALID_ARG,
+                 "the direct-activation kernels need a zero border covering the padding and input features in multiples of 64");
     pl.kchunks = p.FY * p.FX * pl.cb;
     pl.ksteps = (pl.kchunks + 3) / 4;
     if (pl.stream) {
@@ -101,15 +188,37 @@ MfmaPlan mfma_plan(const ConvProblem& p, int tile)
         while (ks < pl.ksteps) ks *= 2;  // compile-time K-step counts: 1, 2, 4, 8 (zero-weight padding chunks)
         pl.ksteps = ks;
     }
+    if (tc.kgroups > 1) pl.ksteps = (pl.ksteps + tc.kgroups - 1) / tc.kgroups * tc.kgroups;  // zero-weight padding steps
+    if (pl.wsl) {
+        wsl_depth(pl.ksteps, &pl.wsl_depth, &pl.ksteps);
+        CHIP_REQUIRE(pl.ksteps * 4096 <= WSL_MAX_LDS, CLDNN_HIP_INVALID_ARG,
+                     "the weights-stationary kernel holds 64 x K weight bytes in LDS: K is limited to 2560");
+    }
     pl.ofm_tiles = (p.OFM + tc.tile_ofm - 1) / tc.tile_ofm;
     pl.m_total = (int64_t)p.B * p.OH * p.OW;
     CHIP_REQUIRE(pl.m_total < (1ll << 31), CLDNN_HIP_UNSUPPORTED_SIZE, "more than 2^31 output pixels");
     pl.mtiles = (int)((pl.m_total + tc.tile_pixels - 1) / tc.tile_pixels);
-    int64_t grid = (int64_t)((pl.mtiles + 7) / 8) * 8 * pl.ofm_tiles;
+    // which operand do the eight dies share out?  the larger one (it is then read from memory once, not 8 times)
+    const int64_t w_bytes = (int64_t)p.OFM * (p.IFM / p.groups) * p.FY * p.FX, in_bytes = (int64_t)p.B * p.IFM * p.IH * p.IW;
+    pl.by_features = !pl.stream && !pl.wsl && w_bytes > in_bytes && (p.OFM + tc.tile_ofm - 1) / tc.tile_ofm >= 8 ? 1 : 0;
+    int64_t grid = pl.by_features ? (int64_t)((pl.ofm_tiles + 7) / 8) * 8 * pl.mtiles : (int64_t)((pl.mtiles + 7) / 8) * 8 * pl.ofm_tiles;
     if (pl.stream) grid = ((int64_t)pl.mtiles * pl.ofm_tiles + 3) / 4;  // one wave per (pixel tile, span)
+    pl.lds_bytes = pl.stream ? 0 : (pl.bdir ? 3 * 4 * tc.tile_ofm * 16 : 2 * 4 * (tc.tile_ofm + tc.tile_pixels) * 16);
+    if (tc.kgroups > 1)  // per-group weight buffers, later reused for the partial sums of groups 1..
+        pl.lds_bytes = std::max(tc.kgroups * pl.lds_bytes, (tc.kgroups - 1) * (tc.tile_ofm / 16) * (tc.wave_pixels / 16) * 4096);
+    if (pl.wsl) {
+        // persistent workgroups: as many as the chip holds at once (LDS and registers allow two per CU at most),
+        // split evenly over the feature tiles; partitions come in eights (one per accelerator die)
+        pl.lds_bytes = pl.ksteps * 4096;
+        const int per_cu = pl.lds_bytes * 2 <= WSL_MAX_LDS ? 2 : 1;
+        int parts = std::max(8, cus * per_cu / pl.ofm_tiles / 8 * 8);
+        pl.wsl_tpp = (pl.mtiles + parts - 1) / parts;
+        parts = ((pl.mtiles + pl.wsl_tpp - 1) / pl.wsl_tpp + 7) / 8 * 8;
+        pl.wsl_parts = parts;
+        grid = (int64_t)parts * pl.ofm_tiles;
+    }
     CHIP_REQUIRE(grid < (1ll << 31), CLDNN_HIP_UNSUPPORTED_SIZE, "convolution too large for one launch");
     pl.grid = (int)grid;
-    pl.lds_bytes = pl.stream ? 0 : 2 * 4 * (tc.tile_ofm + tc.tile_pixels) * 16;
     // the tile kernel requests operands up to MFMA_SLACK_STEPS K-steps past the end (zero weights there)
     pl.packed_bytes = ((size_t)pl.ofm_tiles * pl.ksteps + MFMA_SLACK_STEPS) * 4 * tc.tile_ofm * 16;
     pl.ktab_bytes = (size_t)(pl.ksteps + MFMA_SLACK_STEPS) * 4 * sizeof(int32_t);
@@ -240,6 +349,8 @@ void launch_conv_mfma(hipStream_t s, const ConvProblem& p, const MfmaPlan& pl, c
     a.CB = pl.cb, a.FX = p.FX, a.kchunks = pl.kchunks;
     a.tap_dy = p.dy * (int32_t)p.in_p.py, a.tap_dx = p.dx * 16;
     a.div_cb = make_div((uint32_t)pl.cb), a.div_fx = make_div((uint32_t)p.FX);
+    a.wsl_parts = pl.wsl_parts, a.wsl_tpp = pl.wsl_tpp, a.FY = p.FY;
+    a.by_features = pl.by_features;
     {
         // dense tensors and a 1x1 / stride-1 convolution: pixel m sits at byte m * 16 of every feature slice
         auto dense = [](const cldnn_hip_tensor& t) {
@@ -263,6 +374,21 @@ void launch_conv_mfma(hipStream_t s, const ConvProblem& p, const MfmaPlan& pl, c
         }
     }
     if (pl.stream) launch_stream(s, a, tc.wave_pixels / 16, pl.grid, kind);
+    else if (pl.bdir && tc.kgroups == 2) launch_bdir_k2(s, a, tc.wave_pixels / 16, pl.grid, pl.lds_bytes, kind);
+    else if (pl.bdir && tc.kgroups == 4) launch_bdir_k4(s, a, tc.wave_pixels / 16, pl.grid, pl.lds_bytes, kind);
+    else if (pl.bdir && tc.tile_ofm == 64) launch_bdir_f64(s, a, tc.wave_pixels / 16, pl.grid, pl.lds_bytes, kind);
+    else if (pl.bdir) launch_bdir_f128(s, a, tc.wave_pixels / 16, pl.grid, pl.lds_bytes, kind);
+    else if (pl.wsl) {
+        const int nt = tc.wave_pixels / 16;
+        switch (pl.wsl_depth) {
+        case 1: launch_wsl_d1(s, a, nt, pl.grid, pl.lds_bytes, kind); break;
+        case 2: launch_wsl_d2(s, a, nt, pl.grid, pl.lds_bytes, kind); break;
+        case 3: launch_wsl_d3(s, a, nt, pl.grid, pl.lds_bytes, kind); break;
+        case 4: launch_wsl_d4(s, a, nt, pl.grid, pl.lds_bytes, kind); break;
+        case 6: launch_wsl_d6(s, a, nt, pl.grid, pl.lds_bytes, kind); break;
+        default: launch_wsl_d8(s, a, nt, pl.grid, pl.lds_bytes, kind); break;
+        }
+    }
     else g_launch[pl.tile](s, a, pl.grid, pl.lds_bytes, pl.checked != 0, kind);
     CHIP_CHECK(hipGetLastError());
 }

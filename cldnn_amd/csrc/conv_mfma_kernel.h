@@ -59,6 +59,10 @@ struct MfmaArgs {
     int32_t ksteps;
     // streaming kernel: tap offsets by arithmetic, dense-tensor shortcut
     int32_t CB, FX, kchunks, tap_dy, tap_dx, linear;
+    // weights-stationary kernel: pixel-tile partitions per feature tile, tiles per partition, filter rows
+    int32_t wsl_parts, wsl_tpp, FY;
+    // 1: the eight accelerator dies split the FEATURE tiles between them (weights are the larger operand)
+    int32_t by_features;
     FastDiv div_cb, div_fx;
     uint32_t xor_mask;  // 0x80808080 for u8 activations, 0 for s8
     FastEpi fe;
@@ -81,6 +85,11 @@ __device__ __forceinline__ void lds_barrier()
 {
     asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
 }
+// Keeps the instruction scheduler from moving work across the boundary of two K-steps.  Without it the
+// compiler hoists register-only work on the operands of a LATE step (the sign flip of u8 activations) to the
+// top of the unrolled loop, which makes it wait for the newest outstanding load there and drains the whole
+// look-ahead queue once per loop iteration.
+__device__ __forceinline__ void step_fence() { __builtin_amdgcn_sched_barrier(0); }
 
 // Uniform table lookups go through the scalar data path (constant address space): a vector load here
 // would sit in the same in-order counter as the prefetched operand loads and force them to drain.
@@ -361,13 +370,16 @@ __global__ void __launch_bounds__(256) conv_mfma_kernel(MfmaArgs a)
     const int kq = lane >> 4;
     const int l16 = lane & 15;
 
-    // Workgroups that share activation pixels (same pixel tile, different feature tiles) get ids that are
-    // congruent modulo 8 and adjacent in time: they land on the same accelerator die and share its L2.
+    // Workgroup ids are dealt round-robin to the eight accelerator dies, each with its own L2 that starts
+    // cold.  The dies split the tiles of the SMALLER operand's counterpart between them, so the larger operand
+    // is fetched from memory once in total and only the smaller one once per die: by default a die takes every
+    // eighth pixel tile with all its feature tiles (adjacent in time, they share the activations through L2);
+    // with by_features it takes every eighth feature tile with all pixel tiles (sharing the weights).
     const int xcd = blockIdx.x & 7;
     const int j = blockIdx.x >> 3;
-    const int ptile = (j / a.ofm_tiles) * 8 + xcd;
-    const int ntile = j % a.ofm_tiles;
-    if (ptile >= a.mtiles) return;
+    const int ptile = a.by_features ? j % a.mtiles : (j / a.ofm_tiles) * 8 + xcd;
+    const int ntile = a.by_features ? (j / a.mtiles) * 8 + xcd : j % a.ofm_tiles;
+    if (ptile >= a.mtiles || ntile >= a.ofm_tiles) return;
     const uint32_t m0 = (uint32_t)ptile * BM;
 
     v4i acc[4][NT];
@@ -460,6 +472,7 @@ __global__ void __launch_bounds__(256) conv_mfma_kernel(MfmaArgs a)
             store_lds((d & 1) ^ 1, ra[(d + 1) % D], rb[(d + 1) % D]);
             load_global(ks + 1 + D, ra[(d + 1) % D], rb[(d + 1) % D]);
             lds_barrier();
+            step_fence();
         }
     }
     const int rest = a.ksteps - main_steps;  // < D steps left; their operands are already on the way
@@ -469,6 +482,7 @@ __global__ void __launch_bounds__(256) conv_mfma_kernel(MfmaArgs a)
             compute(d & 1);
             store_lds((d & 1) ^ 1, ra[(d + 1) % D], rb[(d + 1) % D]);
             lds_barrier();
+            step_fence();
         }
     }
 
@@ -493,6 +507,394 @@ __global__ void __launch_bounds__(256) conv_mfma_kernel(MfmaArgs a)
                 if (a.fe.fused) ev4 = *reinterpret_cast<const v4i*>((const int8_t*)a.eltw + ebase);
             finish_pixel<NT, EPI>(a, acc, nt, f0, valid, obase, ebase, sc, ev4, pp.b, pp.oy, pp.ox);
         }
+    }
+}
+
+// =====================================================================================================
+// Direct-activation tile kernel (long K, input with a zero border, feature slices a multiple of 4)
+// =====================================================================================================
+// Same output tile and weight stream as the LDS-staged kernel, but only the WEIGHTS go through LDS.  A wave
+// owns 16*NT pixels and ALL BN features of the tile, so its activation fragments are private to it: lane
+// (kq, l16) loads the 16 bytes of slice s0+kq of its pixel straight from global memory into the register
+// the MFMA reads (per K-step: one scalar tap offset + one per-lane 32-bit offset, no address arithmetic in
+// the vector unit).  Against the LDS-staged kernel this removes the activation store + load through LDS and
+// makes every weight fragment read from LDS feed NT matrix instructions: with BN = 64 a wave issues 4 LDS
+// reads per 4*NT MFMAs (the LDS-staged 64x64 tile: 5 reads per 4 MFMAs), so the LDS pipe stops being the bound.
+#define BDIR_PREFETCH_DISTANCE(loads) ((loads) <= 3 ? 8 : ((loads) <= 4 ? 6 : 4))
+
+template <int BN, int NT, int KG, int EPI>
+__global__ void __launch_bounds__(256 * KG) conv_bdir_kernel(MfmaArgs a)
+{
+    constexpr int MT = BN / 16;       // weight fragments (16 features each) per wave and K-step
+    constexpr int SPANS = BN / 64;
+    constexpr int WP = NT * 16;       // pixels per wave
+    constexpr int BM = 4 * WP;        // pixels per workgroup
+    constexpr int A_LOADS = BN / 64;  // 16-byte weight chunks per thread per K-step
+
+    // KG groups of four waves split the K-steps of the tile between them and add their partial sums through
+    // LDS at the end: long-K layers with few pixels get KG times as many waves per tile to hide latencies with.
+    const int t = threadIdx.x & 255;
+    const int lane = t & 63;
+    const int wave = __builtin_amdgcn_readfirstlane((threadIdx.x >> 6) & 3);
+    const int grp = KG == 1 ? 0 : __builtin_amdgcn_readfirstlane(threadIdx.x >> 8);
+    const int kq = lane >> 4;
+    const int l16 = lane & 15;
+
+    // same workgroup order as the LDS-staged kernel: a die takes every eighth tile of one kind
+    const int xcd = blockIdx.x & 7;
+    const int j = blockIdx.x >> 3;
+    const int ptile = a.by_features ? j % a.mtiles : (j / a.ofm_tiles) * 8 + xcd;
+    const int ntile = a.by_features ? (j / a.mtiles) * 8 + xcd : j % a.ofm_tiles;
+    if (ptile >= a.mtiles || ntile >= a.ofm_tiles) return;
+    const uint32_t m0 = (uint32_t)ptile * BM + (uint32_t)wave * WP;
+
+    v4i acc[MT][NT];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+        const int f = ntile * BN + (mt >> 2) * 64 + kq * 16 + (mt & 3) * 4;
+        v4i init = *reinterpret_cast<const v4i*>(a.acc_init + f);
+        if (grp != 0) init = v4i{0, 0, 0, 0};
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) acc[mt][nt] = init;
+    }
+    const v4i xm = {(int)a.xor_mask, (int)a.xor_mask, (int)a.xor_mask, (int)a.xor_mask};
+
+    extern __shared__ __align__(16) unsigned char smem[];
+    v4i* ldsA = reinterpret_cast<v4i*>(smem) + grp * (3 * 4 * BN);  // per group: [3][4 * BN]
+
+    // byte offset of (pixel, slice kq) of each of the lane's pixels; pixels past the end read pixel 0
+    uint32_t boff[NT];
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) {
+        const uint32_t m = m0 + nt * 16 + l16;
+        const PixelPos pp = pixel_pos(a, m < a.M ? m : 0);
+        boff[nt] = (uint32_t)(a.in_off + (int)pp.b * a.in_pb + ((int)pp.oy * a.sy - a.py) * a.in_py
+                              + ((int)pp.ox * a.sx - a.px) * 16 + kq * a.in_pf);
+    }
+    const int steps = a.ksteps / KG;  // the host pads the K-steps to a multiple of KG
+    const int step0 = grp * steps;
+    const v4i* wsrc = a.wpk + ((size_t)ntile * a.ksteps + step0) * (4 * BN) + t;
+
+    // look-ahead in K-steps for both operands
+    constexpr int D = BDIR_PREFETCH_DISTANCE(A_LOADS + NT);
+    constexpr int DA = D;
+    v4i ra[DA][A_LOADS], rb[D][NT];
+    auto load_a = [&](int ks, v4i (&xa)[A_LOADS]) {
+#pragma unroll
+        for (int q = 0; q < A_LOADS; ++q) xa[q] = wsrc[(size_t)ks * (4 * BN) + q * 256];
+    };
+    auto load_b = [&](int ks, v4i (&xb)[NT]) {
+        // the four k-chunks of a step are one tap and four consecutive slices: one uniform offset per step
+        const int8_t* base = a.in + scalar_table_load(a.ktab, (step0 + ks) * 4);
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) xb[nt] = *reinterpret_cast<const v4i*>(base + boff[nt]);
+    };
+    auto store_a = [&](int buf, const v4i (&xa)[A_LOADS]) {
+#pragma unroll
+        for (int q = 0; q < A_LOADS; ++q) ldsA[buf * 4 * BN + t + q * 256] = xa[q];
+    };
+    auto read_a = [&](int buf, v4i (&fa)[MT]) {
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) fa[mt] = ldsA[buf * 4 * BN + kq * BN + mt * 16 + l16];
+    };
+    auto mma = [&](const v4i (&fa)[MT], const v4i (&xb)[NT]) {
+        v4i fb[NT];
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) fb[nt] = xb[nt] ^ xm;
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt)
+                acc[mt][nt] = __builtin_amdgcn_mfma_i32_16x16x64_i8(fa[mt], fb[nt], acc[mt][nt], 0, 0, 0);
+    };
+
+    // Set d holds the operands of K-steps d, d+D, ...: activations stay in registers until multiplied; weights
+    // pass through a ring of three LDS buffers, written two steps ahead of their use, so that the fragments of
+    // step k+1 are read from LDS while the matrix instructions of step k run (one barrier per step).  The loop
+    // is branch-free; the weight stream and the tap table carry zero slack for the steps requested past the end.
+#pragma unroll
+    for (int u = 0; u < DA; ++u) load_a(u, ra[u]);
+#pragma unroll
+    for (int d = 0; d < D; ++d) load_b(d, rb[d]);
+    store_a(0, ra[0]);
+    store_a(1, ra[1]);
+    load_a(DA, ra[0]);
+    load_a(DA + 1, ra[1]);
+    lds_barrier();
+    v4i fa_cur[MT], fa_nxt[MT];
+    read_a(0, fa_cur);
+    int b1 = 1, b2 = 2, b0 = 0;  // ring positions of steps k+1, k+2, k
+    const int main_steps = (steps / DA) * DA;
+    for (int ks0 = 0; ks0 < main_steps; ks0 += DA) {
+#pragma unroll
+        for (int u = 0; u < DA; ++u) {
+            const int ks = ks0 + u;
+            read_a(b1, fa_nxt);
+            mma(fa_cur, rb[u % D]);
+            store_a(b2, ra[(u + 2) % DA]);
+            load_a(ks + 2 + DA, ra[(u + 2) % DA]);
+            load_b(ks + D, rb[u % D]);
+            lds_barrier();
+            step_fence();
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) fa_cur[mt] = fa_nxt[mt];
+            const int tmp = b0;
+            b0 = b1, b1 = b2, b2 = tmp;
+        }
+    }
+    const int rest = steps - main_steps;
+#pragma unroll
+    for (int u = 0; u < DA - 1; ++u) {
+        if (u < rest) {
+            read_a(b1, fa_nxt);
+            mma(fa_cur, rb[u % D]);
+            store_a(b2, ra[(u + 2) % DA]);
+            load_b(main_steps + u + D, rb[u % D]);
+            lds_barrier();
+            step_fence();
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) fa_cur[mt] = fa_nxt[mt];
+            const int tmp = b0;
+            b0 = b1, b1 = b2, b2 = tmp;
+        }
+    }
+
+    if constexpr (KG > 1) {
+        // partial sums of groups 1.. go to LDS as [group - 1][wave][register][lane]; group 0 adds them up
+        constexpr int REGS = MT * NT * 4;
+        int* part = reinterpret_cast<int*>(smem);
+        __syncthreads();  // every group is done with its weight buffers
+        if (grp != 0) {
+            int* dst = part + ((grp - 1) * 4 + wave) * REGS * 64 + lane;
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+                for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) dst[((mt * NT + nt) * 4 + i) * 64] = acc[mt][nt][i];
+        }
+        __syncthreads();
+        if (grp != 0) return;
+#pragma unroll
+        for (int g = 1; g < KG; ++g) {
+            const int* src = part + ((g - 1) * 4 + wave) * REGS * 64 + lane;
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+                for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) acc[mt][nt][i] += src[((mt * NT + nt) * 4 + i) * 64];
+        }
+    }
+
+    // ---- epilogue: per span of 64 features, lane (kq, l16) holds features f0 .. f0+15 of its pixels
+#pragma unroll
+    for (int sp = 0; sp < SPANS; ++sp) {
+        const int f0 = ntile * BN + sp * 64 + kq * 16;
+        if (f0 >= a.OFM) continue;
+        const int fs = f0 >> 4;
+        const int valid = a.OFM - f0;
+        LaneScales sc;
+        load_scales<EPI>(a, f0, sc);
+        const v4i(&acc_sp)[4][NT] = *reinterpret_cast<const v4i(*)[4][NT]>(&acc[sp * 4]);
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) {
+            const uint32_t m = m0 + nt * 16 + l16;
+            if (m < a.M) {
+                const PixelPos pp = pixel_pos(a, m);
+                const int obase = a.out_off + (int)pp.b * a.out_pb + fs * a.out_pf + (int)pp.oy * a.out_py + (int)pp.ox * 16;
+                const int ebase = a.el_off + (int)pp.b * a.el_pb + fs * a.el_pf + (int)(pp.oy * a.esy) * a.el_py
+                                  + (int)(pp.ox * a.esx) * 16;
+                v4i ev4 = {0, 0, 0, 0};
+                if constexpr (EPI == EPI_KIND_FUSED) ev4 = *reinterpret_cast<const v4i*>((const int8_t*)a.eltw + ebase);
+                else if constexpr (EPI == EPI_KIND_FAST)
+                    if (a.fe.fused) ev4 = *reinterpret_cast<const v4i*>((const int8_t*)a.eltw + ebase);
+                finish_pixel<NT, EPI>(a, acc_sp, nt, f0, valid, obase, ebase, sc, ev4, pp.b, pp.oy, pp.ox);
+            }
+        }
+    }
+}
+
+// =====================================================================================================
+// Weights-stationary kernel (input with a zero border, feature slices a multiple of 4, BN * K <= LDS)
+// =====================================================================================================
+// A persistent workgroup owns ONE tile of 64 output features and a contiguous range of pixel tiles.  It
+// copies its whole weight tile (64 x K bytes, already in fragment order) into LDS once; after that the K
+// loop has no barrier, no LDS store and no weight traffic from global memory: per K-step a wave reads its
+// four weight fragments from LDS (one step ahead of their use), multiplies them with activation fragments
+// that come straight from global memory D steps ahead of their use, and the look-ahead runs across pixel
+// tiles, so the activations (and the residual) of the next tile are in flight while the current tile is
+// requantised and stored.  Requantisation factors, accumulator start values and all pointers stay in
+// registers for the lifetime of the wave.  Tap offsets are walked with scalar counters (no table loads).
+// K-steps are padded by the host to a multiple of D with zero weights.
+struct TapWalk {
+    int sg, fx, fy, off;
+};
+__device__ __forceinline__ void tap_reset(TapWalk& w) { w.sg = 0, w.fx = 0, w.fy = 0, w.off = 0; }
+__device__ __forceinline__ void tap_advance(const MfmaArgs& a, TapWalk& w, int cb4)
+{
+    w.sg += 1;
+    w.off += 4 * a.in_pf;
+    if (w.sg == cb4) {
+        w.sg = 0;
+        w.off += a.tap_dx - cb4 * 4 * a.in_pf;
+        w.fx += 1;
+        if (w.fx == a.FX) {
+            w.fx = 0;
+            w.off += a.tap_dy - a.FX * a.tap_dx;
+            w.fy += 1;
+        }
+    }
+}
+
+template <int NT, int D, int EPI>
+__global__ void __launch_bounds__(256) conv_wsl_kernel(MfmaArgs a)
+{
+    constexpr int WP = NT * 16;  // pixels per wave and tile
+    const int t = threadIdx.x;
+    const int lane = t & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(t >> 6);
+    const int kq = lane >> 4;
+    const int l16 = lane & 15;
+
+    // partitions of one pixel range that differ in the feature tile get ids congruent modulo 8 and adjacent
+    // in time: they run on the same accelerator die and share the activations through its L2
+    const int xcd = blockIdx.x & 7;
+    const int j = blockIdx.x >> 3;
+    const int part = (j / a.ofm_tiles) * 8 + xcd;
+    const int ntile = j % a.ofm_tiles;
+    const int t_begin = part * a.wsl_tpp;
+    const int t_end = min(t_begin + a.wsl_tpp, a.mtiles);
+    if (t_begin >= t_end) return;
+
+    extern __shared__ __align__(16) unsigned char smem[];
+    v4i* ldsA = reinterpret_cast<v4i*>(smem);  // [ksteps][4][64]
+    {
+        const v4i* src = a.wpk + (size_t)ntile * a.ksteps * 256;
+        const int total = a.ksteps * 256;
+        for (int i = t; i < total; i += 8 * 256) {  // eight requests in flight per thread
+            v4i r[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) r[u] = src[min(i + u * 256, total - 1)];
+#pragma unroll
+            for (int u = 0; u < 8; ++u)
+                if (i + u * 256 < total) ldsA[i + u * 256] = r[u];
+        }
+    }
+
+    const int f0 = ntile * 64 + kq * 16;
+    const bool live = f0 < a.OFM;
+    const int fs = f0 >> 4;
+    const int valid = a.OFM - f0;
+    v4i init[4];
+#pragma unroll
+    for (int mt = 0; mt < 4; ++mt) init[mt] = *reinterpret_cast<const v4i*>(a.acc_init + f0 + mt * 4);
+    LaneScales sc;
+    if (live) load_scales<EPI>(a, f0, sc);
+    const v4i xm = {(int)a.xor_mask, (int)a.xor_mask, (int)a.xor_mask, (int)a.xor_mask};
+    const int cb4 = a.CB >> 2;
+
+    struct TileRefs {
+        uint32_t boff[NT];
+        int ob[NT], eb[NT];
+        PixelPos pos[NT];
+    };
+    auto setup = [&](int tile, TileRefs& r) {
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) {
+            const uint32_t m = ((uint32_t)tile * 4 + (uint32_t)wave) * WP + nt * 16 + l16;
+            const bool ok = tile < t_end && m < a.M;
+            const PixelPos pp = pixel_pos(a, ok ? m : 0);
+            r.boff[nt] = (uint32_t)(a.in_off + (int)pp.b * a.in_pb + ((int)pp.oy * a.sy - a.py) * a.in_py
+                                    + ((int)pp.ox * a.sx - a.px) * 16 + kq * a.in_pf);
+            const int o = a.out_off + (int)pp.b * a.out_pb + fs * a.out_pf + (int)pp.oy * a.out_py + (int)pp.ox * 16;
+            r.ob[nt] = ok && live ? o : -1;
+            r.eb[nt] = a.el_off + (int)pp.b * a.el_pb + fs * a.el_pf + (int)(pp.oy * a.esy) * a.el_py
+                       + (int)(pp.ox * a.esx) * 16;
+            if constexpr (EPI == EPI_KIND_GENERIC) r.pos[nt] = pp;
+        }
+    };
+    auto load_residual = [&](const TileRefs& r, v4i (&ev)[NT]) {
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) {
+            ev[nt] = v4i{0, 0, 0, 0};
+            if constexpr (EPI == EPI_KIND_FUSED) {
+                if (live) ev[nt] = *reinterpret_cast<const v4i*>((const int8_t*)a.eltw + r.eb[nt]);
+            } else if constexpr (EPI == EPI_KIND_FAST) {
+                if (a.fe.fused && live) ev[nt] = *reinterpret_cast<const v4i*>((const int8_t*)a.eltw + r.eb[nt]);
+            }
+        }
+    };
+    auto load_b = [&](const TileRefs& r, const TapWalk& w, v4i (&xb)[NT]) {
+        const int8_t* base = a.in + (w.fy < a.FY ? w.off : 0);  // padded K-steps read tap 0 (their weights are zero)
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) xb[nt] = *reinterpret_cast<const v4i*>(base + r.boff[nt]);
+    };
+    auto load_a = [&](int ks, v4i (&fa)[4]) {
+#pragma unroll
+        for (int mt = 0; mt < 4; ++mt) fa[mt] = ldsA[(ks * 4 + kq) * 64 + mt * 16 + l16];
+    };
+
+    TileRefs cur, nxt;
+    v4i rb[D][NT], ev_cur[NT], ev_nxt[NT], fa_cur[4], fa_nxt[4];
+    v4i acc[4][NT];
+    TapWalk walk;  // tap of the next activation request
+    setup(t_begin, cur);
+    tap_reset(walk);
+#pragma unroll
+    for (int d = 0; d < D; ++d) {
+        load_b(cur, walk, rb[d]);
+        tap_advance(a, walk, cb4);
+    }
+    load_residual(cur, ev_cur);
+    __syncthreads();  // the weight tile is in LDS
+    load_a(0, fa_cur);
+
+    auto step = [&](int ks, int d, const TileRefs& refill_from) {
+        load_a(ks + 1 < a.ksteps ? ks + 1 : 0, fa_nxt);
+        v4i fb[NT];
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) fb[nt] = rb[d][nt] ^ xm;
+#pragma unroll
+        for (int mt = 0; mt < 4; ++mt)
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt)
+                acc[mt][nt] = __builtin_amdgcn_mfma_i32_16x16x64_i8(fa_cur[mt], fb[nt], acc[mt][nt], 0, 0, 0);
+        load_b(refill_from, walk, rb[d]);
+        tap_advance(a, walk, cb4);
+#pragma unroll
+        for (int mt = 0; mt < 4; ++mt) fa_cur[mt] = fa_nxt[mt];
+        step_fence();
+    };
+
+    for (int tile = t_begin; tile < t_end; ++tile) {
+        setup(tile + 1, nxt);
+#pragma unroll
+        for (int mt = 0; mt < 4; ++mt)
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt) acc[mt][nt] = init[mt];
+        // chunks whose requests stay inside this tile
+        for (int ks0 = 0; ks0 + D < a.ksteps; ks0 += D) {
+#pragma unroll
+            for (int d = 0; d < D; ++d) step(ks0 + d, d, cur);
+        }
+        // last chunk: its requests are the first D steps of the next tile
+        tap_reset(walk);
+#pragma unroll
+        for (int d = 0; d < D; ++d) step(a.ksteps - D + d, d, nxt);
+        load_residual(nxt, ev_nxt);
+
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) {
+            if (cur.ob[nt] >= 0) {
+                PixelPos pp = PixelPos{0, 0, 0};
+                if constexpr (EPI == EPI_KIND_GENERIC) pp = cur.pos[nt];
+                finish_pixel<NT, EPI>(a, acc, nt, f0, valid, cur.ob[nt], cur.eb[nt], sc, ev_cur[nt], pp.b, pp.oy, pp.ox);
+            }
+        }
+        cur = nxt;
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) ev_cur[nt] = ev_nxt[nt];
     }
 }
 
@@ -623,6 +1025,55 @@ void launch_mfma_instance(hipStream_t s, const MfmaArgs& a, int grid, int lds, i
     case EPI_KIND_FAST: hipLaunchKernelGGL((conv_mfma_kernel<BM, BN, WP, CHECKED, EPI_KIND_FAST>), g, b, lds, s, a); break;
     default: hipLaunchKernelGGL((conv_mfma_kernel<BM, BN, WP, CHECKED, EPI_KIND_GENERIC>), g, b, lds, s, a); break;
     }
+}
+
+template <int BN, int NT, int KG>
+void launch_bdir_instance(hipStream_t s, const MfmaArgs& a, int grid, int lds, int epi)
+{
+    const dim3 g(grid), b(256 * KG);
+#define BDIR_LAUNCH(KIND)                                                                                       \
+    {                                                                                                           \
+        static bool allowed = false;                                                                            \
+        if (!allowed && lds > 48 * 1024) {                                                                      \
+            CHIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(&conv_bdir_kernel<BN, NT, KG, KIND>),  \
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));            \
+            allowed = true;                                                                                     \
+        }                                                                                                       \
+        hipLaunchKernelGGL((conv_bdir_kernel<BN, NT, KG, KIND>), g, b, lds, s, a);                              \
+    }
+    switch (epi) {
+    case EPI_KIND_RELU: BDIR_LAUNCH(EPI_KIND_RELU) break;
+    case EPI_KIND_FUSED: BDIR_LAUNCH(EPI_KIND_FUSED) break;
+    case EPI_KIND_LINEAR: BDIR_LAUNCH(EPI_KIND_LINEAR) break;
+    case EPI_KIND_FAST: BDIR_LAUNCH(EPI_KIND_FAST) break;
+    default: BDIR_LAUNCH(EPI_KIND_GENERIC) break;
+    }
+#undef BDIR_LAUNCH
+}
+
+template <int NT, int D>
+void launch_wsl_instance(hipStream_t s, const MfmaArgs& a, int grid, int lds, int epi)
+{
+    const dim3 g(grid), b(256);
+    // more than 64 KiB of dynamic LDS has to be allowed per kernel, once
+#define WSL_LAUNCH(KIND)                                                                                       \
+    {                                                                                                          \
+        static bool allowed = false;                                                                           \
+        if (!allowed) {                                                                                        \
+            CHIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(&conv_wsl_kernel<NT, D, KIND>),       \
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));           \
+            allowed = true;                                                                                    \
+        }                                                                                                      \
+        hipLaunchKernelGGL((conv_wsl_kernel<NT, D, KIND>), g, b, lds, s, a);                                   \
+    }
+    switch (epi) {
+    case EPI_KIND_RELU: WSL_LAUNCH(EPI_KIND_RELU) break;
+    case EPI_KIND_FUSED: WSL_LAUNCH(EPI_KIND_FUSED) break;
+    case EPI_KIND_LINEAR: WSL_LAUNCH(EPI_KIND_LINEAR) break;
+    case EPI_KIND_FAST: WSL_LAUNCH(EPI_KIND_FAST) break;
+    default: WSL_LAUNCH(EPI_KIND_GENERIC) break;
+    }
+#undef WSL_LAUNCH
 }
 
 template <int NT, int KS>

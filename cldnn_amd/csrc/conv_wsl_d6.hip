@@ -1,0 +1,17 @@
+// Instances of the weights-stationary kernel with an activation look-ahead of 6 K-step(s):
+// 16, 32 or 64 pixels per wave.
+#include "conv_mfma_kernel.h"
+
+namespace chip {
+
+void launch_wsl_d6(hipStream_t s, const MfmaArgs& a, int nt, int grid, int lds, int epi)
+{
+    switch (nt) {
+    case 1: launch_wsl_instance<1, 6>(s, a, grid, lds, epi); break;
+    case 2: launch_wsl_instance<2, 6>(s, a, grid, lds, epi); break;
+    case 4: launch_wsl_instance<4, 6>(s, a, grid, lds, epi); break;
+    default: throw error(CLDNN_HIP_INVALID_ARG, "weights-stationary kernel: pixels per wave must be 16, 32 or 64");
+    }
+}
+
+}  // namespace chip

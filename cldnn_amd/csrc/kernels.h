@@ -28,6 +28,7 @@ struct TileConfig {
     int tile_pixels;  // BM: output pixels per workgroup
     int tile_ofm;     // BN: output features per workgroup (multiple of 64)
     int wave_pixels;  // pixels per wave (4 waves: (BM / wave_pixels) * (BN / 64) == 4)
+    int kgroups = 1;  // groups of four waves that split K inside the workgroup (direct-activation kernel)
 };
 int tile_config_count();
 const TileConfig& tile_config(int i);
@@ -36,6 +37,12 @@ const TileConfig& tile_config(int i);
 struct MfmaPlan {
     int tile;            // row of the tile table
     int stream;          // 1: streaming kernel (no LDS), 0: LDS-staged tile kernel
+    int bdir;            // 1: direct-activation tile kernel (weights through LDS, activations into registers)
+    int by_features;     // 1: accelerator dies split the feature tiles (weights larger than activations)
+    int wsl;             // 1: weights-stationary persistent kernel (weight tile resident in LDS)
+    int wsl_depth;       // its activation look-ahead in K-steps
+    int wsl_parts;       // pixel-range partitions per feature tile (multiple of 8)
+    int wsl_tpp;         // pixel tiles per partition
     int checked;         // 1: taps bounds-checked per load, 0: input carries a sufficient zero border
     int cb;              // input feature slices of 16
     int kchunks;         // FY*FX*cb
@@ -50,7 +57,7 @@ struct MfmaPlan {
 };
 // table lookup: row of the tile table for a problem
 int mfma_choose(const ConvProblem& p, int cus);
-MfmaPlan mfma_plan(const ConvProblem& p, int tile);
+MfmaPlan mfma_plan(const ConvProblem& p, int tile, int cus);
 // host-side packing: weights [OFM][IFM][FY][FX] s8 -> MFMA operand stream, ktab -> per-kchunk tap table
 void mfma_pack_weights(const ConvProblem& p, const MfmaPlan& plan, const int8_t* w, int8_t* packed, int32_t* ktab);
 struct MfmaBuffers {

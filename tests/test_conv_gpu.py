@@ -142,8 +142,13 @@ def test_mfma_kernel_all_tiles(eng, shape, in_dt):
             kw = dict(stride=stride, pad=pad, out_dt="s8", act="relu", fmt="fs_b_yx_fsv16", in_pad=in_pad, tile=tile,
                       want_acc=True, want_info=True)
             ksteps = -(-(FY * FX * -(-IFM // 16)) // 4)
-            if tile and names[tile - 1].startswith(("stream", "shot")) and ((not border and pad != (0, 0)) or ksteps > 8):
+            no_border = not border and pad != (0, 0)
+            if tile and names[tile - 1].startswith("stream") and (no_border or ksteps > 8):
                 with pytest.raises(hip.HipError):  # needs constant tap offsets (zero border) and K <= 512
+                    hip.conv_forward(eng, x, w, bias, wqf, calib, **kw)
+                continue
+            if tile and names[tile - 1].startswith(("bdir", "wsl")) and (no_border or -(-IFM // 16) % 4 != 0):
+                with pytest.raises(hip.HipError):  # needs constant tap offsets and feature slices in fours
                     hip.conv_forward(eng, x, w, bias, wqf, calib, **kw)
                 continue
             go, ga, info = hip.conv_forward(eng, x, w, bias, wqf, calib, **kw)
@@ -154,6 +159,8 @@ def test_mfma_kernel_all_tiles(eng, shape, in_dt):
             assert_same(ref_o, go)
     assert any("conv_mfma" in n and "border" in n for n in seen)
     assert any("stream" in n for n in seen) == (-(-(FY * FX * -(-IFM // 16)) // 4) <= 8)
+    assert any("bdir" in n for n in seen) == (-(-IFM // 16) % 4 == 0)
+    assert any("wsl" in n for n in seen) == (-(-IFM // 16) % 4 == 0)
     if pad != (0, 0):
         assert any("checked" in n for n in seen)
 
@@ -168,11 +175,13 @@ def test_mfma_epilogue_variants(eng, out_dt, act):
     calib = np.full(96, 127 / 6, np.float32) * r.uniform(0.9, 1.1, 96).astype(np.float32)
     calib[::7] *= -1  # negative scales: relu cannot be folded into the final clamp
     kw = dict(stride=(1, 1), pad=(1, 1), out_dt=out_dt, act=act[0], act_m=act[1], act_n=act[2], iqf=0.75)
-    (ro, ra), (go, ga, info) = both(eng, x, w, bias, wqf, calib, fmt="fs_b_yx_fsv16", **kw)
-    # the short epilogue covers int8 outputs with none / relu / clamp; everything else takes the long form
-    assert (b"generic" in info.kernel_name) == (out_dt == "f32" or act[0] == "relu_slope")
-    np.testing.assert_array_equal(ga, ra)
-    assert_same(ro, go)
+    for tile, in_pad in ((0, (0, 0)), (0, (1, 1)), (10, (1, 1)), (13, (1, 1)), (15, (1, 1)), (16, (1, 1)), (18, (1, 1)), (19, (1, 1)), (20, (1, 1))):  # table's choice, direct-activation, weights-stationary and split-K rows
+        (ro, ra), (go, ga, info) = both(eng, x, w, bias, wqf, calib, fmt="fs_b_yx_fsv16", tile=tile, in_pad=in_pad, **kw)
+        # the short epilogue covers int8 outputs with none / relu / clamp; everything else takes the long form
+        assert (b"generic" in info.kernel_name) == (out_dt == "f32" or act[0] == "relu_slope")
+        assert tile == 0 or b"bdir" in info.kernel_name or b"wsl" in info.kernel_name
+        np.testing.assert_array_equal(ga, ra)
+        assert_same(ro, go)
 
 
 def test_mfma_f32_bias_added_after_dequantisation(eng):
@@ -204,7 +213,7 @@ def test_mfma_fused_eltwise(eng, fast, eltw_dt):
     ecal = r.uniform(0.3, 1.2, 256).astype(np.float32)
     kw = dict(out_dt="s8", act="none", eltw=e, eltw_act="relu", eltw_calib=ecal,
               non_conv_scale=1.0 if fast else 0.5)
-    for tile in (0, 1, 6, 7, 8):
+    for tile in [0] + tiles():
         (ro, ra), (go, ga, info) = both(eng, x, w, bias, wqf, calib, fmt="fs_b_yx_fsv16", tile=tile, **kw)
         assert (b"fast" in info.kernel_name) == fast
         np.testing.assert_array_equal(ga, ra)
