@@ -22,6 +22,7 @@ struct cldnn_hip_conv_s {
     // device allocations
     void* w_raw = nullptr;    // dense weights (reference kernel)
     void* w_packed = nullptr; // MFMA / depthwise operand stream
+    void* w_masked = nullptr; // depthwise 3x3 kernel: one weight byte per dword
     void* ktab = nullptr;
     void* acc_init = nullptr;      // int32: offset correction + int32 bias
     void* acc_init_raw = nullptr;  // int32: offset correction only (accumulator probe)
@@ -194,13 +195,20 @@ void build(cldnn_hip_conv c, const void* weights, const void* bias, const float*
     // ---- accumulator start values: 128*sum(w) for u8 on the signed matrix cores, plus an int32 bias
     const int8_t* w8 = (const int8_t*)weights;
     std::vector<int32_t> init(ofm_pad, 0), init_raw(ofm_pad, 0);
-    const bool xor_u8 = impl == CLDNN_HIP_IMPL_MFMA && p.in_dt == CLDNN_HIP_U8;
+    // can the short epilogue reproduce the long one?  (an int32 bias is folded into the start values, a float one is not)
+    {
+        Epilogue probe = e;
+        probe.bias = bias && d.bias_dtype == CLDNN_HIP_F32 ? (const void*)weights : nullptr;
+        c->fast = mfma_fast_epilogue(p, probe, calib_on ? calib : nullptr, eltw_calib, wqf, &c->fe);
+    }
+    const bool dw_fast = impl == CLDNN_HIP_IMPL_DEPTHWISE && dw_fast_applies(p, c->fast);
+    const bool xor_u8 = (impl == CLDNN_HIP_IMPL_MFMA || dw_fast) && p.in_dt == CLDNN_HIP_U8;
     for (int f = 0; f < p.OFM; ++f) {
         int64_t s = 0;
         if (xor_u8)
             for (size_t i = 0; i < (size_t)ifm_g * p.FY * p.FX; ++i) s += w8[(size_t)f * ifm_g * p.FY * p.FX + i];
         uint32_t v = (uint32_t)(int32_t)(128 * s);
-        init_raw[f] = (int32_t)v;
+        init_raw[f] = impl == CLDNN_HIP_IMPL_MFMA ? (int32_t)v : 0;  // the accumulator probe of the depthwise path never flips signs
         if (bias && d.bias_dtype == CLDNN_HIP_I32 && !e.bias_after) v += (uint32_t)((const int32_t*)bias)[f];
         init[f] = (int32_t)v;
     }
@@ -223,7 +231,6 @@ void build(cldnn_hip_conv c, const void* weights, const void* bias, const float*
         mfma_pack_weights(p, c->mplan, w8, packed.data(), ktab.data());
         c->w_packed = upload(c, packed.data(), packed.size());
         c->ktab = upload(c, ktab.data(), ktab.size() * 4);
-        c->fast = mfma_fast_epilogue(p, e, calib_on ? calib : nullptr, eltw_calib, wqf, &c->fe);
         const TileConfig& tc = tile_config(tile);
         inf.tile_index = tile, inf.tile_pixels = tc.tile_pixels, inf.tile_ofm = tc.tile_ofm;
         inf.grid = c->mplan.grid, inf.block = 256, inf.lds_bytes = c->mplan.lds_bytes;
@@ -234,8 +241,14 @@ void build(cldnn_hip_conv c, const void* weights, const void* bias, const float*
         std::vector<int8_t> packed(c->dplan.packed_bytes);
         dw_pack_weights(p, w8, packed.data());
         c->w_packed = upload(c, packed.data(), packed.size());
-        inf.grid = c->dplan.grid * ((p.OFM + 15) / 16), inf.block = c->dplan.block, inf.lds_bytes = p.FY * p.FX * 16;
-        std::snprintf(inf.kernel_name, sizeof(inf.kernel_name), "conv_dw_kernel<%s>", p.in_dt == CLDNN_HIP_U8 ? "u8" : "s8");
+        if (dw_fast) {
+            std::vector<int32_t> masked(c->dplan.mask_bytes / 4);
+            dw_mask_weights(p, w8, masked.data());
+            c->w_masked = upload(c, masked.data(), c->dplan.mask_bytes);
+        }
+        inf.grid = c->dplan.grid * ((p.OFM + 15) / 16), inf.block = c->dplan.block, inf.lds_bytes = dw_fast ? 0 : p.FY * p.FX * 16;
+        std::snprintf(inf.kernel_name, sizeof(inf.kernel_name), "%s<%s>", dw_fast ? "conv_dw3x3_kernel" : "conv_dw_kernel",
+                      p.in_dt == CLDNN_HIP_U8 ? "u8" : "s8");
     }
 }
 
@@ -312,8 +325,9 @@ static void run(cldnn_hip_conv c, const void* in, void* out, const void* eltw, i
         break;
     }
     case CLDNN_HIP_IMPL_DEPTHWISE:
-        launch_conv_dw(s, p, c->dplan, (const int8_t*)c->w_packed,
-                       (const int32_t*)(raw ? c->acc_init_raw : c->acc_init), c->epi, in, eltw, out, raw);
+        launch_conv_dw(s, p, c->dplan, (const int8_t*)c->w_packed, (const int32_t*)c->w_masked,
+                       (const int32_t*)(raw ? c->acc_init_raw : c->acc_init), c->epi, c->fast ? &c->fe : nullptr, in, eltw, out,
+                       raw);
         break;
     default: throw error(CLDNN_HIP_ERROR, "convolution without an implementation");
     }

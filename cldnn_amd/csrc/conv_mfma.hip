@@ -58,7 +58,9 @@ static const tile_launcher g_launch[] = {launch_mfma_tile_0, launch_mfma_tile_1,
 int tile_config_count() { return (int)(sizeof(g_tiles) / sizeof(g_tiles[0])); }
 const TileConfig& tile_config(int i) { return g_tiles[i]; }
 
-static FastDiv make_div(uint32_t d)
+FastDiv make_fast_div(uint32_t d);
+static FastDiv make_div(uint32_t d) { return make_fast_div(d); }
+FastDiv make_fast_div(uint32_t d)
 {
     FastDiv f{};
     if (d <= 1) {
@@ -74,6 +76,8 @@ static FastDiv make_div(uint32_t d)
 }
 
 // does the input buffer carry a zero border that covers every tap of every output pixel?
+static bool border_covers(const ConvProblem& p);
+bool conv_border_covers(const ConvProblem& p) { return border_covers(p); }
 static bool border_covers(const ConvProblem& p)
 {
     const cldnn_hip_tensor& t = p.in_t;
@@ -122,7 +126,8 @@ int mfma_choose(const ConvProblem& p, int cus)
     const int stream_row = stream_waves >= 4ll * cus ? ROW_STREAM_P32 : ROW_STREAM_P16;
 
     if (ksteps <= 2 || !direct) {
-        // one or two K-steps: bound by HBM bandwidth, one memory round trip per wave
+        // one or two K-steps (or a first layer with three input features): bound by HBM bandwidth
+        if (!direct && ksteps >= 3 && m >= 500000) return choose_lds_tile(p, m, cus);  // VGG conv1
         if (stream_fits) return stream_row;
         return choose_lds_tile(p, m, cus);
     }
@@ -136,11 +141,16 @@ int mfma_choose(const ConvProblem& p, int cus)
         return stream_fits ? stream_row : ROW_BDIR_P64_F64;
     }
     // long K
-    if (ksteps <= 40 && m >= 50000 && p.OFM <= 64) return ROW_WSL_P128;          // 3x3 at 56x56, 64 features
-    if (m >= 100000 && p.OFM >= 128) return ROW_BDIR_P256_F128;                  // VGG-sized layers
-    if (m >= 16384) return p.OFM > 64 || m >= 50000 ? ROW_BDIR_P128_F64 : ROW_BDIR_P64_F64;
-    if (m >= 4096) return ROW_BDIR_P64_F64;                                      // 14x14
-    if (ksteps >= 32) return ROW_BDIR_K2_P64_F64;                                // 7x7 with K >= 2048: split K in the workgroup
+    if (m >= 50000) {
+        if (ksteps <= 18) return ksteps <= 9 && p.OFM <= 128 ? ROW_WSL_P128 : ROW_WSL_P64;  // 3x3 at 56x56 .. 112x112
+        return p.OFM >= 128 ? ROW_P256_F128 : ROW_BDIR_P256_F64;
+    }
+    if (m >= 8192) {
+        if (p.OFM >= 512) return ksteps >= 64 ? ROW_BDIR_P128_F128 : ROW_BDIR_P256_F64;
+        return ROW_BDIR_P128_F64;                                  // 3x3 at 28x28
+    }
+    if (m >= 4096) return ROW_BDIR_P64_F64;                        // 14x14
+    if (ksteps >= 32) return m >= 2048 ? ROW_BDIR_K2_P128_F64 : ROW_BDIR_K2_P64_F64;  // few pixels, K >= 2048: split K
     if (p.OFM >= 1024) return ROW_P128_F128;
     return ROW_BDIR_P64_F64;
 }

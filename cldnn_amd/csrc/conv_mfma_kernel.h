@@ -40,6 +40,8 @@ struct FastDiv {
     __device__ __forceinline__ uint32_t div(uint32_t n) const { return one ? n : (__umulhi(n, mul) >> shift); }
 };
 
+FastDiv make_fast_div(uint32_t d);  // host
+
 struct MfmaArgs {
     const int8_t* in;
     const v4i* wpk;
@@ -124,8 +126,8 @@ __device__ __forceinline__ int pack_signed(const float* v)
 // (the bounds are integers), round-half-away is trunc(x + copysign(0.49999997f, x)), and
 // max(0, x) * s becomes clamp(x * s, 0, hi) when s >= 0.  The truncating float->int conversion
 // completes the rounding.
-template <int NT, int EPI>
-__device__ __forceinline__ v4i epilogue_fast16(const MfmaArgs& a, const v4i (&acc)[4][NT], int nt, const float (&wq)[16],
+template <int NT, int EPI, class Args>
+__device__ __forceinline__ v4i epilogue_fast16(const Args& a, const v4i (&acc)[4][NT], int nt, const float (&wq)[16],
                                                const float (&cal)[16], const float (&ecal)[16], const v4i& ev4,
                                                int valid)
 {
@@ -265,8 +267,8 @@ struct LaneScales {
     float wq[16], cal[16], ecal[16];
 };
 
-template <int EPI>
-__device__ __forceinline__ void load_scales(const MfmaArgs& a, int f0, LaneScales& sc)
+template <int EPI, class Args>
+__device__ __forceinline__ void load_scales(const Args& a, int f0, LaneScales& sc)
 {
     if constexpr (EPI == EPI_KIND_RELU || EPI == EPI_KIND_FUSED || EPI == EPI_KIND_LINEAR) {
         // these kinds are only chosen when the vectors they read exist

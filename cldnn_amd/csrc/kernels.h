@@ -92,10 +92,15 @@ void launch_conv_mfma(hipStream_t s, const ConvProblem& p, const MfmaPlan& plan,
 struct DwPlan {
     int grid, block;
     size_t packed_bytes;
+    size_t mask_bytes;  // masked weight dwords of the 3x3 kernel
 };
 DwPlan dw_plan(const ConvProblem& p);
 void dw_pack_weights(const ConvProblem& p, const int8_t* w, int8_t* packed);
-void launch_conv_dw(hipStream_t s, const ConvProblem& p, const DwPlan& plan, const int8_t* packed, const int32_t* acc_init,
-                    const Epilogue& epi, const void* in, const void* eltw, void* out, int32_t* raw);
+void dw_mask_weights(const ConvProblem& p, const int8_t* w, int32_t* masked);
+bool dw_fast_applies(const ConvProblem& p, bool fast_epilogue);
+bool conv_border_covers(const ConvProblem& p);
+void launch_conv_dw(hipStream_t s, const ConvProblem& p, const DwPlan& plan, const int8_t* packed, const int32_t* masked,
+                    const int32_t* acc_init, const Epilogue& epi, const FastEpi* fast, const void* in, const void* eltw,
+                    void* out, int32_t* raw);
 
 }  // namespace chip

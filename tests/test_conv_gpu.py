@@ -256,9 +256,18 @@ def test_depthwise_kernel(eng, shape, in_dt):
     calib = np.full(C, 127 / 6, np.float32)
     kw = dict(stride=(s, s), pad=(p, p), groups=C, out_dt="s8", act="clamp", act_m=0.0, act_n=6.0)
     (ro, ra), (go, ga, info) = both(eng, x, w, bias, wqf, calib, fmt="fs_b_yx_fsv16", **kw)
-    assert info.impl == hip.IMPL_DEPTHWISE
+    assert info.impl == hip.IMPL_DEPTHWISE and b"conv_dw_kernel" in info.kernel_name
     np.testing.assert_array_equal(ga, ra)
     assert_same(ro, go)
+    # with a physical zero border the 3x3 layers take the dot-product kernel; relu6, relu, no activation, u8 output
+    variants = [kw, dict(kw, act="relu", act_m=0.0, act_n=0.0), dict(kw, act="none", out_dt="u8"), dict(kw, out_dt="u8")]
+    for i, v in enumerate(variants):
+        wq = wqf if i != 1 else np.ones(C, np.float32)
+        cal = calib if i != 1 else (40.0 / (F * 147.4 * 73.3) * r.uniform(0.5, 2, C)).astype(np.float32)
+        (ro, ra), (go, ga, info) = both(eng, x, w, bias, wq, cal, fmt="fs_b_yx_fsv16", in_pad=(p, p + 1), out_pad=(0, 1), **v)
+        assert (b"conv_dw3x3_kernel" in info.kernel_name) == (F == 3), info.kernel_name
+        np.testing.assert_array_equal(ga, ra)
+        assert_same(ro, go)
     # the layout-agnostic kernel must agree as well (grouped path, one launch)
     (ro2, _), (go2, _, info2) = both(eng, x, w, bias, wqf, calib, fmt="bfyx", acc=True, **kw)
     assert info2.impl == hip.IMPL_REF
