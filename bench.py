@@ -61,7 +61,9 @@ def build_stack(eng, layers, batch, fuse_residual, seed=1337, tile=0, in_dt=np.u
             L.calib = np.full(ofm, 127.0 / 6.0, np.float32)
         else:
             kw.update(act=act)
-        L.xin = hip.upload(eng, L.x, "fs_b_yx_fsv16", (l["pad"], l["pad"]))  # zero border as wide as the padding
+        # zero border as wide as the padding; a first layer (3 input features) takes b_fs_yx_fsv4
+        first = ifm <= 4 and g == 1
+        L.xin = hip.upload(eng, L.x, "b_fs_yx_fsv4" if first else "fs_b_yx_fsv16", (l["pad"], l["pad"]))
         L.ein = None
         if L.fused:
             L.eltw = r.integers(-128, 128, (batch, ofm, ohw, ohw), dtype=np.int16).astype(np.int8)
@@ -69,7 +71,9 @@ def build_stack(eng, layers, batch, fuse_residual, seed=1337, tile=0, in_dt=np.u
             L.ein = hip.upload(eng, L.eltw, "fs_b_yx_fsv16")
             kw.update(act="none", eltw_t=L.ein.tensor, eltw_act="relu", has_eltw_calib=True)
         L.kw = kw
-        L.desc = hip.conv_desc(L.xin.tensor, L.w.shape, "s8", tile=tile, **kw)
+        if first:
+            kw["out_fmt"] = hip.FS_B_YX_FSV16
+        L.desc = hip.conv_desc(L.xin.tensor, L.w.shape, "s8", tile=0 if first else tile, **kw)
         try:
             L.conv = hip.Conv(eng, L.desc, L.w, L.bias, L.wqf, L.calib, L.ecal)
         except hip.HipError:

@@ -147,15 +147,20 @@ void build(cldnn_hip_conv c, const void* weights, const void* bias, const float*
                          && (!d.fused || p.eltw_t.format == CLDNN_HIP_FMT_FS_B_YX_FSV16);
     const bool int_path = in8 && p.w_dt == CLDNN_HIP_S8 && e.mode != MODE_NAT;
     const bool depthwise = d.groups > 1 && d.groups == d.ifm && d.groups == d.ofm;
+    // first layers: at most 4 input features in b_fs_yx_fsv4 (4 horizontal taps x 4 features = one 16-byte fragment)
+    const bool stem = d.input.format == CLDNN_HIP_FMT_B_FS_YX_FSV4 && d.output.format == CLDNN_HIP_FMT_FS_B_YX_FSV16
+                      && (!d.fused || p.eltw_t.format == CLDNN_HIP_FMT_FS_B_YX_FSV16) && d.ifm <= 4 && d.groups == 1
+                      && d.dilation_x == 1 && conv_border_covers(p) && (p.FY * ((p.FX + 3) / 4) + 3) / 4 <= 8;
     int impl = d.impl;
     if (impl == CLDNN_HIP_IMPL_AUTO) {
-        if (blocked && int_path && d.groups == 1) impl = CLDNN_HIP_IMPL_MFMA;
+        if ((blocked || stem) && int_path && d.groups == 1) impl = CLDNN_HIP_IMPL_MFMA;
         else if (blocked && int_path && depthwise) impl = CLDNN_HIP_IMPL_DEPTHWISE;
         else impl = CLDNN_HIP_IMPL_REF;
     }
     if (impl == CLDNN_HIP_IMPL_MFMA)
-        CHIP_REQUIRE(blocked && int_path && d.groups == 1, CLDNN_HIP_UNSUPPORTED_FORMAT,
-                     "the MFMA kernel needs int8 data in fs_b_yx_fsv16, quantisation and groups == 1");
+        CHIP_REQUIRE((blocked || stem) && int_path && d.groups == 1, CLDNN_HIP_UNSUPPORTED_FORMAT,
+                     "the MFMA kernel needs int8 data in fs_b_yx_fsv16 (first layers: bordered b_fs_yx_fsv4 input), "
+                     "quantisation and groups == 1");
     if (impl == CLDNN_HIP_IMPL_DEPTHWISE)
         CHIP_REQUIRE(blocked && int_path && depthwise, CLDNN_HIP_UNSUPPORTED_FORMAT,
                      "the depthwise kernel needs int8 data in fs_b_yx_fsv16, quantisation and groups == features");

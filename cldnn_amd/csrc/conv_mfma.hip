@@ -48,8 +48,11 @@ static const TileConfig g_tiles[] = {
     {"bdir_k2_p64_f64", 64, 64, 16, 2},
     {"bdir_k4_p64_f64", 64, 64, 16, 4},
     {"bdir_k2_p128_f64", 128, 64, 32, 2},
+    // first layers (at most 4 input features) read b_fs_yx_fsv4: a 16-byte fragment is 4 horizontal taps x 4 features;
+    // streaming kernel
+    {"stem_p32", 32, 64, 32},
 };
-enum { FIRST_STREAM_ROW = 6, FIRST_BDIR_ROW = 8, FIRST_WSL_ROW = 14, FIRST_BDIRK_ROW = 17 };
+enum { FIRST_STREAM_ROW = 6, FIRST_BDIR_ROW = 8, FIRST_WSL_ROW = 14, FIRST_BDIRK_ROW = 17, STEM_ROW = 20 };
 enum { WSL_MAX_LDS = 160 * 1024 };
 enum { MFMA_SLACK_STEPS = 40 };  // >= weight look-ahead + activation look-ahead + 3
 static const tile_launcher g_launch[] = {launch_mfma_tile_0, launch_mfma_tile_1, launch_mfma_tile_2, launch_mfma_tile_3,
@@ -94,7 +97,7 @@ enum {
     ROW_STREAM_P16 = 6, ROW_STREAM_P32 = 7,
     ROW_BDIR_P64_F64 = 8, ROW_BDIR_P128_F64 = 9, ROW_BDIR_P256_F64 = 10, ROW_BDIR_P64_F128 = 11, ROW_BDIR_P128_F128 = 12,
     ROW_BDIR_P256_F128 = 13, ROW_WSL_P64 = 14, ROW_WSL_P128 = 15, ROW_WSL_P256 = 16,
-    ROW_BDIR_K2_P64_F64 = 17, ROW_BDIR_K4_P64_F64 = 18, ROW_BDIR_K2_P128_F64 = 19
+    ROW_BDIR_K2_P64_F64 = 17, ROW_BDIR_K4_P64_F64 = 18, ROW_BDIR_K2_P128_F64 = 19, ROW_STEM_P32 = 20
 };
 
 static int choose_lds_tile(const ConvProblem& p, int64_t m, int cus)
@@ -116,6 +119,7 @@ static int choose_lds_tile(const ConvProblem& p, int64_t m, int cus)
 
 int mfma_choose(const ConvProblem& p, int cus)
 {
+    if (p.in_t.format == CLDNN_HIP_FMT_B_FS_YX_FSV4) return ROW_STEM_P32;
     const int64_t m = (int64_t)p.B * p.OH * p.OW;
     const int cb = (p.IFM + 15) / 16;
     const int ksteps = (p.FY * p.FX * cb + 3) / 4;
@@ -182,15 +186,20 @@ MfmaPlan mfma_plan(const ConvProblem& p, int tile, int cus)
     MfmaPlan pl{};
     pl.tile = tile;
     pl.checked = border_covers(p) ? 0 : 1;
-    pl.stream = tile >= FIRST_STREAM_ROW && tile < FIRST_BDIR_ROW ? 1 : 0;
-    pl.bdir = (tile >= FIRST_BDIR_ROW && tile < FIRST_WSL_ROW) || tile >= FIRST_BDIRK_ROW ? 1 : 0;
+    pl.stem = tile == STEM_ROW ? 1 : 0;
+    CHIP_REQUIRE(pl.stem == (p.in_t.format == CLDNN_HIP_FMT_B_FS_YX_FSV4 ? 1 : 0), CLDNN_HIP_INVALID_ARG,
+                 "b_fs_yx_fsv4 input goes with the first-layer row of the tile table and only with it");
+    pl.stream = (tile >= FIRST_STREAM_ROW && tile < FIRST_BDIR_ROW) || pl.stem ? 1 : 0;
+    pl.bdir = ((tile >= FIRST_BDIR_ROW && tile < FIRST_WSL_ROW) || tile >= FIRST_BDIRK_ROW) && !pl.stem ? 1 : 0;
     pl.wsl = tile >= FIRST_WSL_ROW && tile < FIRST_BDIRK_ROW ? 1 : 0;
     CHIP_REQUIRE(!(pl.stream && pl.checked), CLDNN_HIP_INVALID_ARG,
                  "the streaming kernel needs an input whose physical zero border covers the convolution's padding");
     pl.cb = (p.IFM + 15) / 16;
+    if (pl.stem) CHIP_REQUIRE(p.IFM <= 4 && p.dx == 1 && p.groups == 1, CLDNN_HIP_INVALID_ARG,
+                              "the first-layer kernel takes at most 4 input features and no horizontal dilation");
     CHIP_REQUIRE(!(pl.bdir || pl.wsl) || (!pl.checked && pl.cb % 4 == 0), CLDNN_HIP_INVALID_ARG,
                  "the direct-activation kernels need a zero border covering the padding and input features in multiples of 64");
-    pl.kchunks = p.FY * p.FX * pl.cb;
+    pl.kchunks = pl.stem ? p.FY * ((p.FX + 3) / 4) : p.FY * p.FX * pl.cb;  // first layer: a chunk is 4 horizontal taps
     pl.ksteps = (pl.kchunks + 3) / 4;
     if (pl.stream) {
         CHIP_REQUIRE(pl.ksteps <= 8, CLDNN_HIP_INVALID_ARG, "the streaming kernel handles at most 8 K-steps (K <= 512)");
@@ -245,6 +254,24 @@ void mfma_pack_weights(const ConvProblem& p, const MfmaPlan& pl, const int8_t* w
     const TileConfig& tc = g_tiles[pl.tile];
     const int BN = tc.tile_ofm;
     std::memset(packed, 0, pl.packed_bytes);
+    auto row_of = [&](int f) {
+        const int fl = f % BN, span = fl / 64, o = fl % 64;
+        return span * 64 + ((o % 16) / 4) * 16 + (o / 16) * 4 + (o % 4);  // permuted row inside the span
+    };
+    if (pl.stem) {
+        // k-chunk = (filter row, group of 4 horizontal taps); byte = (tap in group) * 4 + feature; absent taps / features stay zero
+        const int fxg = (p.FX + 3) / 4;
+        for (int kc = 0; kc < (pl.ksteps + MFMA_SLACK_STEPS) * 4; ++kc) ktab[kc] = 0;  // offsets are computed in the kernel
+        for (int f = 0; f < p.OFM; ++f)
+            for (int fy = 0; fy < p.FY; ++fy)
+                for (int fx = 0; fx < p.FX; ++fx)
+                    for (int ch = 0; ch < p.IFM; ++ch) {
+                        const int kc = fy * fxg + fx / 4, ks = kc / 4, kq = kc % 4;
+                        packed[((((size_t)(f / BN) * pl.ksteps + ks) * 4 + kq) * BN + row_of(f)) * 16 + (fx % 4) * 4 + ch] =
+                            w[(((size_t)f * p.IFM + ch) * p.FY + fy) * p.FX + fx];
+                    }
+        return;
+    }
     // k-chunk order: tap-major, feature slice minor
     for (int kc = 0; kc < (pl.ksteps + MFMA_SLACK_STEPS) * 4; ++kc) {
         if (kc >= pl.kchunks) {
@@ -257,9 +284,8 @@ void mfma_pack_weights(const ConvProblem& p, const MfmaPlan& pl, const int8_t* w
         else ktab[kc] = (int32_t)(cb * p.in_p.pf + fyd * p.in_p.py + fxd * 16);
     }
     for (int f = 0; f < p.OFM; ++f) {
-        const int nt = f / BN, fl = f % BN;
-        const int span = fl / 64, o = fl % 64;
-        const int row = span * 64 + ((o % 16) / 4) * 16 + (o / 16) * 4 + (o % 4);  // permuted row inside the span
+        const int nt = f / BN;
+        const int row = row_of(f);
         for (int kc = 0; kc < pl.kchunks; ++kc) {
             const int tap = kc / pl.cb, cb = kc % pl.cb;
             const int ks = kc / 4, kq = kc % 4;
@@ -361,12 +387,21 @@ void launch_conv_mfma(hipStream_t s, const ConvProblem& p, const MfmaPlan& pl, c
     a.div_cb = make_div((uint32_t)pl.cb), a.div_fx = make_div((uint32_t)p.FX);
     a.wsl_parts = pl.wsl_parts, a.wsl_tpp = pl.wsl_tpp, a.FY = p.FY;
     a.by_features = pl.by_features;
+    a.px_bytes = 16;
+    if (pl.stem) {
+        // the streaming kernel's tap arithmetic with "taps" = groups of 4 horizontal taps, 16 bytes apart
+        a.px_bytes = 4;
+        a.CB = 1, a.FX = (p.FX + 3) / 4, a.kchunks = pl.kchunks;
+        a.tap_dx = 16;
+        a.div_cb = make_div(1u), a.div_fx = make_div((uint32_t)a.FX);
+        a.linear = 0;
+    }
     {
         // dense tensors and a 1x1 / stride-1 convolution: pixel m sits at byte m * 16 of every feature slice
         auto dense = [](const cldnn_hip_tensor& t) {
             return t.pad_lo_y == 0 && t.pad_lo_x == 0 && t.pad_hi_y == 0 && t.pad_hi_x == 0;
         };
-        a.linear = p.FY == 1 && p.FX == 1 && p.sy == 1 && p.sx == 1 && p.py == 0 && p.px == 0 && dense(p.in_t)
+        a.linear = !pl.stem && p.FY == 1 && p.FX == 1 && p.sy == 1 && p.sx == 1 && p.py == 0 && p.px == 0 && dense(p.in_t)
                    && dense(p.out_t) && p.out_dt != CLDNN_HIP_F32
                    && (!epi.fused || (dense(p.eltw_t) && p.esy == 1 && p.esx == 1 && p.eltw_t.y == p.OH && p.eltw_t.x == p.OW));
     }

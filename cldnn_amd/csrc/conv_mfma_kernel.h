@@ -65,6 +65,8 @@ struct MfmaArgs {
     int32_t wsl_parts, wsl_tpp, FY;
     // 1: the eight accelerator dies split the FEATURE tiles between them (weights are the larger operand)
     int32_t by_features;
+    // bytes per pixel of one input slice: 16 (fs_b_yx_fsv16) or 4 (b_fs_yx_fsv4, first layers; streaming kernel only)
+    int32_t px_bytes;
     FastDiv div_cb, div_fx;
     uint32_t xor_mask;  // 0x80808080 for u8 activations, 0 for s8
     FastEpi fe;
@@ -959,7 +961,7 @@ __global__ void __launch_bounds__(256) conv_stream_kernel(MfmaArgs a)
         } else {
             const PixelPos pp = pixel_pos(a, mm);
             pos[nt] = pp;
-            pix = a.in_off + (int)pp.b * a.in_pb + ((int)pp.oy * a.sy - a.py) * a.in_py + ((int)pp.ox * a.sx - a.px) * 16;
+            pix = a.in_off + (int)pp.b * a.in_pb + ((int)pp.oy * a.sy - a.py) * a.in_py + ((int)pp.ox * a.sx - a.px) * a.px_bytes;
             o = a.out_off + (int)pp.b * a.out_pb + fs * a.out_pf + (int)pp.oy * a.out_py + (int)pp.ox * 16;
             e = a.el_off + (int)pp.b * a.el_pb + fs * a.el_pf + (int)(pp.oy * a.esy) * a.el_py + (int)(pp.ox * a.esx) * 16;
         }

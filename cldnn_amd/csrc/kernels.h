@@ -38,6 +38,7 @@ struct MfmaPlan {
     int tile;            // row of the tile table
     int stream;          // 1: streaming kernel (no LDS), 0: LDS-staged tile kernel
     int bdir;            // 1: direct-activation tile kernel (weights through LDS, activations into registers)
+    int stem;            // 1: first-layer row (b_fs_yx_fsv4 input, streaming kernel)
     int by_features;     // 1: accelerator dies split the feature tiles (weights larger than activations)
     int wsl;             // 1: weights-stationary persistent kernel (weight tile resident in LDS)
     int wsl_depth;       // its activation look-ahead in K-steps

@@ -368,11 +368,13 @@ def conv_forward(engine, x, w, bias=None, wqf=None, calib=None, *, stride=(1, 1)
     if out_dt is None:
         out_dt = DT_OF[x.dtype]
     e_buf = None
+    # a first layer reads b_fs_yx_fsv4 and writes the blocked layout the rest of the network runs in
+    first_layer = FMT_NAME.get(fmt, fmt) == B_FS_YX_FSV4
     if eltw is not None:
-        e_buf = upload(engine, np.ascontiguousarray(eltw), fmt)
+        e_buf = upload(engine, np.ascontiguousarray(eltw), "fs_b_yx_fsv16" if first_layer else fmt)
     bias_dt = NO_TYPE if bias is None else DT_OF[np.asarray(bias).dtype]
     d = conv_desc(xin.tensor, w.shape, out_dt, stride=stride, pad=pad, dilation=dilation, groups=groups,
-                  out_pad=out_pad, bias_dt=bias_dt, w_dt=DT_OF[w.dtype], has_wqf=wqf is not None,
+                  out_fmt=FS_B_YX_FSV16 if first_layer else None, out_pad=out_pad, bias_dt=bias_dt, w_dt=DT_OF[w.dtype], has_wqf=wqf is not None,
                   has_calib=calib is not None, iqf=iqf, oqf=oqf, act=act, act_m=act_m, act_n=act_n,
                   eltw_t=None if e_buf is None else e_buf.tensor, non_conv_scale=non_conv_scale, eltw_act=eltw_act,
                   eltw_m=eltw_m, eltw_n=eltw_n, has_eltw_calib=eltw_calib is not None, eltw_stride=eltw_stride,

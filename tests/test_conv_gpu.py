@@ -147,6 +147,10 @@ def test_mfma_kernel_all_tiles(eng, shape, in_dt):
                 with pytest.raises(hip.HipError):  # needs constant tap offsets (zero border) and K <= 512
                     hip.conv_forward(eng, x, w, bias, wqf, calib, **kw)
                 continue
+            if tile and names[tile - 1].startswith("stem"):
+                with pytest.raises(hip.HipError):  # the first-layer row goes with b_fs_yx_fsv4 input
+                    hip.conv_forward(eng, x, w, bias, wqf, calib, **kw)
+                continue
             if tile and names[tile - 1].startswith(("bdir", "wsl")) and (no_border or -(-IFM // 16) % 4 != 0):
                 with pytest.raises(hip.HipError):  # needs constant tap offsets and feature slices in fours
                     hip.conv_forward(eng, x, w, bias, wqf, calib, **kw)
@@ -213,7 +217,7 @@ def test_mfma_fused_eltwise(eng, fast, eltw_dt):
     ecal = r.uniform(0.3, 1.2, 256).astype(np.float32)
     kw = dict(out_dt="s8", act="none", eltw=e, eltw_act="relu", eltw_calib=ecal,
               non_conv_scale=1.0 if fast else 0.5)
-    for tile in [0] + tiles():
+    for tile in [0] + [t for t in tiles() if not tile_names()[t - 1].startswith("stem")]:
         (ro, ra), (go, ga, info) = both(eng, x, w, bias, wqf, calib, fmt="fs_b_yx_fsv16", tile=tile, **kw)
         assert (b"fast" in info.kernel_name) == fast
         np.testing.assert_array_equal(ga, ra)
@@ -272,6 +276,26 @@ def test_depthwise_kernel(eng, shape, in_dt):
     (ro2, _), (go2, _, info2) = both(eng, x, w, bias, wqf, calib, fmt="bfyx", acc=True, **kw)
     assert info2.impl == hip.IMPL_REF
     assert_same(ro2, go2)
+
+
+@pytest.mark.parametrize("shape", [(2, 3, 32, 32, 64, 7, 7, 2, 3), (1, 3, 20, 20, 32, 3, 3, 1, 1), (2, 3, 19, 21, 32, 3, 3, 2, 1),
+                                   (1, 4, 9, 9, 16, 5, 5, 1, 2), (1, 1, 12, 12, 80, 3, 1, 1, 0)],
+                         ids=lambda s: "x".join(map(str, s)))
+@pytest.mark.parametrize("in_dt", [np.uint8, np.int8], ids=["u8", "s8"])
+def test_first_layer_fsv4(eng, shape, in_dt):
+    """First layers (at most 4 input features) read b_fs_yx_fsv4 and write fs_b_yx_fsv16: a matrix-core fragment is
+    4 horizontal taps x 4 features (the role b_fs_yx_fsv4 has in the reference, convolution_gpu_test.cpp:4931-5115)."""
+    B, IFM, H, W, OFM, FY, FX, s, p = shape
+    x, w, bias, wqf, calib = problem(21, B, IFM, H, W, OFM, FY, FX, in_dt)
+    kw = dict(stride=(s, s), pad=(p, p), out_dt="s8", act="relu")
+    (ro, ra), (go, ga, info) = both(eng, x, w, bias, wqf, calib, fmt="b_fs_yx_fsv4", in_pad=(p, p), **kw)
+    assert info.impl == hip.IMPL_MFMA and b"stem_p32" in info.kernel_name, info.kernel_name
+    np.testing.assert_array_equal(ga, ra)
+    assert_same(ro, go)
+    # without the zero border the layout-agnostic kernel takes over
+    (ro, ra), (go, ga, info) = both(eng, x, w, bias, wqf, calib, fmt="b_fs_yx_fsv4", **kw)
+    assert info.impl == (hip.IMPL_MFMA if p == 0 else hip.IMPL_REF)
+    assert_same(ro, go)
 
 
 def test_benchmark_calibration_data(eng):
