@@ -142,6 +142,7 @@ struct node {
     cldnn_layout out{};             // output layout incl. physical padding
     int32_t user_format = cldnn_format_any;  // output format before the layout pass (what the topology implies)
     bool is_output = false;
+    bool first_layer = false;       // convolution that reads b_fs_yx_fsv4 and writes fs_b_yx_fsv16
     bool constant = false;          // data primitive
     // activation folded into a convolution (reference prepare_primitive_fusing.cpp:396-433)
     int32_t fused_act = activation_none;

@@ -207,6 +207,7 @@ static void calc_layout(node* n)
         node* w = dep_named(n, p.weights.at(0));
         conv_geom g = conv_geometry(p, in, w->out);
         n->out = in;  // format follows the input (reference src/convolution.cpp:129)
+        if (n->first_layer) n->out.format = cldnn_format_fs_b_yx_fsv16;  // b_fs_yx_fsv4 in, blocked out
         n->out.size = make_tensor(g.B, g.OFM, g.OW, g.OH);
         if (p.out_dt.enabled) n->out.data_type = p.out_dt.data_type;
         break;
@@ -392,13 +393,14 @@ static bool wants_blocked(node* n)
 // fs_b_yx_fsv16; reorders are inserted where a tensor enters or leaves that format.
 static void select_layouts(cldnn_program_impl* prog)
 {
-    std::map<node*, node*> blocked_copy;  // producer -> its reorder into fs_b_yx_fsv16
+    std::map<std::pair<node*, int32_t>, node*> blocked_copy;  // (producer, format) -> its reorder into that format
     int counter = 0;
-    auto blocked_version = [&](node* src, node* before) -> node* {
-        if (src->out.format == cldnn_format_fs_b_yx_fsv16) return src;
-        auto it = blocked_copy.find(src);
+    auto blocked_version = [&](node* src, node* before, int32_t fmt = cldnn_format_fs_b_yx_fsv16) -> node* {
+        if (src->out.format == fmt) return src;
+        auto it = blocked_copy.find({src, fmt});
         if (it != blocked_copy.end()) return it->second;
-        auto r = make_reorder(src->p->id + "_to_fsv16_" + std::to_string(counter++), src->p->id, cldnn_format_fs_b_yx_fsv16);
+        auto r = make_reorder(src->p->id + (fmt == cldnn_format_b_fs_yx_fsv4 ? "_to_fsv4_" : "_to_fsv16_") + std::to_string(counter++),
+                              src->p->id, fmt);
         node* rn = add_node(prog, r, "");
         rn->deps = {src};
         src->users.push_back(rn);
@@ -407,7 +409,7 @@ static void select_layouts(cldnn_program_impl* prog)
         auto self = std::move(prog->nodes.back());
         prog->nodes.pop_back();
         prog->nodes.insert(prog->nodes.begin() + position(prog, before), std::move(self));
-        blocked_copy[src] = rn;
+        blocked_copy[{src, fmt}] = rn;
         return rn;
     };
     for (size_t i = 0; i < prog->nodes.size(); ++i) {
@@ -417,7 +419,15 @@ static void select_layouts(cldnn_program_impl* prog)
             if (!d->constant && d->out.format == cldnn_format_any) calc_layout(d);
         if (wants_blocked(n)) {
             const int32_t user_format = n->user_format;
-            node* a = blocked_version(n->deps[0], n);
+            // a first layer (at most 4 input features, no horizontal dilation) reads b_fs_yx_fsv4
+            {
+                node* wn = dep_named(n, n->p->weights.at(0));
+                const int fx = wn->out.size.sizes[2], fy = wn->out.size.sizes[3];
+                n->first_layer = n->p->type == prim_type::convolution && n->p->groups <= 1 && n->deps[0]->out.size.sizes[1] <= 4
+                                 && spatial(n->p->dilation, 0) == 1 && n->deps[0]->out.format != cldnn_format_fs_b_yx_fsv16
+                                 && (fy * ((fx + 3) / 4) + 3) / 4 <= 8;  // what the first-layer kernel holds in registers
+            }
+            node* a = blocked_version(n->deps[0], n, n->first_layer ? cldnn_format_b_fs_yx_fsv4 : cldnn_format_fs_b_yx_fsv16);
             if (a != n->deps[0]) replace_dep(n, n->deps[0], a);
             if (n->p->type == prim_type::fused_conv_eltwise && !n->p->second_input_in_output) {
                 node* b = blocked_version(n->deps[1], n);
@@ -479,7 +489,9 @@ static void prepare_borders(cldnn_program_impl* prog)
 {
     for (auto& u : prog->nodes) {
         node* n = u.get();
-        if (!wants_blocked(n) || n->deps[0]->out.format != cldnn_format_fs_b_yx_fsv16) continue;
+        if (!wants_blocked(n)) continue;
+        if (n->deps[0]->out.format != cldnn_format_fs_b_yx_fsv16 && !(n->first_layer && n->deps[0]->out.format == cldnn_format_b_fs_yx_fsv4))
+            continue;
         node* w = dep_named(n, n->p->weights.at(0));
         conv_geom g = conv_geometry(*n->p, n->deps[0]->out, w->out);
         if (g.px == 0 && g.py == 0 && g.FX == 1 && g.FY == 1) continue;

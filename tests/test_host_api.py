@@ -357,6 +357,19 @@ def test_layout_rule_takes_depthwise():
     assert by_id(opt)["conv_fsv16"]["format"] == F.fs_b_yx_fsv16
 
 
+def test_layout_rule_first_layer_reads_fsv4():
+    """A quantized convolution with at most 4 input features takes its input in b_fs_yx_fsv4 (the format the reference
+    has for first layers) and already writes fs_b_yx_fsv16."""
+    opt = by_id(cl.plan(conv_topology(IFM=3, OFM=64, FY=7, FX=7, H=32, W=32, stride=cl.tensor(1, 1, 2, 2),
+                                      input_offset=cl.tensor(0, 0, -3, -3, 0)), cl.build_options(optimize_data=True)))
+    assert opt["in_to_fsv4_0"]["format"] == F.b_fs_yx_fsv4 and opt["in_to_fsv4_0"]["pad_lower"] == [0, 0, 3, 3]
+    assert opt["conv_fsv16"]["format"] == F.fs_b_yx_fsv16 and opt["conv_fsv16"]["deps"][0] == "in_to_fsv4_0"
+    assert opt["conv"]["format"] == F.bfyx
+    # 11x11 filters are more than the first-layer kernel holds: the general blocked layout is used
+    opt = by_id(cl.plan(conv_topology(IFM=3, OFM=64, FY=11, FX=11, H=32, W=32), cl.build_options(optimize_data=True)))
+    assert "in_to_fsv16_0" in opt
+
+
 def test_one_reorder_serves_all_blocked_consumers():
     opt = cl.plan(residual_block(), cl.build_options(optimize_data=True))
     assert sum(n["id"].startswith("in_to_fsv16") for n in opt) == 1

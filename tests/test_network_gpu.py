@@ -223,6 +223,27 @@ def test_user_blocked_input_and_padded_input(eng):
     np.testing.assert_array_equal(outs["plain"].get_memory().read(), expected)
 
 
+def test_first_layer_through_network(eng):
+    """3-channel image -> 7x7 stride-2 quantized convolution: with optimize_data the input goes through b_fs_yx_fsv4."""
+    r = np.random.default_rng(12)
+    x = r.integers(0, 256, (2, 3, 30, 30)).astype(np.uint8)
+    w = r.integers(-127, 128, (32, 3, 7, 7)).astype(np.int8)
+    b = r.integers(-500, 500, 32).astype(np.int32)
+    q = np.ones(32, np.float32)
+    c = (40.0 / (np.sqrt(147) * 147.4 * 73.3) * r.uniform(0.5, 2, 32)).astype(np.float32)
+    expected = rc.conv(x, w, b, wqf=q, calib=c, pad=(3, 3), stride=(2, 2), out_dt="s8", act="relu")
+    topo = cl.topology(cl.input_layout("input", cl.layout(DT.u8, F.bfyx, cl.tensor(2, 3, 30, 30))),
+                       cl.data("w", cl.make_memory(eng, w)), cl.data("b", vec_mem(eng, b)), cl.data("q", vec_mem(eng, q)),
+                       cl.data("c", vec_mem(eng, c)),
+                       cl.convolution("stem", "input", ["w"], ["b"], ["q"], ["c"], stride=cl.tensor(1, 1, 2, 2),
+                                      input_offset=cl.tensor(0, 0, -3, -3, 0), with_activation=True, output_data_type=DT.i8))
+    for optimize in OPT:
+        net, outs = run(eng, topo, {"input": cl.make_memory(eng, x)}, optimize)
+        np.testing.assert_array_equal(outs["stem"].get_memory().read(), expected)
+    assert "stem_p32" in net.get_primitive_info("stem_fsv16")["kernel"]
+    assert net.get_primitive_info("input_to_fsv4_0")["format"] == F.b_fs_yx_fsv4
+
+
 def test_depthwise_through_network(eng):
     r = np.random.default_rng(9)
     C = 32
