@@ -346,7 +346,7 @@ def main():
             "unit": "TOP/s",
             "frac": ops * args.steps / t_gpu / PEAK_INT8_OPS,
             "traffic": measured_traffic(wl),
-            "kernel": "conv_mfma_kernel (all tile instances)",
+            "kernel": "convolution kernels of the step (all instances of the tile table)",
             "launches": launches,
             "avg_launch_us": t_gpu / launches * 1e6,
             "ops_per_launch": ops / len(stack),
