@@ -213,6 +213,10 @@ MfmaPlan mfma_plan(const ConvProblem& p, int tile, int cus)
         CHIP_REQUIRE(pl.ksteps * 4096 <= WSL_MAX_LDS, CLDNN_HIP_INVALID_ARG,
                      "the weights-stationary kernel holds 64 x K weight bytes in LDS: K is limited to 2560");
     }
+    // K order.  With the taps innermost, consecutive K-steps of a wave read the same cache lines of the input shifted
+    // by one pixel (or one row), so most activation loads of a 3x3 filter hit in the CU's L1 instead of going to L2.
+    // The weights-stationary and streaming kernels walk the taps with counters in (tap, slice) order.
+    pl.tap_minor = !pl.stream && !pl.wsl && pl.cb % 4 == 0 && p.FY * p.FX > 1 ? 1 : 0;
     pl.ofm_tiles = (p.OFM + tc.tile_ofm - 1) / tc.tile_ofm;
     pl.m_total = (int64_t)p.B * p.OH * p.OW;
     CHIP_REQUIRE(pl.m_total < (1ll << 31), CLDNN_HIP_UNSUPPORTED_SIZE, "more than 2^31 output pixels");
@@ -272,13 +276,16 @@ void mfma_pack_weights(const ConvProblem& p, const MfmaPlan& pl, const int8_t* w
                     }
         return;
     }
-    // k-chunk order: tap-major, feature slice minor
+    // k-chunk -> (tap, feature slice): tap-major with the slices innermost, or groups of 4 slices with the taps innermost
+    const int taps = p.FY * p.FX;
+    auto chunk_tap = [&](int kc) { return pl.tap_minor ? (kc / 4) % taps : kc / pl.cb; };
+    auto chunk_slice = [&](int kc) { return pl.tap_minor ? (kc / 4) / taps * 4 + kc % 4 : kc % pl.cb; };
     for (int kc = 0; kc < (pl.ksteps + MFMA_SLACK_STEPS) * 4; ++kc) {
         if (kc >= pl.kchunks) {
             ktab[kc] = pl.checked ? (int32_t)0x80000000 : 0;  // padding chunk: zero weights
             continue;
         }
-        const int tap = kc / pl.cb, cb = kc % pl.cb;
+        const int tap = chunk_tap(kc), cb = chunk_slice(kc);
         const int fyd = (tap / p.FX) * p.dy, fxd = (tap % p.FX) * p.dx;
         if (pl.checked) ktab[kc] = fyd | (fxd << 10) | (cb << 20);
         else ktab[kc] = (int32_t)(cb * p.in_p.pf + fyd * p.in_p.py + fxd * 16);
@@ -287,7 +294,7 @@ void mfma_pack_weights(const ConvProblem& p, const MfmaPlan& pl, const int8_t* w
         const int nt = f / BN;
         const int row = row_of(f);
         for (int kc = 0; kc < pl.kchunks; ++kc) {
-            const int tap = kc / pl.cb, cb = kc % pl.cb;
+            const int tap = chunk_tap(kc), cb = chunk_slice(kc);
             const int ks = kc / 4, kq = kc % 4;
             int8_t* dst = packed + ((((size_t)nt * pl.ksteps + ks) * 4 + kq) * BN + row) * 16;
             for (int c = 0; c < 16; ++c) {

@@ -95,6 +95,28 @@ __device__ __forceinline__ void lds_barrier()
 // look-ahead queue once per loop iteration.
 __device__ __forceinline__ void step_fence() { __builtin_amdgcn_sched_barrier(0); }
 
+// Instruction order inside one K-step: after each of the M matrix instructions (16 clocks in the matrix pipe, 4 to
+// issue) the scheduler is told to place a share of the step's other work -- R LDS reads, W LDS writes, V global
+// loads, VALU register work -- so that it issues in the shadow of the matrix pipe instead of in front of it.  The
+// memory operations go behind the first half of the matrix instructions, so that their latency has passed when the
+// step ends in a wait and a barrier.
+template <int I, int M, int R, int W, int V, int VALU>
+__device__ __forceinline__ void interleave_step()
+{
+    if constexpr (I < M) {
+        constexpr int H = (M + 1) / 2;  // slots that take memory operations
+        constexpr int i0 = I < H ? I : H, i1 = I + 1 < H ? I + 1 : H;
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        constexpr int r = i1 * R / H - i0 * R / H, w = i1 * W / H - i0 * W / H, v = i1 * V / H - i0 * V / H;
+        constexpr int va = (I + 1) * VALU / M - I * VALU / M;
+        if constexpr (w > 0) __builtin_amdgcn_sched_group_barrier(0x200, w, 0);
+        if constexpr (r > 0) __builtin_amdgcn_sched_group_barrier(0x100, r, 0);
+        if constexpr (v > 0) __builtin_amdgcn_sched_group_barrier(0x020, v, 0);
+        if constexpr (va > 0) __builtin_amdgcn_sched_group_barrier(0x002, va, 0);
+        interleave_step<I + 1, M, R, W, V, VALU>();
+    }
+}
+
 // Uniform table lookups go through the scalar data path (constant address space): a vector load here
 // would sit in the same in-order counter as the prefetched operand loads and force them to drain.
 typedef const int32_t __attribute__((address_space(4))) * const_i32_ptr;
@@ -601,10 +623,13 @@ __global__ void __launch_bounds__(256 * KG) conv_bdir_kernel(MfmaArgs a)
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) fa[mt] = ldsA[buf * 4 * BN + kq * BN + mt * 16 + l16];
     };
-    auto mma = [&](const v4i (&fa)[MT], const v4i (&xb)[NT]) {
-        v4i fb[NT];
+    // u8 activations become s8 by flipping the top bit (the accumulators start at 128 * sum of the weights); the flip
+    // of step k+1's fragments is done during step k, so a step starts with its matrix instructions
+    auto flip = [&](const v4i (&xb)[NT], v4i (&fb)[NT]) {
 #pragma unroll
         for (int nt = 0; nt < NT; ++nt) fb[nt] = xb[nt] ^ xm;
+    };
+    auto mma = [&](const v4i (&fa)[MT], const v4i (&fb)[NT]) {
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
@@ -625,8 +650,9 @@ __global__ void __launch_bounds__(256 * KG) conv_bdir_kernel(MfmaArgs a)
     load_a(DA, ra[0]);
     load_a(DA + 1, ra[1]);
     lds_barrier();
-    v4i fa_cur[MT], fa_nxt[MT];
+    v4i fa_cur[MT], fa_nxt[MT], fb_cur[NT], fb_nxt[NT];
     read_a(0, fa_cur);
+    flip(rb[0], fb_cur);
     int b1 = 1, b2 = 2, b0 = 0;  // ring positions of steps k+1, k+2, k
     const int main_steps = (steps / DA) * DA;
     for (int ks0 = 0; ks0 < main_steps; ks0 += DA) {
@@ -634,14 +660,18 @@ __global__ void __launch_bounds__(256 * KG) conv_bdir_kernel(MfmaArgs a)
         for (int u = 0; u < DA; ++u) {
             const int ks = ks0 + u;
             read_a(b1, fa_nxt);
-            mma(fa_cur, rb[u % D]);
+            mma(fa_cur, fb_cur);
+            flip(rb[(u + 1) % D], fb_nxt);
             store_a(b2, ra[(u + 2) % DA]);
             load_a(ks + 2 + DA, ra[(u + 2) % DA]);
             load_b(ks + D, rb[u % D]);
+            interleave_step<0, MT * NT, MT, A_LOADS, A_LOADS + NT, NT * 6 + 4>();
             lds_barrier();
             step_fence();
 #pragma unroll
             for (int mt = 0; mt < MT; ++mt) fa_cur[mt] = fa_nxt[mt];
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt) fb_cur[nt] = fb_nxt[nt];
             const int tmp = b0;
             b0 = b1, b1 = b2, b2 = tmp;
         }
@@ -651,13 +681,17 @@ __global__ void __launch_bounds__(256 * KG) conv_bdir_kernel(MfmaArgs a)
     for (int u = 0; u < DA - 1; ++u) {
         if (u < rest) {
             read_a(b1, fa_nxt);
-            mma(fa_cur, rb[u % D]);
+            mma(fa_cur, fb_cur);
+            flip(rb[(u + 1) % D], fb_nxt);
             store_a(b2, ra[(u + 2) % DA]);
             load_b(main_steps + u + D, rb[u % D]);
+            interleave_step<0, MT * NT, MT, A_LOADS, NT, NT * 6 + 4>();
             lds_barrier();
             step_fence();
 #pragma unroll
             for (int mt = 0; mt < MT; ++mt) fa_cur[mt] = fa_nxt[mt];
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt) fb_cur[nt] = fb_nxt[nt];
             const int tmp = b0;
             b0 = b1, b1 = b2, b2 = tmp;
         }

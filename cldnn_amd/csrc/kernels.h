@@ -45,6 +45,7 @@ struct MfmaPlan {
     int wsl_parts;       // pixel-range partitions per feature tile (multiple of 8)
     int wsl_tpp;         // pixel tiles per partition
     int checked;         // 1: taps bounds-checked per load, 0: input carries a sufficient zero border
+    int tap_minor;       // K order: 1 = (group of 4 slices, tap), taps innermost; 0 = (tap, slice)
     int cb;              // input feature slices of 16
     int kchunks;         // FY*FX*cb
     int ksteps;          // ceil(kchunks / 4)
