@@ -38,11 +38,11 @@ namespace {
 
 bool is_int8(int dt) { return dt == CLDNN_HIP_S8 || dt == CLDNN_HIP_U8; }
 
-int out_extent(int in, int pad, int filt, int dil, int stride)
+int out_extent(int in, int pad, int filt, int dil, int stride, int pad_end_delta = 0)
 {
     // reference src/include/sliding_window_utils.h:113-126; a window larger than the padded input gives 1
     const int wnd = (filt - 1) * dil + 1;
-    const int span = in + 2 * pad;
+    const int span = in + 2 * pad + pad_end_delta;
     if (wnd > span) return 1;
     return (span - wnd) / stride + 1;
 }
@@ -73,7 +73,8 @@ void build(cldnn_hip_conv c, const void* weights, const void* bias, const float*
                  "feature counts must divide into groups");
     CHIP_REQUIRE(d.fy > 0 && d.fx > 0 && d.stride_y > 0 && d.stride_x > 0 && d.dilation_y > 0 && d.dilation_x > 0,
                  CLDNN_HIP_INVALID_ARG, "filter size, stride and dilation must be positive");
-    CHIP_REQUIRE(d.pad_y >= 0 && d.pad_x >= 0, CLDNN_HIP_INVALID_ARG, "negative padding");
+    CHIP_REQUIRE(d.pad_y >= 0 && d.pad_x >= 0 && d.pad_y + d.pad_end_delta_y >= 0 && d.pad_x + d.pad_end_delta_x >= 0,
+                 CLDNN_HIP_INVALID_ARG, "negative padding");
     CHIP_REQUIRE(d.input.f == d.ifm, CLDNN_HIP_DIMENSION_MISMATCH, "input feature count differs from weights");
     CHIP_REQUIRE(d.output.f == d.ofm && d.output.b == d.input.b, CLDNN_HIP_DIMENSION_MISMATCH,
                  "output batch/feature count mismatch");
@@ -88,8 +89,8 @@ void build(cldnn_hip_conv c, const void* weights, const void* bias, const float*
     p.B = d.input.b, p.IFM = d.ifm, p.IH = d.input.y, p.IW = d.input.x, p.OFM = d.ofm;
     p.FY = d.fy, p.FX = d.fx, p.sy = d.stride_y, p.sx = d.stride_x, p.dy = d.dilation_y, p.dx = d.dilation_x;
     p.py = d.pad_y, p.px = d.pad_x, p.groups = d.groups;
-    p.OH = out_extent(p.IH, p.py, p.FY, p.dy, p.sy);
-    p.OW = out_extent(p.IW, p.px, p.FX, p.dx, p.sx);
+    p.OH = out_extent(p.IH, p.py, p.FY, p.dy, p.sy, d.pad_end_delta_y);
+    p.OW = out_extent(p.IW, p.px, p.FX, p.dx, p.sx, d.pad_end_delta_x);
     CHIP_REQUIRE(d.output.y == p.OH && d.output.x == p.OW, CLDNN_HIP_DIMENSION_MISMATCH,
                  "output spatial size differs from the computed one");
     p.in_dt = d.input.dtype, p.w_dt = d.weights_dtype, p.out_dt = d.output.dtype;

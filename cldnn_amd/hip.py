@@ -66,6 +66,7 @@ class ConvDesc(C.Structure):
         ("has_eltw_calib", C.c_int32), ("eltw_stride_y", C.c_int32), ("eltw_stride_x", C.c_int32),
         ("second_input_in_output", C.c_int32), ("round_to_even", C.c_int32),
         ("impl", C.c_int32), ("tile_override", C.c_int32),
+        ("pad_end_delta_y", C.c_int32), ("pad_end_delta_x", C.c_int32),
     ]
 
 
@@ -321,14 +322,15 @@ def conv_desc(x_t, w_shape, out_dt, *, stride=(1, 1), pad=(0, 0), dilation=(1, 1
               out_pad=(0, 0), bias_dt=NO_TYPE, w_dt=S8, has_wqf=False, has_calib=False, iqf=1.0, oqf=1.0,
               act="none", act_m=0.0, act_n=0.0, eltw_t=None, non_conv_scale=1.0, eltw_act="none", eltw_m=0.0,
               eltw_n=0.0, has_eltw_calib=False, eltw_stride=(1, 1), in_place=False, round_even=False,
-              impl=IMPL_AUTO, tile=0):
-    """Fill a ConvDesc from an input Tensor and the weight shape [OFM, IFM/groups, FY, FX]."""
+              impl=IMPL_AUTO, tile=0, pad_end=None):
+    """Fill a ConvDesc from an input Tensor and the weight shape [OFM, IFM/groups, FY, FX].
+    pad = zero padding on the low side (y, x); pad_end = on the high side (default: the same)."""
     L = lib()
     ofm, ifm_g, fy, fx = w_shape
     d = ConvDesc()
     d.input = x_t
-    oh = L.cldnn_hip_conv_out_extent(x_t.y, pad[0], fy, dilation[0], stride[0])
-    ow = L.cldnn_hip_conv_out_extent(x_t.x, pad[1], fx, dilation[1], stride[1])
+    pad_end = pad if pad_end is None else pad_end
+    oh, ow = out_extent(x_t.y, pad[0], pad_end[0], fy, dilation[0], stride[0]), out_extent(x_t.x, pad[1], pad_end[1], fx, dilation[1], stride[1])
     out_dt = DT_NAME[out_dt] if isinstance(out_dt, str) else out_dt
     d.output = Tensor.make(out_dt, x_t.format if out_fmt is None else out_fmt, x_t.b, ofm, oh, ow, out_pad[0], out_pad[1])
     d.weights_dtype, d.bias_dtype = w_dt, bias_dt
@@ -350,14 +352,21 @@ def conv_desc(x_t, w_shape, out_dt, *, stride=(1, 1), pad=(0, 0), dilation=(1, 1
     d.second_input_in_output = int(in_place)
     d.round_to_even = int(round_even)
     d.impl, d.tile_override = impl, tile
+    d.pad_end_delta_y, d.pad_end_delta_x = pad_end[0] - pad[0], pad_end[1] - pad[1]
     return d
+
+
+def out_extent(n, pad_lo, pad_hi, filt, dil, stride):
+    """output extent along one axis; a window larger than the padded input gives 1"""
+    wnd, span = (filt - 1) * dil + 1, n + pad_lo + pad_hi
+    return 1 if wnd > span else (span - wnd) // stride + 1
 
 
 def conv_forward(engine, x, w, bias=None, wqf=None, calib=None, *, stride=(1, 1), pad=(0, 0), dilation=(1, 1),
                  groups=1, out_dt=None, iqf=1.0, oqf=1.0, act="none", act_m=0.0, act_n=0.0, eltw=None,
                  non_conv_scale=1.0, eltw_act="none", eltw_m=0.0, eltw_n=0.0, eltw_calib=None, eltw_stride=(1, 1),
                  round_even=False, fmt="bfyx", in_pad=(0, 0), out_pad=(0, 0), impl=IMPL_AUTO, tile=0,
-                 want_acc=False, want_info=False):
+                 want_acc=False, want_info=False, pad_end=None):
     """numpy in, numpy out: upload (reordering to `fmt`), run the HIP convolution, download.
 
     Argument meaning follows oracle.refconv.conv so that parity tests can call both alike.
@@ -378,7 +387,7 @@ def conv_forward(engine, x, w, bias=None, wqf=None, calib=None, *, stride=(1, 1)
                   has_calib=calib is not None, iqf=iqf, oqf=oqf, act=act, act_m=act_m, act_n=act_n,
                   eltw_t=None if e_buf is None else e_buf.tensor, non_conv_scale=non_conv_scale, eltw_act=eltw_act,
                   eltw_m=eltw_m, eltw_n=eltw_n, has_eltw_calib=eltw_calib is not None, eltw_stride=eltw_stride,
-                  round_even=round_even, impl=impl, tile=tile)
+                  round_even=round_even, impl=impl, tile=tile, pad_end=pad_end)
     c = Conv(engine, d, w, bias, wqf, calib, eltw_calib)
     out = Buffer(engine, d.output)
     c.enqueue(xin, out, e_buf)

@@ -114,16 +114,29 @@ static int spatial(const cldnn_tensor& t, int i) { return t.sizes[2 + i]; }
 
 struct conv_geom {
     int B, IFM, IH, IW, OFM, FY, FX, sy, sx, dy, dx, py, px, OH, OW, groups;
+    int ey, ex;  // zero padding on the high side minus the padding on the low side (asymmetric padding_above / below)
 };
+
+// output extent with `lo` zeros in front of and `hi` behind the input (reference sliding_window_utils.h:113-126)
+static int window_extent(int in, int lo, int hi, int filt, int dil, int stride)
+{
+    const int wnd = (filt - 1) * dil + 1, span = in + lo + hi;
+    return wnd > span ? 1 : (span - wnd) / stride + 1;
+}
 
 static conv_geom conv_geometry(const prim& p, const cldnn_layout& in, const cldnn_layout& w)
 {
     conv_geom g{};
     g.B = in.size.sizes[0], g.IFM = in.size.sizes[1], g.IW = in.size.sizes[2], g.IH = in.size.sizes[3];
     g.groups = p.groups ? (int)p.groups : 1;
-    HOST_REQUIRE(p.split == 1, CLDNN_INVALID_ARG, "convolution split > 1 is not supported (use groups)");
+    // split: one weights / bias / ... primitive per part, each [OFM/split][IFM/split][y][x]; part i reads input features
+    // [i*IFM/split, ...) and writes output features [i*OFM/split, ...) (reference fused_conv_eltwise_gpu_ref.cl:111,
+    // 134-136,194) -- the same arithmetic as `groups = split` on the concatenated constants
+    const int split = p.split ? (int)p.split : 1;
+    HOST_REQUIRE(split == 1 || g.groups == 1, CLDNN_INVALID_ARG, "convolution: split and groups exclude each other");
+    if (split > 1) g.groups = split;
     HOST_REQUIRE(w.format == cldnn_format_bfyx, CLDNN_UNSUPPORTED_FORMAT, "convolution weights must be given in bfyx (o, i, y, x)");
-    g.OFM = w.size.sizes[0];
+    g.OFM = w.size.sizes[0] * split;
     g.FX = w.size.sizes[2], g.FY = w.size.sizes[3];
     HOST_REQUIRE(w.size.sizes[1] * g.groups == g.IFM, CLDNN_DIMENSION_MISMATCH,
                  "weights input feature count (x groups) differs from the input's feature count");
@@ -137,20 +150,24 @@ static conv_geom conv_geometry(const prim& p, const cldnn_layout& in, const cldn
                  "input offset in batch / feature is not supported");
     int ox = spatial(p.input_offset, 0), oy = spatial(p.input_offset, 1);
     HOST_REQUIRE(ox <= 0 && oy <= 0, CLDNN_INVALID_ARG, "positive input offsets are not supported");
-    // symmetric padding_above / padding_below fold into the offset (reference handle_input_padding.cpp:27-92)
+    // padding_above / padding_below: zeros in front of / behind the input.  The reference folds the symmetric case
+    // into the offset and puts a zero border primitive in front of the convolution otherwise
+    // (handle_input_padding.cpp:27-92); here both are padding of the convolution itself.
     int pax = spatial(p.padding_above, 0), pay = spatial(p.padding_above, 1);
     int pbx = spatial(p.padding_below, 0), pby = spatial(p.padding_below, 1);
-    HOST_REQUIRE(pax == pbx && pay == pby, CLDNN_INVALID_ARG, "asymmetric padding_above / padding_below is not supported");
+    HOST_REQUIRE(p.padding_above.sizes[0] == 0 && p.padding_above.sizes[1] == 0 && p.padding_below.sizes[0] == 0
+                     && p.padding_below.sizes[1] == 0, CLDNN_INVALID_ARG, "padding above / below in batch or feature is not supported");
+    HOST_REQUIRE(pax >= 0 && pay >= 0 && pbx >= 0 && pby >= 0, CLDNN_INVALID_ARG, "padding above / below cannot be negative");
     g.px = -ox + pax, g.py = -oy + pay;
+    g.ex = pbx - pax, g.ey = pby - pay;
+    const int ow = window_extent(g.IW, g.px, g.px + g.ex, g.FX, g.dx, g.sx);
+    const int oh = window_extent(g.IH, g.py, g.py + g.ey, g.FY, g.dy, g.sy);
     if (p.with_output_size) {
         g.OW = spatial(p.output_size, 0), g.OH = spatial(p.output_size, 1);
         HOST_REQUIRE(g.OW > 0 && g.OH > 0, CLDNN_INVALID_ARG, "user-defined output size must be positive");
-        HOST_REQUIRE(g.OW == cldnn_hip_conv_out_extent(g.IW, g.px, g.FX, g.dx, g.sx)
-                         && g.OH == cldnn_hip_conv_out_extent(g.IH, g.py, g.FY, g.dy, g.sy),
-                     CLDNN_INVALID_ARG, "user-defined output size differs from the computed one");
+        HOST_REQUIRE(g.OW == ow && g.OH == oh, CLDNN_INVALID_ARG, "user-defined output size differs from the computed one");
     } else {
-        g.OW = cldnn_hip_conv_out_extent(g.IW, g.px, g.FX, g.dx, g.sx);
-        g.OH = cldnn_hip_conv_out_extent(g.IH, g.py, g.FY, g.dy, g.sy);
+        g.OW = ow, g.OH = oh;
     }
     return g;
 }
@@ -538,30 +555,52 @@ static void compile_conv(cldnn_program_impl* prog, node* n)
     d.ofm = g.OFM, d.ifm = g.IFM, d.fy = g.FY, d.fx = g.FX;
     d.stride_y = g.sy, d.stride_x = g.sx, d.dilation_y = g.dy, d.dilation_x = g.dx;
     d.pad_y = g.py, d.pad_x = g.px, d.groups = g.groups;
+    d.pad_end_delta_y = g.ey, d.pad_end_delta_x = g.ex;
     d.input_quantization_factor = p.iqf;
     d.output_quantization_factor = p.oqf;
     d.bias_dtype = CLDNN_HIP_NO_TYPE;
 
+    // constants: one primitive per part of a split convolution, concatenated along the output features
+    const size_t parts = p.weights.size();
     const size_t wcount = (size_t)g.OFM * ifm_g * g.FY * g.FX;
-    std::vector<uint8_t> wv = read_constant(w, wcount, "weights"), bv, qv, cv, ev;
+    auto gather = [&](const std::vector<std::string>& ids, size_t total, const char* what, size_t* dt) {
+        HOST_REQUIRE(ids.size() == parts, CLDNN_INVALID_ARG, std::string(what) + ": one primitive per part of the split is needed");
+        std::vector<uint8_t> all;
+        for (const std::string& id : ids) {
+            node* c = dep_named(n, id);
+            if (dt) {
+                HOST_REQUIRE(all.empty() || *dt == c->out.data_type, CLDNN_INVALID_ARG, std::string(what) + ": parts differ in data type");
+                *dt = c->out.data_type;
+            }
+            std::vector<uint8_t> part = read_constant(c, total / parts, what);
+            all.insert(all.end(), part.begin(), part.end());
+        }
+        return all;
+    };
+    size_t wdt = w->out.data_type, bdt = cldnn_f32, fdt = cldnn_f32;
+    std::vector<uint8_t> wv = gather(p.weights, wcount, "weights", &wdt), bv, qv, cv, ev;
+    for (const std::string& id : p.weights) {
+        const cldnn_layout& wl = dep_named(n, id)->out;
+        HOST_REQUIRE(wl.format == cldnn_format_bfyx && wl.size.sizes[0] == w->out.size.sizes[0] && wl.size.sizes[1] == w->out.size.sizes[1]
+                         && wl.size.sizes[2] == w->out.size.sizes[2] && wl.size.sizes[3] == w->out.size.sizes[3],
+                     CLDNN_DIMENSION_MISMATCH, "the weights of a split convolution must agree in size and format");
+    }
     if (!p.bias.empty()) {
-        node* b = dep_named(n, p.bias[0]);
-        bv = read_constant(b, g.OFM, "bias");
-        d.bias_dtype = hip_dtype(b->out.data_type);
+        bv = gather(p.bias, g.OFM, "bias", &bdt);
+        d.bias_dtype = hip_dtype(bdt);
         HOST_REQUIRE(d.bias_dtype == CLDNN_HIP_I32 || d.bias_dtype == CLDNN_HIP_F32, CLDNN_INVALID_ARG, "bias must be i32 or f32");
     }
     if (!p.wqf.empty()) {
-        node* q = dep_named(n, p.wqf[0]);
-        HOST_REQUIRE(q->out.data_type == cldnn_f32, CLDNN_INVALID_ARG, "weights_quantization_factors must be f32");
-        qv = read_constant(q, g.OFM, "weights_quantization_factors");
+        qv = gather(p.wqf, g.OFM, "weights_quantization_factors", &fdt);
+        HOST_REQUIRE(fdt == cldnn_f32, CLDNN_INVALID_ARG, "weights_quantization_factors must be f32");
         d.has_wqf = 1;
     }
     if (!p.calib.empty()) {
         // the API requires quantization factors whenever calibration factors are given (reference api/CPP/convolution.hpp:462-463)
         HOST_REQUIRE(!p.wqf.empty() || fused, CLDNN_INVALID_ARG, "output_calibration_factors need weights_quantization_factors");
-        node* c = dep_named(n, p.calib[0]);
-        HOST_REQUIRE(c->out.data_type == cldnn_f32, CLDNN_INVALID_ARG, "output_calibration_factors must be f32");
-        cv = read_constant(c, g.OFM, "output_calibration_factors");
+        fdt = cldnn_f32;
+        cv = gather(p.calib, g.OFM, "output_calibration_factors", &fdt);
+        HOST_REQUIRE(fdt == cldnn_f32, CLDNN_INVALID_ARG, "output_calibration_factors must be f32");
         d.has_calib = 1;
     }
     // with_activation overrides whatever activation was folded in (reference convolution_gpu.cpp:100-101)

@@ -209,6 +209,10 @@ typedef struct {
     int32_t round_to_even;        /* 0 = reference behaviour (half away from zero) */
     int32_t impl;                 /* CLDNN_HIP_IMPL_* */
     int32_t tile_override;        /* 0 = table decides; otherwise row + 1 of the tile-config table (tuning / tests) */
+    /* zero padding on the high side MINUS the padding on the low side (pad_y / pad_x); 0 = symmetric.  Asymmetric
+     * padding_above / padding_below of the primitive, which the reference realises with a border primitive
+     * (src/graph_optimizer/handle_input_padding.cpp:43-77). */
+    int32_t pad_end_delta_y, pad_end_delta_x;
 } cldnn_hip_conv_desc;
 
 /* Host pointers: weights [ofm][ifm/groups][fy][fx] dense, bias/wqf/calib/eltw_calib [ofm] or NULL.

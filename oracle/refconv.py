@@ -85,11 +85,13 @@ def _dense(F, H, W):
 def conv(x, w, bias=None, wqf=None, calib=None, *, stride=(1, 1), pad=(0, 0), dilation=(1, 1), groups=1,
          out_dt=None, iqf=1.0, oqf=1.0, act="none", act_m=0.0, act_n=0.0,
          eltw=None, non_conv_scale=1.0, eltw_act="none", eltw_m=0.0, eltw_n=0.0, eltw_calib=None,
-         eltw_stride=(1, 1), round_even=False, want_acc=False, nthreads=0):
+         eltw_stride=(1, 1), round_even=False, want_acc=False, nthreads=0, pad_end=None):
     """Reference convolution on dense bfyx numpy arrays.
 
     x [B,IFM,IH,IW]; w [OFM,IFM/groups,FY,FX]; bias/wqf/calib/eltw_calib [OFM];
-    eltw [B,OFM,>=OH*esy..,>=OW*esx..].  stride/pad/dilation are (y, x).
+    eltw [B,OFM,>=OH*esy..,>=OW*esx..].  stride/pad/dilation are (y, x); pad is the zero padding on the
+    low side, pad_end on the high side (default: the same; the reference reaches the asymmetric case with a
+    zero border in front of the convolution, src/graph_optimizer/handle_input_padding.cpp:43-77).
     Returns out (and the int32 accumulators when want_acc).
     """
     L = lib()
@@ -98,8 +100,15 @@ def conv(x, w, bias=None, wqf=None, calib=None, *, stride=(1, 1), pad=(0, 0), di
     B, IFM, IH, IW = x.shape
     OFM, IFMg, FY, FX = w.shape
     assert IFMg * groups == IFM, (IFMg, groups, IFM)
-    OH = out_extent(IH, pad[0], FY, dilation[0], stride[0])
-    OW = out_extent(IW, pad[1], FX, dilation[1], stride[1])
+    if pad_end is None:
+        OH = out_extent(IH, pad[0], FY, dilation[0], stride[0])
+        OW = out_extent(IW, pad[1], FX, dilation[1], stride[1])
+    else:  # the border primitive enlarges the input; the window then slides over the enlarged tensor
+        def ext(n, lo, hi, k, dil, st):
+            wnd, span = (k - 1) * dil + 1, n + lo + hi
+            return 1 if wnd > span else (span - wnd) // st + 1
+        OH = ext(IH, pad[0], pad_end[0], FY, dilation[0], stride[0])
+        OW = ext(IW, pad[1], pad_end[1], FX, dilation[1], stride[1])
     d = Desc()
     d.in_dt, d.w_dt = DT_OF[x.dtype], DT_OF[w.dtype]
     d.bias_dt = NONE if bias is None else DT_OF[np.asarray(bias).dtype]

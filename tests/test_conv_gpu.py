@@ -76,6 +76,66 @@ def test_kat_indexing(eng, case):
     np.testing.assert_allclose(out.astype(np.float64), p["expected"], atol=max(p["tol"], 1e-5), rtol=0)
 
 
+@pytest.mark.parametrize("case", K["api"], ids=lambda c: c["name"])
+def test_kat_api_tables(eng, case):
+    """further tables of the reference's convolution tests: padding above / below, output padding, split as groups"""
+    p = kat.api_problem(case, K["indexing"])
+    lo = (p["pad"][0] + p["pad_above"][0], p["pad"][1] + p["pad_above"][1])
+    hi = (p["pad"][0] + p["pad_below"][0], p["pad"][1] + p["pad_below"][1])
+    assert p["out_pad_lower"] == p["out_pad_upper"]
+    out = hip.conv_forward(eng, p["x"], p["w"], p["bias"], stride=p["stride"], pad=lo, pad_end=hi,
+                           groups=max(p["groups"], p["split"]), act="relu_slope" if p["act_slope"] else p["act"],
+                           act_m=p["act_slope"], out_pad=p["out_pad_lower"])
+    kat.assert_close_where_given(out, p["expected"], p["tol"])
+
+
+@pytest.mark.parametrize("case", [c for c in K["quantized_recipe"] if c["scale"] != "two_layers"], ids=lambda c: c["name"])
+@pytest.mark.parametrize("fmt", ["bfyx", "fs_b_yx_fsv16"])
+def test_kat_quantized_recipe(eng, case, fmt):
+    """float-vs-int8 tolerance tests of the reference (convolution_gpu_test.cpp:3741-3969): int8 result / factor within 3 of
+    the float table, and identical to the oracle"""
+    x = np.array(case["input"], np.float32).reshape(case["in_shape"])
+    wf = np.array(case["weights_f"], np.float32).reshape(case["w_shape"])
+    bias = np.array(case["bias"], np.float32)
+    exp = np.array(case["float_output"], np.float64).reshape(case["out_shape"])
+    wq, wqf = kat.quantize_weights(wf)
+    kw = dict(stride=tuple(case["stride"]), out_dt="s8")
+    if case["scale"] == "single":
+        scale = np.float32(127.0) / np.float32(np.abs(exp).max())
+        kw.update(oqf=float(scale))
+        calib = None
+    else:
+        calib = scale = kat.calibrate(exp.astype(np.float32))
+    out = hip.conv_forward(eng, x.astype(np.int8), wq.astype(np.int8), bias, wqf, calib, fmt=fmt, **kw)
+    ref = rc.conv(x.astype(np.int8), wq.astype(np.int8), bias, wqf=wqf, calib=calib, **kw)
+    np.testing.assert_array_equal(out, ref)
+    assert np.abs(out.astype(np.float64) / np.reshape(scale, (1, -1, 1, 1)) - exp).max() <= case["tol"]
+
+
+ASYM = [
+    # IFM OFM  H   W  k groups stride pad(lo)  pad_end  in_pad  fmt
+    (64, 64, 14, 14, 3, 1, (1, 1), (1, 1), (2, 3), (0, 0), "fs_b_yx_fsv16"),   # bounds-checked taps
+    (64, 64, 14, 14, 3, 1, (1, 1), (1, 1), (2, 3), (2, 3), "fs_b_yx_fsv16"),   # zero border wide enough for the high side
+    (64, 128, 15, 13, 3, 1, (2, 2), (0, 1), (2, 1), (2, 2), "fs_b_yx_fsv16"),
+    (32, 32, 12, 12, 3, 32, (1, 1), (1, 0), (0, 2), (0, 0), "fs_b_yx_fsv16"),  # depthwise
+    (32, 32, 12, 12, 3, 32, (2, 2), (0, 1), (1, 1), (1, 2), "fs_b_yx_fsv16"),
+    (3, 64, 20, 20, 7, 1, (2, 2), (3, 3), (2, 4), (4, 4), "b_fs_yx_fsv4"),     # first layer
+    (16, 24, 9, 11, 3, 1, (1, 1), (2, 0), (0, 2), (0, 0), "bfyx"),             # layout-agnostic kernel
+]
+
+
+@pytest.mark.parametrize("shape", ASYM, ids=lambda s: "x".join(str(v) for v in s[:6]) + "_" + s[-1])
+def test_asymmetric_padding(eng, shape):
+    """different zero padding in front of and behind the input (padding_above / padding_below of the primitive)"""
+    IFM, OFM, H, W, k, groups, stride, lo, hi, in_pad, fmt = shape
+    x, w, bias, wqf, calib = problem(77, 2, IFM, H, W, OFM, k, k, groups=groups)
+    kw = dict(stride=stride, pad=lo, pad_end=hi, groups=groups, out_dt="u8", act="relu")
+    out = hip.conv_forward(eng, x, w, bias, wqf, calib, fmt=fmt, in_pad=in_pad, **kw)
+    ref = rc.conv(x, w, bias, wqf=wqf, calib=calib, **kw)
+    assert out.shape == ref.shape
+    np.testing.assert_array_equal(out, ref)
+
+
 # ------------------------------------------------------------------ seeded random problems vs the oracle
 def problem(seed, B, IFM, H, W, OFM, FY, FX, in_dt=np.uint8, groups=1, spread=True):
     r = np.random.default_rng(seed)

@@ -190,12 +190,41 @@ def test_user_output_size_must_agree():
     (dict(dilation=cl.tensor(1, 1, 1, 0)), "dilation"),
     (dict(input_offset=cl.tensor(0, 1, 0, 0, 0)), "input offset"),
     (dict(groups=3), "feature count"),
-    (dict(padding_above=cl.tensor(0, 0, 1, 1, 0)), "asymmetric"),
+    (dict(padding_above=cl.tensor(0, 0, -1, 0, 0)), "cannot be negative"),
+    (dict(padding_below=cl.tensor(0, 1, 0, 0, 0)), "batch or feature"),
 ])
 def test_conv_argument_validation(kw, msg):
     with pytest.raises(cl.error) as e:
         cl.plan(conv_topology(**kw))
     assert msg in str(e.value)
+
+
+def test_padding_above_below_output_size():
+    """reference tests basic_convolution_sym / asym_input_padding (convolution_gpu_test.cpp:1064-1257): zeros above
+    (in front of) and below (behind) the input; the symmetric case equals a negative input offset"""
+    # 12 x 10 input, 3x3 filter: (12 + 1 + 2 - 3) + 1 = 13 rows, (10 + 2 + 3 - 3) + 1 = 13 columns
+    t = conv_topology(padding_above=cl.tensor(0, 0, 2, 1, 0), padding_below=cl.tensor(0, 0, 3, 2, 0))
+    assert by_id(cl.plan(t))["conv"]["size"] == [2, 8, 13, 13]
+    sym = conv_topology(padding_above=cl.tensor(0, 0, 1, 1, 0), padding_below=cl.tensor(0, 0, 1, 1, 0))
+    off = conv_topology(input_offset=cl.tensor(0, 0, -1, -1, 0))
+    assert by_id(cl.plan(sym))["conv"]["size"] == by_id(cl.plan(off))["conv"]["size"] == [2, 8, 10, 12]
+    # together with an input offset (reference ..._with_input_offset, :1259-1478)
+    both = conv_topology(input_offset=cl.tensor(0, 0, -1, -2, 0), padding_above=cl.tensor(0, 0, 1, 0, 0),
+                         padding_below=cl.tensor(0, 0, 0, 1, 0))
+    assert by_id(cl.plan(both))["conv"]["size"] == [2, 8, 11, 15]
+
+
+def test_split_convolution_layout():
+    """split = one weights primitive per part; output features = parts x weights.batch (reference src/convolution.cpp:103)"""
+    w = np.ones((4, 8, 1, 1), np.int8)
+    t = cl.topology(cl.input_layout("in", cl.layout(DT.i8, F.bfyx, cl.tensor(1, 16, 4, 4))),
+                    cl.data("w0", attach(w)), cl.data("w1", attach(w)), cl.convolution("conv", "in", ["w0", "w1"]))
+    assert by_id(cl.plan(t))["conv"]["size"] == [1, 8, 4, 4]
+    bad = cl.topology(cl.input_layout("in", cl.layout(DT.i8, F.bfyx, cl.tensor(1, 16, 4, 4))),
+                      cl.data("w0", attach(w)), cl.data("w1", attach(w)), cl.convolution("conv", "in", ["w0", "w1"], groups=2))
+    with pytest.raises(cl.error) as e:
+        cl.plan(bad)
+    assert "split and groups" in str(e.value)
 
 
 def test_weights_feature_mismatch():

@@ -99,6 +99,112 @@ def test_kat_indexing(eng, case):
     np.testing.assert_allclose(out.astype(np.float64), p["expected"], atol=max(p["tol"], 1e-5), rtol=0)
 
 
+def yx(t):
+    """(y, x) -> tensor with batch / feature 0 (offsets, paddings)"""
+    return cl.tensor(0, 0, t[1], t[0], 0)
+
+
+@pytest.mark.parametrize("optimize", OPT, ids=["plain", "optimize_data"])
+@pytest.mark.parametrize("case", K["api"], ids=lambda c: c["name"])
+def test_kat_api_tables(eng, case, optimize):
+    """further tables of the reference's convolution tests through the primitive's own arguments: padding_above / below,
+    input offset, output padding, one weights / bias primitive per part of a split, groups, negative slope"""
+    p = kat.api_problem(case, K["indexing"])
+    b, f, h, w = p["x"].shape
+    prims = [cl.input_layout("input", cl.layout(cl.DT_OF[p["x"].dtype], F.bfyx, cl.tensor(b, f, w, h)))]
+    wid, bid = [], []
+    for i, (wp, bp) in enumerate(zip(p["w_parts"], p["bias_parts"])):
+        prims += [cl.data(f"weights{i}", cl.make_memory(eng, np.ascontiguousarray(wp))), cl.data(f"biases{i}", vec_mem(eng, bp))]
+        wid.append(f"weights{i}"), bid.append(f"biases{i}")
+    lo, up = p["out_pad_lower"], p["out_pad_upper"]
+    prims.append(cl.convolution("conv", "input", wid, bid, stride=cl.tensor(1, 1, p["stride"][1], p["stride"][0]),
+                                input_offset=yx((-p["pad"][0], -p["pad"][1])), groups=p["groups"],
+                                with_activation=p["act"] == "relu", activation_slp=p["act_slope"],
+                                padding_above=yx(p["pad_above"]), padding_below=yx(p["pad_below"]),
+                                output_padding=cl.padding((0, 0, lo[0], lo[1]), (0, 0, up[0], up[1]))))
+    net, outs = run(eng, cl.topology(*prims), {"input": cl.make_memory(eng, p["x"])}, optimize)
+    mem = outs["conv"].get_memory()
+    l = mem.get_layout()
+    assert [l.padding.lower_size.sizes[i] for i in (3, 2)] == list(lo) and [l.padding.upper_size.sizes[i] for i in (3, 2)] == list(up)
+    kat.assert_close_where_given(mem.read(), p["expected"], p["tol"])
+
+
+@pytest.mark.parametrize("optimize", OPT, ids=["plain", "optimize_data"])
+@pytest.mark.parametrize("case", [c for c in K["quantized_recipe"] if c["scale"] != "two_layers"], ids=lambda c: c["name"])
+def test_kat_quantized_recipe(eng, case, optimize):
+    """reference convolution_gpu_test.cpp:3741-3969: a float network gives the scale, the int8 network must come within 3"""
+    x = np.array(case["input"], np.float32).reshape(case["in_shape"])
+    wf = np.array(case["weights_f"], np.float32).reshape(case["w_shape"])
+    bias = np.array(case["bias"], np.float32)
+    b, f, h, w = x.shape
+    stride = cl.tensor(0, 0, case["stride"][1], case["stride"][0])  # the test passes { 0, 0, 1, 2 }
+    tf = cl.topology(cl.input_layout("input_f", cl.layout(DT.f32, F.bfyx, cl.tensor(b, f, w, h))), cl.data("weights_f", cl.make_memory(eng, wf)),
+                     cl.data("biases", vec_mem(eng, bias)), cl.convolution("conv_f", "input_f", ["weights_f"], ["biases"], stride=stride))
+    net_f, outs_f = run(eng, tf, {"input_f": cl.make_memory(eng, x)}, optimize)
+    fl = outs_f["conv_f"].get_memory().read()
+    np.testing.assert_allclose(fl, np.array(case["float_output"], np.float32).reshape(case["out_shape"]), atol=1e-4)
+    wq, wqf = kat.quantize_weights(wf)
+    prims = [cl.input_layout("input", cl.layout(DT.i8, F.bfyx, cl.tensor(b, f, w, h))), cl.data("weights", cl.make_memory(eng, wq.astype(np.int8))),
+             cl.data("biases", vec_mem(eng, bias)), cl.data("w_qfs", vec_mem(eng, wqf))]
+    if case["scale"] == "single":
+        scale = np.float32(127.0) / np.abs(fl).max()
+        prims.append(cl.convolution("conv", "input", ["weights"], ["biases"], ["w_qfs"], None, 1.0, float(scale), stride=stride))
+    else:
+        scale = kat.calibrate(fl)
+        prims += [cl.data("out_calibrations", vec_mem(eng, scale)),
+                  cl.convolution("conv", "input", ["weights"], ["biases"], ["w_qfs"], ["out_calibrations"], 1.0, stride=stride)]
+    net, outs = run(eng, cl.topology(*prims), {"input": cl.make_memory(eng, x.astype(np.int8))}, optimize)
+    out = outs["conv"].get_memory().read()
+    assert out.dtype == np.int8
+    assert np.abs(out.astype(np.float64) / np.reshape(scale, (1, -1, 1, 1)) - fl).max() <= case["tol"]
+
+
+@pytest.mark.parametrize("optimize", OPT, ids=["plain", "optimize_data"])
+def test_kat_calibration_advance(eng, optimize):
+    """reference convolution_gpu_test.cpp:4199-4343: two convolutions, calibration of the first divided out of the second's
+    weights, both outputs requested; int8 network within 3 of the float network"""
+    case = next(c for c in K["quantized_recipe"] if c["scale"] == "two_layers")
+    x = np.array(case["input"], np.float32).reshape(case["in_shape"])
+    w1 = np.array(case["weights_f"], np.float32).reshape(case["w_shape"])
+    w2 = np.array(case["weights_f_2"], np.float32).reshape(case["w2_shape"])
+    b1, b2 = np.array(case["bias"], np.float32), np.array(case["bias_2"], np.float32)
+    b, f, h, w = x.shape
+    s1, s2 = cl.tensor(0, 0, case["stride"][1], case["stride"][0]), cl.tensor(0, 0, case["stride_2"][1], case["stride_2"][0])
+    tf = cl.topology(cl.input_layout("input_f", cl.layout(DT.f32, F.bfyx, cl.tensor(b, f, w, h))),
+                     cl.data("weights_f", cl.make_memory(eng, w1)), cl.data("biases", vec_mem(eng, b1)),
+                     cl.data("weights_f_2", cl.make_memory(eng, w2)), cl.data("biases_2", vec_mem(eng, b2)),
+                     cl.convolution("conv_f", "input_f", ["weights_f"], ["biases"], stride=s1),
+                     cl.convolution("conv_f_2", "conv_f", ["weights_f_2"], ["biases_2"], stride=s2))
+    net_f = cl.network(eng, tf, cl.build_options(optimize_data=optimize, outputs=["conv_f", "conv_f_2"]))
+    net_f.set_input_data("input_f", cl.make_memory(eng, x))
+    outs_f = net_f.execute()
+    assert sorted(outs_f) == ["conv_f", "conv_f_2"]
+    f1, f2 = outs_f["conv_f"].get_memory().read(), outs_f["conv_f_2"].get_memory().read()
+    np.testing.assert_allclose(f1, rc.conv(x, w1, b1, stride=tuple(case["stride"])), atol=1e-4)
+    c1, c2 = kat.calibrate(f1), kat.calibrate(f2)
+    w2c = w2 / c1.reshape(1, -1, 1, 1)  # apply_calibration_on_weights (:3618-3632): per INPUT feature
+    q1, wqf1 = kat.quantize_weights(w1)
+    q2, wqf2 = kat.quantize_weights(w2c)
+    t = cl.topology(cl.input_layout("input", cl.layout(DT.i8, F.bfyx, cl.tensor(b, f, w, h))),
+                    cl.data("weights", cl.make_memory(eng, q1.astype(np.int8))), cl.data("biases", vec_mem(eng, b1)),
+                    cl.data("weights_2", cl.make_memory(eng, q2.astype(np.int8))), cl.data("biases_2", vec_mem(eng, b2)),
+                    cl.data("w_qf", vec_mem(eng, wqf1)), cl.data("w_qf_2", vec_mem(eng, wqf2)),
+                    cl.data("calib", vec_mem(eng, c1)), cl.data("calib_2", vec_mem(eng, c2)),
+                    cl.convolution("conv", "input", ["weights"], ["biases"], ["w_qf"], ["calib"], 1.0, stride=s1),
+                    cl.convolution("conv_2", "conv", ["weights_2"], ["biases_2"], ["w_qf_2"], ["calib_2"], 1.0, stride=s2))
+    net = cl.network(eng, t, cl.build_options(optimize_data=optimize, outputs=["conv", "conv_2"]))
+    net.set_input_data("input", cl.make_memory(eng, x.astype(np.int8)))
+    outs = net.execute()
+    assert sorted(outs) == ["conv", "conv_2"]
+    o2 = outs["conv_2"].get_memory().read()
+    assert np.abs(o2.astype(np.float64) / c2.reshape(1, -1, 1, 1) - f2).max() <= case["tol"]
+    # and bit-exact against the oracle run layer by layer
+    r1 = rc.conv(x.astype(np.int8), q1.astype(np.int8), b1, wqf=wqf1, calib=c1, stride=tuple(case["stride"]), out_dt="s8")
+    r2 = rc.conv(r1, q2.astype(np.int8), b2, wqf=wqf2, calib=c2, stride=tuple(case["stride_2"]), out_dt="s8")
+    np.testing.assert_array_equal(outs["conv"].get_memory().read(), r1)
+    np.testing.assert_array_equal(o2, r2)
+
+
 # ------------------------------------------------------------------------------------------ networks vs the oracle
 def rand_layer(r, ofm, ifm, k, in_u8=True):
     w = r.integers(-127, 128, (ofm, ifm, k, k)).astype(np.int8)

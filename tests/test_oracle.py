@@ -49,6 +49,49 @@ def test_kat_indexing(case):
     np.testing.assert_allclose(out.astype(np.float64), p["expected"], atol=max(p["tol"], 1e-12), rtol=0)
 
 
+def _api_pads(p):
+    """padding above / below add to the padding the input offset asks for (low side, high side)"""
+    lo = (p["pad"][0] + p["pad_above"][0], p["pad"][1] + p["pad_above"][1])
+    hi = (p["pad"][0] + p["pad_below"][0], p["pad"][1] + p["pad_below"][1])
+    return lo, hi
+
+
+@pytest.mark.parametrize("case", K["api"], ids=lambda c: c["name"])
+def test_kat_api_tables(case):
+    p = kat.api_problem(case, K["indexing"])
+    lo, hi = _api_pads(p)
+    out = rc.conv(p["x"], p["w"], p["bias"], stride=p["stride"], pad=lo, pad_end=hi, groups=max(p["groups"], p["split"]),
+                  act="relu_slope" if p["act_slope"] else p["act"], act_m=p["act_slope"])
+    kat.assert_close_where_given(out, p["expected"], p["tol"])
+
+
+def quantized_recipe(case):
+    """the reference's recipe (convolution_gpu_test.cpp:3741-3969): float network first, then weights requantised per
+    feature and the output scaled by 127 / max|float output| (one factor, or one per feature)"""
+    x = np.array(case["input"], np.float32).reshape(case["in_shape"])
+    wf = np.array(case["weights_f"], np.float32).reshape(case["w_shape"])
+    bias = np.array(case["bias"], np.float32)
+    fl = rc.conv(x, wf, bias, stride=tuple(case["stride"]))
+    wq, wqf = kat.quantize_weights(wf)
+    return x, wf, bias, fl, wq.astype(np.int8), wqf
+
+
+@pytest.mark.parametrize("case", [c for c in K["quantized_recipe"] if c["scale"] != "two_layers"], ids=lambda c: c["name"])
+def test_kat_quantized_recipe(case):
+    x, wf, bias, fl, wq, wqf = quantized_recipe(case)
+    exp = np.array(case["float_output"], np.float64).reshape(case["out_shape"])
+    np.testing.assert_allclose(fl, exp, atol=1e-4, rtol=0)  # the table in the test's source is the float network's output
+    if case["scale"] == "single":
+        oqf = np.float32(127.0) / np.abs(fl).max()
+        out = rc.conv(x.astype(np.int8), wq, bias, wqf=wqf, oqf=float(oqf), stride=tuple(case["stride"]), out_dt="s8")
+        back = out.astype(np.float64) / oqf
+    else:
+        calib = kat.calibrate(fl)
+        out = rc.conv(x.astype(np.int8), wq, bias, wqf=wqf, calib=calib, stride=tuple(case["stride"]), out_dt="s8")
+        back = out.astype(np.float64) / calib.reshape(1, -1, 1, 1)
+    assert np.abs(back - exp).max() <= case["tol"]
+
+
 def test_round_to_even_variant_differs_only_on_ties():
     case = next(c for c in K["conv_quantized"] if c["name"] == "i8_to_u8")
     p = kat.diag_problem(case)
