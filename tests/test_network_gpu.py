@@ -205,6 +205,60 @@ def test_kat_calibration_advance(eng, optimize):
     np.testing.assert_array_equal(o2, r2)
 
 
+FUSE_INPUT = [1.0, 2.0, -15.0, 3.0, 4.0, -15.0, 5.0, 6.0, -15.0, 7.0, -15.0, 0.0, 0.0, -15.0, 0.5, -0.5, -15.0, 8.0, 1.5, 5.2]
+
+
+@pytest.mark.parametrize("with_reorder", [True, False], ids=["basic_0", "dont_fuse_if_conv_elt_are_outputs"])
+def test_conv_eltwise_float_graphs(eng, with_reorder):
+    """reference fused_conv_eltwise_gpu_test.cpp:41-118: a float 1x1 convolution summed with its own input, optimised build;
+    the reference asserts the output's id and layout, the values here are input + w * input"""
+    x = np.array(FUSE_INPUT, np.float32).reshape(1, 1, 5, 4)
+    wv = np.array([[[[2.5]]]], np.float32)
+    prims = [cl.input_layout("input", cl.layout(DT.f32, F.bfyx, cl.tensor(1, 1, 4, 5))), cl.data("weights", cl.make_memory(eng, wv)),
+             cl.convolution("conv", "input", ["weights"])]
+    if with_reorder:
+        prims += [cl.eltwise("eltwise", "input", "conv", cl.eltwise_mode.sum), cl.reorder("out", "eltwise", F.bfyx, DT.f32)]
+    else:
+        prims += [cl.eltwise("out", "input", "conv", cl.eltwise_mode.sum)]
+    net, outs = run(eng, cl.topology(*prims), {"input": cl.make_memory(eng, x)}, True)
+    assert list(outs) == ["out"]
+    mem = outs["out"].get_memory()
+    l = mem.get_layout()
+    assert l.format == F.bfyx and [l.size.sizes[i] for i in range(4)] == [1, 1, 4, 5]
+    np.testing.assert_allclose(mem.read(), x + 2.5 * x, rtol=1e-6)
+
+
+def test_three_convolutions_same_weights(eng):
+    """reference convolution_gpu_test.cpp:762-824: one weights primitive feeds three chained 1x1 convolutions"""
+    x = np.ones((1, 2, 2, 2), np.float32)
+    t = cl.topology(cl.input_layout("input", cl.layout(DT.f32, F.bfyx, cl.tensor(1, 2, 2, 2))),
+                    cl.data("weights", cl.make_memory(eng, np.ones((2, 2, 1, 1), np.float32))),
+                    cl.convolution("conv1", "input", ["weights"]), cl.convolution("conv2", "conv1", ["weights"]),
+                    cl.convolution("conv3", "conv2", ["weights"]))
+    net, outs = run(eng, t, {"input": cl.make_memory(eng, x)}, True)
+    out = outs["conv3"].get_memory().read()
+    assert out.shape == (1, 2, 2, 2) and np.all(out == 8.0)
+
+
+def test_with_output_size_same_input(eng):
+    """reference convolution_gpu_test.cpp:737-760: two convolutions with user-given output sizes read one input; both
+    are outputs, in the order of their ids"""
+    r = np.random.default_rng(5)
+    x = r.standard_normal((1, 4, 320, 320)).astype(np.float32)
+    w1, w2 = (r.standard_normal((64, 4, 7, 7)).astype(np.float32) for _ in range(2))
+    t = cl.topology(cl.input_layout("input", cl.layout(DT.f32, F.bfyx, cl.tensor(1, 4, 320, 320))),
+                    cl.data("weights", cl.make_memory(eng, w1)), cl.data("weights2", cl.make_memory(eng, w2)),
+                    cl.convolution("conv1", "input", ["weights"], stride=cl.tensor(1, 1, 2, 2), input_offset=cl.tensor(0, 0, -3, -3, 0),
+                                   output_size=cl.tensor(1, 64, 160, 160)),
+                    cl.convolution("conv2", "input", ["weights2"], stride=cl.tensor(1, 1, 1, 1), input_offset=cl.tensor(0, 0, -3, -3, 0),
+                                   output_size=cl.tensor(1, 64, 320, 320)))
+    net, outs = run(eng, t, {"input": cl.make_memory(eng, x)}, False)
+    assert sorted(outs) == ["conv1", "conv2"]
+    o1 = outs["conv1"].get_memory().read()
+    assert o1.shape == (1, 64, 160, 160) and outs["conv2"].get_memory().read().shape == (1, 64, 320, 320)
+    np.testing.assert_allclose(o1[:, :4], rc.conv(x, w1[:4], None, stride=(2, 2), pad=(3, 3)), rtol=1e-4, atol=1e-3)
+
+
 # ------------------------------------------------------------------------------------------ networks vs the oracle
 def rand_layer(r, ofm, ifm, k, in_u8=True):
     w = r.integers(-127, 128, (ofm, ifm, k, k)).astype(np.int8)
