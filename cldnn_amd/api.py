@@ -37,6 +37,10 @@ class activation_func:  # noqa: N801
     softrelu, abs, linear, square, sqrt, elu, negative = 6, 7, 8, 9, 10, 11, 25
 
 
+class pooling_mode:  # noqa: N801
+    max, average, average_no_padding, max_with_argmax, bilinear = range(5)
+
+
 class eltwise_mode:  # noqa: N801
     sum, sub, max, prod = 0, 1, 2, 3
 
@@ -102,6 +106,11 @@ class c_act_params(C.Structure):
 class c_activation_desc(C.Structure):
     _fields_ = _BASE + [("activation_func", C.c_int), ("additional_params", c_act_params),
                         ("additional_params_input", C.c_char_p)]
+
+
+class c_pooling_desc(C.Structure):
+    _fields_ = _BASE + [("argmax", C.c_char_p), ("mode", C.c_int32), ("global_pooling", C.c_int8), ("input_offset", c_tensor),
+                        ("stride", c_tensor), ("size", c_tensor), ("with_output_size", C.c_uint32), ("output_size", c_tensor)]
 
 
 _ELTW = [("output_calibration_factors", C.c_char_p), ("output_quantization_factor", C.c_float), ("mode", C.c_int32),
@@ -237,6 +246,7 @@ SIGNATURES = {
     "cldnn_eltwise_type_id": (C.c_void_p, [_ST]),
     "cldnn_convolution_type_id": (C.c_void_p, [_ST]),
     "cldnn_fused_conv_eltwise_type_id": (C.c_void_p, [_ST]),
+    "cldnn_pooling_type_id": (C.c_void_p, [_ST]),
 }
 
 _lib = None
@@ -520,6 +530,24 @@ class activation(_primitive):  # noqa: N801
         d.activation_func = func
         d.additional_params = c_act_params(*params)
         d.additional_params_input = b""
+
+
+class pooling(_primitive):  # noqa: N801
+    """pooling(id, input, mode, size, stride, input_offset) or, without a size, global pooling over the whole plane;
+    output_size = the reference's create_with_output_size (api/CPP/pooling.hpp:59-190)."""
+    type_fn = "cldnn_pooling_type_id"
+
+    def __init__(self, prim_id, inp, mode, size=None, stride=None, input_offset=None, output_size=None, output_padding=None):
+        d = c_pooling_desc()
+        self._base(d, prim_id, [inp], output_padding)
+        d.argmax = b""
+        d.mode = mode
+        d.global_pooling = 1 if size is None else 0
+        d.size = size if size is not None else tensor(0, 0, 0, 0, 0)
+        d.stride = stride if stride is not None else tensor(1, 1, 1, 1)
+        d.input_offset = input_offset if input_offset is not None else tensor(0, 0, 0, 0, 0)
+        d.with_output_size = 0 if output_size is None else 1
+        d.output_size = output_size if output_size is not None else tensor(0, 0, 0, 0, 0)
 
 
 def _eltw_fields(e, keep, output_calibration_factors, oqf, mode, with_activation, slope, stride):

@@ -394,4 +394,24 @@ cldnn_hip_status cldnn_hip_eltwise_sum(cldnn_hip_engine e, const void* a_dev, co
     });
 }
 
+cldnn_hip_status cldnn_hip_pooling(cldnn_hip_engine e, const cldnn_hip_pooling_desc* desc, const void* input_dev, void* output_dev)
+{
+    return guarded([&] {
+        CHIP_REQUIRE(e && desc && input_dev && output_dev, CLDNN_HIP_INVALID_ARG, "null argument");
+        e->make_current();
+        launch_pooling(e->stream, *desc, input_dev, output_dev);
+    });
+}
+
+int32_t cldnn_hip_pooling_out_extent(int32_t in, int32_t pad, int32_t size, int32_t stride)
+{
+    if (in <= 0 || size <= 0 || stride <= 0) return 0;
+    const int off = -pad, extend = size > stride ? size : stride;
+    // the last window may reach past the padded input once ...
+    const int once = 2 * off + extend <= in + stride - 1 ? (in - 2 * off - extend + stride - 1) / stride + 1 : 1;
+    // ... but has to start inside input + leading padding
+    const int any = off <= in - 1 ? (in - off - 1) / stride + 1 : 1;
+    return once < any ? once : any;
+}
+
 }  // extern "C"

@@ -117,6 +117,38 @@ __device__ __forceinline__ void interleave_step()
     }
 }
 
+// A load whose value is never used: it brings the line towards the CU while other work runs, so that the real load
+// later hits in cache.  The loaded register must stay reserved until the load has landed: keep_until_here(token) goes
+// behind a point where younger loads have been waited for (loads complete in order).
+__device__ __forceinline__ int touch_line(const void* p)
+{
+    int token;
+    asm volatile("global_load_dword %0, %1, off" : "=v"(token) : "v"(p) : "memory");
+    return token;
+}
+__device__ __forceinline__ void keep_until_here(int token) { asm volatile("" ::"v"(token)); }
+
+// The epilogue's per-feature factors of features [f_base, f_base + BN) (BN <= 128): one touch covers 512 bytes.
+struct EarlyTouch {
+    int t0, t1;
+};
+template <int BN, int EPI, class Args>
+__device__ __forceinline__ EarlyTouch touch_scales(const Args& a, int f_base, int lane)
+{
+    EarlyTouch e{0, 0};
+    if constexpr (EPI == EPI_KIND_RELU || EPI == EPI_KIND_FUSED || EPI == EPI_KIND_LINEAR) {
+        const int f = f_base + ((lane * 2) & (BN - 1));
+        e.t0 = touch_line(a.epi.calib + f);
+        if constexpr (EPI == EPI_KIND_FUSED) e.t1 = touch_line(a.epi.eltw_calib + f);
+    }
+    return e;
+}
+__device__ __forceinline__ void keep_until_here(const EarlyTouch& e)
+{
+    keep_until_here(e.t0);
+    keep_until_here(e.t1);
+}
+
 // Uniform table lookups go through the scalar data path (constant address space): a vector load here
 // would sit in the same in-order counter as the prefetched operand loads and force them to drain.
 typedef const int32_t __attribute__((address_space(4))) * const_i32_ptr;
@@ -584,6 +616,7 @@ __global__ void __launch_bounds__(256 * KG) conv_bdir_kernel(MfmaArgs a)
         for (int nt = 0; nt < NT; ++nt) acc[mt][nt] = init;
     }
     const v4i xm = {(int)a.xor_mask, (int)a.xor_mask, (int)a.xor_mask, (int)a.xor_mask};
+    const EarlyTouch early = touch_scales<BN, EPI>(a, ntile * BN, lane);
 
     extern __shared__ __align__(16) unsigned char smem[];
     v4i* ldsA = reinterpret_cast<v4i*>(smem) + grp * (3 * 4 * BN);  // per group: [3][4 * BN]
@@ -697,6 +730,7 @@ __global__ void __launch_bounds__(256 * KG) conv_bdir_kernel(MfmaArgs a)
         }
     }
 
+    keep_until_here(early);
     if constexpr (KG > 1) {
         // partial sums of groups 1.. go to LDS as [group - 1][wave][register][lane]; group 0 adds them up
         constexpr int REGS = MT * NT * 4;

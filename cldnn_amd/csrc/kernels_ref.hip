@@ -136,7 +136,10 @@ struct ReorderArgs {
     int dst_fs_fill;  // features physically present in dst beyond F (zero-filled), blocked formats only
 };
 
-__device__ __forceinline__ float f32_to_int_round(float v) { return round_half_away(v); }
+// float -> integer in a reorder is the reference's convert_char / convert_uchar / convert_int: towards zero
+// (kernel_selector/core/common/jitter.cpp:483,497,511; cl_kernels/reorder_data.cl:142).  Values outside the target
+// range, which OpenCL leaves undefined, saturate here.
+__device__ __forceinline__ float f32_to_int_round(float v) { return truncf(v); }
 
 __global__ void __launch_bounds__(256) reorder_kernel(ReorderArgs a, const void* __restrict__ src, void* __restrict__ dst)
 {

@@ -70,6 +70,11 @@ class ConvDesc(C.Structure):
     ]
 
 
+class PoolingDesc(C.Structure):
+    _fields_ = [("input", Tensor), ("output", Tensor)] + [(n, C.c_int32) for n in (
+        "mode", "divider", "size_y", "size_x", "stride_y", "stride_x", "pad_y", "pad_x")]
+
+
 class ConvInfo(C.Structure):
     _fields_ = [
         ("impl", C.c_int32), ("tile_index", C.c_int32), ("tile_pixels", C.c_int32), ("tile_ofm", C.c_int32),
@@ -141,6 +146,8 @@ SIGNATURES = {
     "cldnn_hip_conv_accumulators": (C.c_int32, [C.c_void_p, C.c_void_p, C.c_void_p]),
     "cldnn_hip_conv_get_info": (C.c_int32, [C.c_void_p, C.POINTER(ConvInfo)]),
     "cldnn_hip_conv_out_extent": (C.c_int32, [C.c_int32] * 5),
+    "cldnn_hip_pooling": (C.c_int32, [C.c_void_p, C.POINTER(PoolingDesc), C.c_void_p, C.c_void_p]),
+    "cldnn_hip_pooling_out_extent": (C.c_int32, [C.c_int32] * 4),
     "cldnn_hip_tile_config_count": (C.c_int32, []),
     "cldnn_hip_tile_config_name": (C.c_char_p, [C.c_int32]),
 }
@@ -237,6 +244,38 @@ class Buffer:
 
 def reorder(engine, src, dst):
     check(lib().cldnn_hip_reorder(engine.h, src.ptr, C.byref(src.tensor), dst.ptr, C.byref(dst.tensor)))
+
+
+POOL_MAX, POOL_AVERAGE = 0, 1
+POOL_DIV_FIXED, POOL_DIV_VALID, POOL_DIV_PADDED = 0, 1, 2
+
+
+def pool_forward(engine, x, mode, size, stride=(1, 1), pad=(0, 0), *, fmt="bfyx", in_pad=(0, 0), out_pad=(0, 0), out_size=None,
+                 global_pooling=False):
+    """numpy in, numpy out through cldnn_hip_pooling; arguments as oracle.refconv.pool (mode "max" / "average" /
+    "average_no_padding", (y, x) pairs)."""
+    L = lib()
+    x = np.ascontiguousarray(x)
+    xin = upload(engine, x, fmt, in_pad)
+    t = xin.tensor
+    if global_pooling:
+        size = (t.y, t.x)
+    if out_size is None:
+        out_size = (L.cldnn_hip_pooling_out_extent(t.y, pad[0], size[0], stride[0]),
+                    L.cldnn_hip_pooling_out_extent(t.x, pad[1], size[1], stride[1]))
+    d = PoolingDesc()
+    d.input = t
+    d.output = Tensor.make(t.dtype, t.format, t.b, t.f, out_size[0], out_size[1], out_pad[0], out_pad[1])
+    d.mode = POOL_MAX if mode == "max" else POOL_AVERAGE
+    overhang = (out_size[0] - 1) * stride[0] + size[0] > t.y + 2 * pad[0] or (out_size[1] - 1) * stride[1] + size[1] > t.x + 2 * pad[1]
+    d.divider = POOL_DIV_VALID if mode == "average_no_padding" else (POOL_DIV_PADDED if mode == "average" and overhang else POOL_DIV_FIXED)
+    d.size_y, d.size_x, d.stride_y, d.stride_x, d.pad_y, d.pad_x = size[0], size[1], stride[0], stride[1], pad[0], pad[1]
+    out = Buffer(engine, d.output)
+    check(L.cldnn_hip_pooling(engine.h, C.byref(d), xin.ptr, out.ptr))
+    res = download(engine, out)
+    out.close()
+    xin.close()
+    return res
 
 
 def upload(engine, arr, fmt="bfyx", pad=(0, 0)):

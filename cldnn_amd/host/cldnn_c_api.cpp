@@ -14,6 +14,7 @@ cldnn_hip_tensor to_hip(const cldnn_layout& l);
 size_t layout_bytes(const cldnn_layout& l);
 cldnn_tensor make_tensor(int b, int f, int x, int y);
 int hip_activation_code(int32_t f);
+cldnn_hip_pooling_desc pooling_descriptor(const node* n);
 void build_program(cldnn_program_impl* prog, cldnn_topology_impl* topo, const std::vector<std::string>& outputs);
 std::string describe_node(const node* n);
 std::string describe_program(const cldnn_program_impl* prog);
@@ -147,6 +148,12 @@ static void execute(cldnn_network_impl* net, cldnn_event* deps, size_t ndeps)
             hip_check(cldnn_hip_reorder(eng->h, in->device_ptr(), &it, out->device_ptr(), &ot));
             break;
         }
+        case prim_type::pooling: {
+            cldnn_memory_impl* in = mem_of(n->deps[0]);
+            cldnn_hip_pooling_desc pd = pooling_descriptor(n);
+            hip_check(cldnn_hip_pooling(eng->h, &pd, in->device_ptr(), out->device_ptr()));
+            break;
+        }
         case prim_type::activation: {
             cldnn_memory_impl* in = mem_of(n->deps[0]);
             const cldnn_hip_tensor it = to_hip(n->deps[0]->out);
@@ -233,7 +240,7 @@ struct cldnn_primitive_type {
 static const cldnn_primitive_type g_types[] = {
     {prim_type::input_layout, "input_layout"}, {prim_type::data, "data"},       {prim_type::reorder, "reorder"},
     {prim_type::activation, "activation"},     {prim_type::eltwise, "eltwise"}, {prim_type::convolution, "convolution"},
-    {prim_type::fused_conv_eltwise, "fused_conv_eltwise"},
+    {prim_type::fused_conv_eltwise, "fused_conv_eltwise"}, {prim_type::pooling, "pooling"},
 };
 
 extern "C" {
@@ -251,6 +258,7 @@ TYPE_ID_FN(activation, 3)
 TYPE_ID_FN(eltwise, 4)
 TYPE_ID_FN(convolution, 5)
 TYPE_ID_FN(fused_conv_eltwise, 6)
+TYPE_ID_FN(pooling, 7)
 
 const char* cldnn_get_last_error_message() { return g_last_error.c_str(); }
 
@@ -291,6 +299,16 @@ void cldnn_add_primitive(cldnn_topology topology, const struct cldnn_primitive_d
             HOST_REQUIRE((!d->mean_subtract || !*d->mean_subtract) && d->subtract_per_feature.size == 0, CLDNN_INVALID_ARG,
                          "reorder with mean subtraction is not supported by this library");
             p->reorder_format = d->output_format;
+            break;
+        }
+        case prim_type::pooling: {
+            auto* d = reinterpret_cast<const cldnn_pooling_desc*>(dto);
+            HOST_REQUIRE(!d->argmax || !*d->argmax, CLDNN_INVALID_ARG, "pooling with an argmax output is not supported by this library");
+            HOST_REQUIRE(d->mode == cldnn_pooling_max || d->mode == cldnn_pooling_average || d->mode == cldnn_pooling_average_no_padding,
+                         CLDNN_INVALID_ARG, "pooling mode not supported by this library (max, average, average_no_padding)");
+            p->pool_mode = d->mode, p->pool_global = d->global_pooling != 0;
+            p->input_offset = d->input_offset, p->stride = d->stride, p->pool_size = d->size;
+            p->with_output_size = d->with_output_size != 0, p->output_size = d->output_size;
             break;
         }
         case prim_type::activation: {

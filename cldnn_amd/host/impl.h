@@ -62,7 +62,7 @@ struct ref {  // owning smart pointer for refcounted objects
     explicit operator bool() const { return p != nullptr; }
 };
 
-enum class prim_type { input_layout, data, reorder, activation, eltwise, convolution, fused_conv_eltwise };
+enum class prim_type { input_layout, data, reorder, activation, eltwise, convolution, fused_conv_eltwise, pooling };
 
 }  // namespace host
 
@@ -106,6 +106,10 @@ struct prim {
     // activation
     int32_t act_func = activation_none;
     float act_a = 0.f, act_b = 0.f;
+    // pooling (shares input_offset / stride / output_size / with_output_size with the convolution fields)
+    int32_t pool_mode = cldnn_pooling_max;
+    bool pool_global = false;
+    cldnn_tensor pool_size{};
     // eltwise / fused eltw part
     std::string eltw_calib;
     float eltw_oqf = 1.f;

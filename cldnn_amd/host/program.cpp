@@ -172,6 +172,39 @@ static conv_geom conv_geometry(const prim& p, const cldnn_layout& in, const cldn
     return g;
 }
 
+struct pool_geom {
+    int ky, kx, sy, sx, py, px, OH, OW, divider;
+};
+
+static pool_geom pooling_geometry(const prim& p, const cldnn_layout& in)
+{
+    pool_geom g{};
+    const int IW = in.size.sizes[2], IH = in.size.sizes[3];
+    g.kx = p.pool_global ? IW : spatial(p.pool_size, 0), g.ky = p.pool_global ? IH : spatial(p.pool_size, 1);
+    g.sx = spatial(p.stride, 0), g.sy = spatial(p.stride, 1);
+    const int ox = spatial(p.input_offset, 0), oy = spatial(p.input_offset, 1);
+    HOST_REQUIRE(g.sx > 0 && g.sy > 0, CLDNN_INVALID_ARG, "pooling: stride spatial X/Y must be positive");
+    HOST_REQUIRE(g.kx > 0 && g.ky > 0, CLDNN_INVALID_ARG, "pooling: window size spatial X/Y must be positive");
+    HOST_REQUIRE(2 * ox <= IW && 2 * oy <= IH, CLDNN_INVALID_ARG, "pooling: input offset is greater than the input data range");
+    HOST_REQUIRE(-ox <= g.kx && -oy <= g.ky, CLDNN_INVALID_ARG, "pooling: first window is outside of the image, reduce the input offset");
+    HOST_REQUIRE(p.input_offset.sizes[0] == 0 && p.input_offset.sizes[1] == 0, CLDNN_INVALID_ARG,
+                 "pooling: input offset in batch / feature is not supported");
+    HOST_REQUIRE(ox <= 0 && oy <= 0, CLDNN_INVALID_ARG, "pooling: positive input offsets are not supported");
+    g.px = -ox, g.py = -oy;
+    if (p.with_output_size) {
+        g.OW = spatial(p.output_size, 0), g.OH = spatial(p.output_size, 1);
+        HOST_REQUIRE(g.OW > 0 && g.OH > 0, CLDNN_INVALID_ARG, "pooling: user-defined output size must be positive");
+    } else {
+        g.OW = cldnn_hip_pooling_out_extent(IW, g.px, g.kx, g.sx);
+        g.OH = cldnn_hip_pooling_out_extent(IH, g.py, g.ky, g.sy);
+    }
+    // divisor of an average (reference src/gpu/pooling_gpu.cpp:36-52,100-108)
+    const bool overhang = (g.OW - 1) * g.sx + g.kx > 2 * g.px + IW || (g.OH - 1) * g.sy + g.ky > 2 * g.py + IH;
+    g.divider = p.pool_mode == cldnn_pooling_average_no_padding ? CLDNN_HIP_POOL_DIV_VALID
+                : (p.pool_mode == cldnn_pooling_average && overhang ? CLDNN_HIP_POOL_DIV_PADDED : CLDNN_HIP_POOL_DIV_FIXED);
+    return g;
+}
+
 static node* dep_named(node* n, const std::string& id)
 {
     for (node* d : n->deps)
@@ -195,6 +228,15 @@ static void calc_layout(node* n)
     case prim_type::activation: {
         n->out = n->deps[0]->out;
         if (p.out_dt.enabled) n->out.data_type = p.out_dt.data_type;
+        break;
+    }
+    case prim_type::pooling: {
+        // reference src/pooling.cpp:30-117
+        const cldnn_layout& in = n->deps[0]->out;
+        HOST_REQUIRE(!p.out_dt.enabled, CLDNN_INVALID_ARG, "output data type forcing is not supported for pooling");
+        const pool_geom g = pooling_geometry(p, in);
+        n->out = in;
+        n->out.size = make_tensor(in.size.sizes[0], in.size.sizes[1], g.OW, g.OH);
         break;
     }
     case prim_type::eltwise: {
@@ -537,6 +579,19 @@ static int hip_act(int32_t f)
 }
 int hip_activation_code(int32_t f) { return hip_act(f); }
 
+// pooling node -> descriptor of the C-ABI call (reference src/gpu/pooling_gpu.cpp:78-130)
+cldnn_hip_pooling_desc pooling_descriptor(const node* n)
+{
+    const prim& p = *n->p;
+    const pool_geom g = pooling_geometry(p, n->deps[0]->out);
+    cldnn_hip_pooling_desc d{};
+    d.input = to_hip(n->deps[0]->out), d.output = to_hip(n->out);
+    d.mode = p.pool_mode == cldnn_pooling_max ? CLDNN_HIP_POOL_MAX : CLDNN_HIP_POOL_AVERAGE;
+    d.divider = g.divider;
+    d.size_y = g.ky, d.size_x = g.kx, d.stride_y = g.sy, d.stride_x = g.sx, d.pad_y = g.py, d.pad_x = g.px;
+    return d;
+}
+
 // convolution / fused_conv_eltwise -> one cldnn_hip_conv object (reference convolution_gpu.cpp:71-162)
 static void compile_conv(cldnn_program_impl* prog, node* n)
 {
@@ -707,7 +762,7 @@ static std::string four(const int32_t* s)
 // one node as JSON; sizes and paddings are [b, f, x, y] like cldnn_tensor::sizes
 std::string describe_node(const node* n)
 {
-    static const char* tn[] = {"input_layout", "data", "reorder", "activation", "eltwise", "convolution", "fused_conv_eltwise"};
+    static const char* tn[] = {"input_layout", "data", "reorder", "activation", "eltwise", "convolution", "fused_conv_eltwise", "pooling"};
     const prim& p = *n->p;
     std::string s = "{\"id\":\"" + p.id + "\",\"type\":\"" + tn[(int)p.type] + "\",\"org_id\":\"" + n->org_id + "\",\"deps\":[";
     for (size_t i = 0; i < n->deps.size(); ++i) s += std::string(i ? "," : "") + "\"" + n->deps[i]->p->id + "\"";

@@ -1,7 +1,7 @@
 /*
  * Descriptor structures ("dto") of the primitives a convolution topology needs.  Field order and
  * meaning follow the reference headers: api/C/input_layout.h, data.h, reorder.h, activation.h,
- * eltwise.h, convolution.h:36-74 and api_extension/C/fused_conv_eltwise.h:35-97.
+ * eltwise.h, pooling.h, convolution.h:36-74 and api_extension/C/fused_conv_eltwise.h:35-97.
  */
 #ifndef CLDNN_PRIMITIVES_H
 #define CLDNN_PRIMITIVES_H
@@ -35,6 +35,27 @@ cldnn_activation_additional_params additional_params;
 cldnn_primitive_id additional_params_input; /* not supported: must be empty */
 CLDNN_END_PRIMITIVE_DESC(activation)
 CLDNN_DECLARE_PRIMITIVE_TYPE_ID(activation);
+
+/* pooling (reference api/C/pooling.h:33-69); the argmax and bilinear modes are not implemented */
+typedef enum {
+    cldnn_pooling_max,
+    cldnn_pooling_average,
+    cldnn_pooling_average_no_padding,
+    cldnn_pooling_max_with_argmax,
+    cldnn_pooling_bilinear
+} cldnn_pooling_mode;
+
+CLDNN_BEGIN_PRIMITIVE_DESC(pooling)
+cldnn_primitive_id argmax;    /* not supported: must be empty */
+int32_t mode;                 /* cldnn_pooling_mode */
+int8_t global_pooling;        /* window = the whole input plane */
+cldnn_tensor input_offset;    /* negative = zero padding */
+cldnn_tensor stride;
+cldnn_tensor size;
+uint32_t with_output_size;
+cldnn_tensor output_size;
+CLDNN_END_PRIMITIVE_DESC(pooling)
+CLDNN_DECLARE_PRIMITIVE_TYPE_ID(pooling);
 
 typedef enum {
     cldnn_eltwise_sum,

@@ -539,6 +539,53 @@ private:
     mutable id_list _in;
 };
 
+enum class pooling_mode : int32_t {
+    max = cldnn_pooling_max,
+    average = cldnn_pooling_average,
+    average_no_padding = cldnn_pooling_average_no_padding,
+    max_with_argmax = cldnn_pooling_max_with_argmax,
+    bilinear = cldnn_pooling_bilinear
+};
+
+// pooling(id, input, mode, size, stride, input_offset), with a user-given output size, or global over the whole plane
+// (reference api/CPP/pooling.hpp:59-190); the argmax forms are not implemented
+struct pooling : primitive {
+    pooling_mode mode;
+    bool global_pooling;
+    tensor input_offset{0}, stride{1}, size{0}, output_size{0};
+    bool with_output_size = false;
+    pooling(const primitive_id& id, const primitive_id& input, pooling_mode mode, const tensor& size, const tensor& stride,
+            const tensor& input_offset = {0, 0, 0, 0}, const padding& output_padding = padding())
+        : primitive(id, {input}, output_padding), mode(mode), global_pooling(false), input_offset(input_offset), stride(stride), size(size) {}
+    pooling(const primitive_id& id, const primitive_id& input, pooling_mode mode, const tensor& size, const tensor& stride,
+            const tensor& input_offset, tensor output_size, const padding& output_padding = padding())
+        : primitive(id, {input}, output_padding), mode(mode), global_pooling(false), input_offset(input_offset), stride(stride), size(size),
+          output_size(output_size), with_output_size(true) {}
+    pooling(const primitive_id& id, const primitive_id& input, pooling_mode mode, const padding& output_padding = padding())
+        : primitive(id, {input}, output_padding), mode(mode), global_pooling(true) {}
+    static pooling create_with_output_size(const primitive_id& id, const primitive_id& input, tensor output_size, pooling_mode mode,
+                                           const tensor& size, const tensor& stride, const tensor& input_offset = {0, 0, 0, 0},
+                                           const padding& output_padding = padding())
+    {
+        return pooling(id, input, mode, size, stride, input_offset, output_size, output_padding);
+    }
+    CLDNN_CPP_TYPE_ID(pooling)
+    const ::cldnn_primitive_desc* get_dto() const override
+    {
+        fill_base(_d, type_id(), _in);
+        _d.argmax = "";
+        _d.mode = static_cast<int32_t>(mode);
+        _d.global_pooling = global_pooling;
+        _d.input_offset = input_offset, _d.stride = stride, _d.size = size;
+        _d.with_output_size = with_output_size, _d.output_size = output_size;
+        return reinterpret_cast<const ::cldnn_primitive_desc*>(&_d);
+    }
+
+private:
+    mutable cldnn_pooling_desc _d{};
+    mutable id_list _in;
+};
+
 enum class eltwise_mode : int32_t { sum = cldnn_eltwise_sum, sub = cldnn_eltwise_sub, max = cldnn_eltwise_max, prod = cldnn_eltwise_prod };
 
 struct eltwise : primitive {

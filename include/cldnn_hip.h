@@ -145,7 +145,8 @@ int64_t cldnn_hip_tensor_offset(const cldnn_hip_tensor* t, int32_t b, int32_t f,
 
 /* layout / precision change; replaces the reorder kernels the path needs
  * (reference src/gpu/reorder_gpu.cpp, kernel_selector/core/cl_kernels/reorder_data.cl).
- * f32 -> int8 conversions saturate and round half away from zero; padding of dst is left untouched. */
+ * f32 -> integer conversions go towards zero like the reference's convert_char (kernel_selector/core/common/jitter.cpp:483)
+ * and saturate where OpenCL leaves the result undefined; padding of dst is left untouched. */
 cldnn_hip_status cldnn_hip_reorder(cldnn_hip_engine e, const void* src_dev, const cldnn_hip_tensor* src,
                                    void* dst_dev, const cldnn_hip_tensor* dst);
 
@@ -163,6 +164,32 @@ cldnn_hip_status cldnn_hip_eltwise_sum(cldnn_hip_engine e, const void* a_dev, co
                                        const void* b_dev, const cldnn_hip_tensor* b, void* dst_dev,
                                        const cldnn_hip_tensor* dst, int32_t quantized, const float* calib_dev,
                                        float output_quantization_factor, int32_t activation, float m, float n);
+
+/* ------------------------------------------------------------------ pooling
+ * The layers between the convolutions of an int8 network: sliding-window maximum / average.  Replaces the pooling
+ * kernels (reference src/gpu/pooling_gpu.cpp:60-160, kernel_selector/core/cl_kernels/pooling_gpu_int8_ref.cl:15-140,
+ * pooling_gpu_ref.cl): int8 data accumulate in int and an average is round(sum / count), half away from zero; float
+ * data accumulate in float.  Taps outside the input are skipped; the data type and the feature count are kept. */
+enum { CLDNN_HIP_POOL_MAX = 0, CLDNN_HIP_POOL_AVERAGE = 1 };
+enum {
+    CLDNN_HIP_POOL_DIV_FIXED = 0,  /* average divides by the window size (pooling_mode::average) */
+    CLDNN_HIP_POOL_DIV_VALID = 1,  /* ... by the number of taps inside the input (average_no_padding) */
+    CLDNN_HIP_POOL_DIV_PADDED = 2  /* ... by the window clipped to input + padding (average whose last window overhangs) */
+};
+typedef struct {
+    cldnn_hip_tensor input, output;
+    int32_t mode;                 /* CLDNN_HIP_POOL_* */
+    int32_t divider;              /* CLDNN_HIP_POOL_DIV_* */
+    int32_t size_y, size_x;
+    int32_t stride_y, stride_x;
+    int32_t pad_y, pad_x;         /* = max(-input_offset, 0) */
+} cldnn_hip_pooling_desc;
+/* asynchronous on the engine stream; device pointers */
+cldnn_hip_status cldnn_hip_pooling(cldnn_hip_engine e, const cldnn_hip_pooling_desc* desc, const void* input_dev,
+                                   void* output_dev);
+/* output extent along one axis: the last window may overhang the padded input once but must start inside the data
+ * (reference src/include/sliding_window_utils.h:135-186, swor_mode::exceed_once_data; src/pooling.cpp:110-116) */
+int32_t cldnn_hip_pooling_out_extent(int32_t in, int32_t pad, int32_t size, int32_t stride);
 
 /* ------------------------------------------------------------------ convolution
  * One object per convolution / fused_conv_eltwise node; replaces

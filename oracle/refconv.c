@@ -466,3 +466,64 @@ int rc_conv(const rc_desc* d, const void* in, const void* weights, const void* b
     }
     return rc;
 }
+
+/* ------------------------------------------------------------------------------------------------ pooling */
+int rc_pool_out_extent(int in, int pad, int size, int stride)
+{
+    int off = -pad; /* the primitive's input_offset */
+    int extend = size > stride ? size : stride;
+    int once = 2 * off + extend <= in + stride - 1 ? (in - 2 * off - extend + stride - 1) / stride + 1 : 1;
+    int any = off <= in - 1 ? (in - off - 1) / stride + 1 : 1;
+    return once < any ? once : any;
+}
+
+int rc_pool(const rc_pool_desc* d, const void* in, void* out)
+{
+    if (!(d->dt == RC_S8 || d->dt == RC_U8 || d->dt == RC_F32) || d->mode < 0 || d->mode > 1) return -1;
+    for (int b = 0; b < d->B; ++b)
+        for (int f = 0; f < d->F; ++f) {
+            int64_t ib = ((int64_t)b * d->F + f) * d->IH * d->IW, ob = ((int64_t)b * d->F + f) * d->OH * d->OW;
+            for (int y = 0; y < d->OH; ++y)
+                for (int x = 0; x < d->OW; ++x) {
+                    int oy = y * d->sy - d->pad_y, ox = x * d->sx - d->pad_x;
+                    if (oy + d->ky < 0 || oy >= d->IH || ox + d->kx < 0 || ox >= d->IW) continue;
+                    int valid = 0;
+                    int ri = d->mode == 0 ? -128 : 0;
+                    float rf = d->mode == 0 ? -3.402823466e+38f : 0.0f;
+                    for (int j = 0; j < d->ky; ++j) {
+                        int iy = oy + j;
+                        if (iy < 0 || iy >= d->IH) continue;
+                        for (int i = 0; i < d->kx; ++i) {
+                            int ix = ox + i;
+                            if (ix < 0 || ix >= d->IW) continue;
+                            int64_t at = ib + (int64_t)iy * d->IW + ix;
+                            if (d->dt == RC_F32) {
+                                float v = ((const float*)in)[at];
+                                rf = d->mode == 0 ? (v > rf ? v : rf) : rf + v;
+                            } else {
+                                int v = d->dt == RC_U8 ? (int)((const uint8_t*)in)[at] : (int)((const int8_t*)in)[at];
+                                ri = d->mode == 0 ? (v > ri ? v : ri) : ri + v;
+                            }
+                            ++valid;
+                        }
+                    }
+                    int n = d->ky * d->kx;
+                    if (d->divider == 1) n = valid > 0 ? valid : 1;
+                    if (d->divider == 2) {
+                        int hend = oy + d->ky < d->IH + d->pad_y ? oy + d->ky : d->IH + d->pad_y;
+                        int wend = ox + d->kx < d->IW + d->pad_x ? ox + d->kx : d->IW + d->pad_x;
+                        n = (hend - oy) * (wend - ox);
+                        if (n < 1) n = 1;
+                    }
+                    int64_t oi = ob + (int64_t)y * d->OW + x;
+                    if (d->dt == RC_F32) {
+                        ((float*)out)[oi] = d->mode == 0 ? rf : rf / (float)n;
+                    } else {
+                        if (d->mode == 1) ri = (int)rc_round_half_away((float)ri / (float)n);
+                        if (d->dt == RC_U8) ((uint8_t*)out)[oi] = (uint8_t)ri;
+                        else ((int8_t*)out)[oi] = (int8_t)ri;
+                    }
+                }
+        }
+    return 0;
+}

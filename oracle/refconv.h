@@ -98,6 +98,26 @@ int rc_conv(const rc_desc* d, const void* in, const void* weights, const void* b
 double rc_epilogue(const rc_desc* d, int32_t acc, int f, const void* bias, const float* wqf,
                    const float* calib, double eltw_val, const float* eltw_calib);
 
+/*
+ * Pooling over dense bfyx tensors (the layers between the convolutions of an int8 network).  Follows
+ * kernel_selector/core/cl_kernels/pooling_gpu_int8_ref.cl:15-140 for s8 / u8 (int accumulator starting at CHAR_MIN
+ * for the maximum, average = round(sum / count) half away from zero) and pooling_gpu_ref.cl for f32 (float
+ * accumulator, plain division); taps outside the input are skipped, a window wholly outside leaves the output as it
+ * is.  mode: 0 max, 1 average.  divider: 0 window size, 1 taps inside the input, 2 window clipped to input + padding
+ * (src/gpu/pooling_gpu.cpp:36-52,100-108).
+ */
+typedef struct {
+    int dt;
+    int B, F, IH, IW, OH, OW;
+    int ky, kx, sy, sx, pad_y, pad_x;
+    int mode, divider;
+} rc_pool_desc;
+int rc_pool(const rc_pool_desc* d, const void* in, void* out);
+/* Output extent of a pooling window along one axis (sliding_window_utils.h:135-186, swor_mode::exceed_once_data;
+ * src/pooling.cpp:110-116): min(the last window may overhang the padded input once, every window starts inside
+ * input + leading padding); degenerate value 1. */
+int rc_pool_out_extent(int in, int pad, int size, int stride);
+
 /* Helpers exposed for tests. */
 float rc_round_half_away(float x);
 int   rc_threads_available(void);

@@ -40,6 +40,11 @@ class Desc(C.Structure):
     )
 
 
+class PoolDesc(C.Structure):
+    _fields_ = [(n, C.c_int) for n in ("dt", "B", "F", "IH", "IW", "OH", "OW", "ky", "kx", "sy", "sx", "pad_y", "pad_x", "mode",
+                                       "divider")]
+
+
 def build(force=False):
     """Compile oracle/librefconv.so with the Makefile beside it."""
     so = os.path.join(_HERE, "librefconv.so")
@@ -66,6 +71,10 @@ def lib():
         L.rc_round_half_away.restype = C.c_float
         L.rc_round_half_away.argtypes = [C.c_float]
         L.rc_threads_available.restype = C.c_int
+        L.rc_pool.restype = C.c_int
+        L.rc_pool.argtypes = [C.POINTER(PoolDesc), C.c_void_p, C.c_void_p]
+        L.rc_pool_out_extent.restype = C.c_int
+        L.rc_pool_out_extent.argtypes = [C.c_int] * 4
         _LIB = L
     return _LIB
 
@@ -158,3 +167,36 @@ def conv(x, w, bias=None, wqf=None, calib=None, *, stride=(1, 1), pad=(0, 0), di
     if rc != 0:
         raise ValueError("refconv: unsupported combination")
     return (out, acc) if want_acc else out
+
+
+POOL_MODE = {"max": 0, "average": 1, "average_no_padding": 1}
+
+
+def pool_out_extent(n, pad, size, stride):
+    return lib().rc_pool_out_extent(n, pad, size, stride)
+
+
+def pool(x, mode, size, stride=(1, 1), pad=(0, 0), out_size=None, global_pooling=False):
+    """Reference pooling on a dense bfyx array; mode "max" / "average" / "average_no_padding"; size/stride/pad are (y, x);
+    pad = -input_offset.  The divider of an average follows src/gpu/pooling_gpu.cpp:36-52,100-108: the window size, unless
+    the last window reaches past input + 2 * padding (then the window clipped to input + padding); average_no_padding
+    counts the taps inside the input."""
+    x = np.ascontiguousarray(x)
+    B, F, IH, IW = x.shape
+    if global_pooling:
+        size = (IH, IW)
+    if out_size is None:
+        OH, OW = pool_out_extent(IH, pad[0], size[0], stride[0]), pool_out_extent(IW, pad[1], size[1], stride[1])
+    else:
+        OH, OW = out_size
+    d = PoolDesc()
+    d.dt = DT_OF[x.dtype]
+    d.B, d.F, d.IH, d.IW, d.OH, d.OW = B, F, IH, IW, OH, OW
+    d.ky, d.kx, d.sy, d.sx, d.pad_y, d.pad_x = size[0], size[1], stride[0], stride[1], pad[0], pad[1]
+    d.mode = POOL_MODE[mode]
+    overhang = (OH - 1) * stride[0] + size[0] > IH + 2 * pad[0] or (OW - 1) * stride[1] + size[1] > IW + 2 * pad[1]
+    d.divider = 1 if mode == "average_no_padding" else (2 if mode == "average" and overhang else 0)
+    out = np.zeros((B, F, OH, OW), x.dtype)
+    if lib().rc_pool(C.byref(d), _ptr(x), _ptr(out)) != 0:
+        raise ValueError("unsupported pooling")
+    return out

@@ -386,12 +386,14 @@ def test_reorder_round_trip_and_layout_independence(eng, fmt):
     np.testing.assert_array_equal(a, b_)
 
 
-def test_reorder_f32_to_int8_rounds_half_away_and_saturates(eng):
-    v = np.array([0.5, 1.5, -0.5, -1.5, 2.4, 300.0, -300.0, 127.5], np.float32).reshape(1, 8, 1, 1)
+def test_reorder_f32_to_int8_goes_towards_zero_and_saturates(eng):
+    """the reference's reorder converts with convert_char (jitter.cpp:483): towards zero; its pooling test relies on
+    9.5 -> 9 (pooling_gpu_test.cpp:264-309).  Out-of-range values saturate here."""
+    v = np.array([0.5, 1.5, -0.5, -1.5, 2.4, 300.0, -300.0, 127.5, 9.5, -6.99], np.float32).reshape(1, 10, 1, 1)
     src = hip.upload(eng, v)
-    dst = hip.Buffer(eng, hip.Tensor.make("s8", "bfyx", 1, 8, 1, 1))
+    dst = hip.Buffer(eng, hip.Tensor.make("s8", "bfyx", 1, 10, 1, 1))
     hip.reorder(eng, src, dst)
-    np.testing.assert_array_equal(hip.download(eng, dst).ravel(), [1, 2, -1, -2, 2, 127, -128, 127])
+    np.testing.assert_array_equal(hip.download(eng, dst).ravel(), [0, 1, 0, -1, 2, 127, -128, 127, 9, -6])
 
 
 def test_lock_unlock_and_events(eng):
