@@ -113,6 +113,12 @@ class c_pooling_desc(C.Structure):
                         ("stride", c_tensor), ("size", c_tensor), ("with_output_size", C.c_uint32), ("output_size", c_tensor)]
 
 
+class c_fully_connected_desc(C.Structure):
+    _fields_ = _BASE + [("with_activation", C.c_uint32), ("activation_negative_slope", C.c_float), ("weights", C.c_char_p),
+                        ("bias", C.c_char_p), ("weights_quantization_factors", C.c_char_p), ("output_calibration_factors", C.c_char_p),
+                        ("input_quantization_factor", C.c_float), ("output_quantization_factor", C.c_float)]
+
+
 _ELTW = [("output_calibration_factors", C.c_char_p), ("output_quantization_factor", C.c_float), ("mode", C.c_int32),
          ("coefficients", c_float_arr), ("with_activation", C.c_uint32), ("activation_negative_slope", C.c_float),
          ("stride", c_tensor_arr)]
@@ -247,6 +253,7 @@ SIGNATURES = {
     "cldnn_convolution_type_id": (C.c_void_p, [_ST]),
     "cldnn_fused_conv_eltwise_type_id": (C.c_void_p, [_ST]),
     "cldnn_pooling_type_id": (C.c_void_p, [_ST]),
+    "cldnn_fully_connected_type_id": (C.c_void_p, [_ST]),
 }
 
 _lib = None
@@ -548,6 +555,22 @@ class pooling(_primitive):  # noqa: N801
         d.input_offset = input_offset if input_offset is not None else tensor(0, 0, 0, 0, 0)
         d.with_output_size = 0 if output_size is None else 1
         d.output_size = output_size if output_size is not None else tensor(0, 0, 0, 0, 0)
+
+
+class fully_connected(_primitive):  # noqa: N801
+    """fully_connected(id, input, weights, bias, [w_quantization_factor, [output_calibration_factors,] i_quantization_factor,
+    [o_quantization_factor]], with_activation, activation_slp) (reference api/CPP/fully_connected.hpp:60-150)."""
+    type_fn = "cldnn_fully_connected_type_id"
+
+    def __init__(self, prim_id, inp, weights, bias="", w_quantization_factor="", output_calibration_factors="",
+                 i_quantization_factor=1.0, o_quantization_factor=1.0, with_activation=False, activation_slp=0.0, output_padding=None):
+        d = c_fully_connected_desc()
+        self._base(d, prim_id, [inp], output_padding)
+        d.with_activation, d.activation_negative_slope = int(with_activation), activation_slp
+        d.weights, d.bias = weights.encode(), (bias or "").encode()
+        d.weights_quantization_factors = (w_quantization_factor or "").encode()
+        d.output_calibration_factors = (output_calibration_factors or "").encode()
+        d.input_quantization_factor, d.output_quantization_factor = i_quantization_factor, o_quantization_factor
 
 
 def _eltw_fields(e, keep, output_calibration_factors, oqf, mode, with_activation, slope, stride):

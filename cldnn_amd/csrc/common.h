@@ -69,6 +69,7 @@ struct Epilogue {
     float eltw_m, eltw_n;
     int32_t out_dt, eltw_dt, in_dt;
     int32_t round_even;
+    int32_t fc;              // quantized fully_connected form (see cldnn_hip_conv_desc.fully_connected)
 };
 
 }  // namespace chip

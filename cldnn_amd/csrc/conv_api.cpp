@@ -142,6 +142,12 @@ void build(cldnn_hip_conv c, const void* weights, const void* bias, const float*
     e.eltw_act = d.eltw_activation, e.eltw_m = d.eltw_activation_m, e.eltw_n = d.eltw_activation_n;
     e.out_dt = p.out_dt, e.eltw_dt = p.eltw_dt, e.in_dt = p.in_dt;
     e.round_even = d.round_to_even;
+    e.fc = (d.fully_connected && d.has_wqf && !d.fused) ? 1 : 0;
+    if (e.fc) {
+        CHIP_REQUIRE(p.OH == 1 && p.OW == 1 && p.FY == p.IH && p.FX == p.IW && p.py == 0 && p.px == 0, CLDNN_HIP_INVALID_ARG,
+                     "fully_connected: the filter must cover the whole input plane");
+        CHIP_REQUIRE(p.out_dt == CLDNN_HIP_S8, CLDNN_HIP_INVALID_ARG, "quantized fully_connected writes s8");
+    }
 
     // ---- kernel family
     const bool blocked = d.input.format == CLDNN_HIP_FMT_FS_B_YX_FSV16 && d.output.format == CLDNN_HIP_FMT_FS_B_YX_FSV16

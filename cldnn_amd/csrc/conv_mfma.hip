@@ -317,7 +317,7 @@ bool mfma_fast_epilogue(const ConvProblem& p, const Epilogue& e, const float* ca
                         FastEpi* out)
 {
     FastEpi F{};
-    if (e.mode != MODE_Q || e.round_even) return false;
+    if (e.mode != MODE_Q || e.round_even || e.fc) return false;
     if (e.bias) return false;  // an int32 bias is folded into the accumulator start; a float bias takes the long path
     if (!(e.out_dt == CLDNN_HIP_S8 || e.out_dt == CLDNN_HIP_U8)) return false;
     if (!(e.act == CLDNN_HIP_ACT_NONE || e.act == CLDNN_HIP_ACT_RELU || e.act == CLDNN_HIP_ACT_CLAMP)) return false;

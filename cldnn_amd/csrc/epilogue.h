@@ -95,6 +95,22 @@ __device__ __forceinline__ EpiOut finish(const Epilogue& e, float o)
 __device__ __forceinline__ EpiOut epilogue_generic(const Epilogue& e, int acc, int f, float eltw)
 {
     const bool out_fp = e.out_dt == CLDNN_HIP_F32;
+    if (e.mode == MODE_Q && e.fc) {
+        int v = acc;
+        if (e.bias) {
+            const float bv = e.bias_dt == CLDNN_HIP_F32 ? ((const float*)e.bias)[f] : (float)((const int*)e.bias)[f];
+            float x = (float)acc * e.wqf[f];
+            x = x * e.iqf;
+            x = x + bv;
+            x = x * (e.calib ? e.calib[f] : e.oqf);
+            v = (int)(signed char)(int)round_sel(x, e.round_even);
+        }
+        const int c = act_i(e.act, e.act_m, e.act_n, (int)(signed char)v);
+        EpiOut r;
+        r.i = (int)(signed char)c, r.f = (float)r.i;
+        if (e.out_dt == CLDNN_HIP_U8) r.i = r.i < 0 ? 0 : r.i;
+        return r;
+    }
     if (e.mode == MODE_Q) {
         if (e.bias && !e.bias_after) {
             int bv = e.bias_dt == CLDNN_HIP_F32 ? (int)((const float*)e.bias)[f] : ((const int*)e.bias)[f];

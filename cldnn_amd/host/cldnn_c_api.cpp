@@ -241,6 +241,8 @@ static const cldnn_primitive_type g_types[] = {
     {prim_type::input_layout, "input_layout"}, {prim_type::data, "data"},       {prim_type::reorder, "reorder"},
     {prim_type::activation, "activation"},     {prim_type::eltwise, "eltwise"}, {prim_type::convolution, "convolution"},
     {prim_type::fused_conv_eltwise, "fused_conv_eltwise"}, {prim_type::pooling, "pooling"},
+    // kept as a convolution node whose filter covers the input plane
+    {prim_type::convolution, "fully_connected"},
 };
 
 extern "C" {
@@ -259,6 +261,7 @@ TYPE_ID_FN(eltwise, 4)
 TYPE_ID_FN(convolution, 5)
 TYPE_ID_FN(fused_conv_eltwise, 6)
 TYPE_ID_FN(pooling, 7)
+TYPE_ID_FN(fully_connected, 8)
 
 const char* cldnn_get_last_error_message() { return g_last_error.c_str(); }
 
@@ -286,6 +289,25 @@ void cldnn_add_primitive(cldnn_topology topology, const struct cldnn_primitive_d
         p->inputs = ids_of(dto->input);
         p->output_padding = dto->output_padding;
         p->out_dt = dto->output_data_type;
+        if (dto->type == &g_types[8]) {
+            // fully_connected -> convolution node with the filter of the weights' own size (checked against the input when the
+            // program is built), stride 1, no padding (reference src/fully_connected.cpp:58-80, src/gpu/fully_connected_gpu.cpp)
+            auto* d = reinterpret_cast<const cldnn_fully_connected_desc*>(dto);
+            auto one = [](const char* s) { return s && *s ? std::vector<std::string>{s} : std::vector<std::string>{}; };
+            HOST_REQUIRE(!p->out_dt.enabled, CLDNN_INVALID_ARG, "output data type forcing is not supported for fully_connected");
+            p->fully_connected = true;
+            p->stride = make_tensor(1, 1, 1, 1), p->dilation = make_tensor(1, 1, 1, 1), p->input_offset = make_tensor(0, 0, 0, 0);
+            p->padding_above = make_tensor(0, 0, 0, 0), p->padding_below = make_tensor(0, 0, 0, 0);
+            p->with_activation = d->with_activation != 0, p->act_slope = d->activation_negative_slope;
+            p->split = 1, p->groups = 1;
+            p->weights = one(d->weights), p->bias = one(d->bias);
+            p->wqf = one(d->weights_quantization_factors), p->calib = one(d->output_calibration_factors);
+            p->iqf = d->input_quantization_factor, p->oqf = d->output_quantization_factor;
+            HOST_REQUIRE(p->weights.size() == 1, CLDNN_INVALID_ARG, "fully_connected needs weights");
+            topology->prims[p->id] = p;
+            topology->order.push_back(p->id);
+            return;
+        }
         switch (p->type) {
         case prim_type::input_layout: p->layout = reinterpret_cast<const cldnn_input_layout_desc*>(dto)->layout; break;
         case prim_type::data: {

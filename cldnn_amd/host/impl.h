@@ -127,6 +127,7 @@ struct prim {
     float iqf = 1.f, oqf = 1.f;
     float non_conv_scale = 1.f;
     bool second_input_in_output = false;
+    bool fully_connected = false;  // convolution node that stands for a fully_connected primitive
 };
 
 }  // namespace host

@@ -141,6 +141,9 @@ static conv_geom conv_geometry(const prim& p, const cldnn_layout& in, const cldn
     HOST_REQUIRE(w.size.sizes[1] * g.groups == g.IFM, CLDNN_DIMENSION_MISMATCH,
                  "weights input feature count (x groups) differs from the input's feature count");
     HOST_REQUIRE(g.OFM % g.groups == 0, CLDNN_DIMENSION_MISMATCH, "output features do not divide into groups");
+    if (p.fully_connected)
+        HOST_REQUIRE(g.FX == g.IW && g.FY == g.IH, CLDNN_DIMENSION_MISMATCH,
+                     "fully_connected: the weights' spatial size differs from the input's");
     g.sx = spatial(p.stride, 0), g.sy = spatial(p.stride, 1);
     g.dx = spatial(p.dilation, 0), g.dy = spatial(p.dilation, 1);
     // reference src/convolution.cpp:54-61
@@ -269,6 +272,11 @@ static void calc_layout(node* n)
         if (n->first_layer) n->out.format = cldnn_format_fs_b_yx_fsv16;  // b_fs_yx_fsv4 in, blocked out
         n->out.size = make_tensor(g.B, g.OFM, g.OW, g.OH);
         if (p.out_dt.enabled) n->out.data_type = p.out_dt.data_type;
+        if (p.fully_connected && in.format != cldnn_format_fs_b_yx_fsv16) {
+            // reference src/fully_connected.cpp:58-80: batch-innermost output for yxfb inputs and for bfyx inputs with batch > 1
+            const bool batch_last = in.format == cldnn_format_yxfb || (in.format == cldnn_format_bfyx && g.B > 1);
+            n->out.format = batch_last ? cldnn_format_yxfb : cldnn_format_bfyx;
+        }
         break;
     }
     }
@@ -370,7 +378,7 @@ static void fuse_conv_eltwise(cldnn_program_impl* prog)
 {
     std::vector<node*> convs;
     for (auto& u : prog->nodes)
-        if (u->p->type == prim_type::convolution) convs.push_back(u.get());
+        if (u->p->type == prim_type::convolution && !u->p->fully_connected) convs.push_back(u.get());
     for (node* c : convs) {
         if (c->users.size() != 1 || c->is_output) continue;
         node* e = c->users[0];
@@ -414,6 +422,13 @@ static void fuse_conv_eltwise(cldnn_program_impl* prog)
         }
         node* nf = add_node(prog, f, e->org_id);
         nf->user_format = e->user_format;
+        {
+            // the fused node executes where the eltwise did: a later block must still find its own closing convolution
+            // to be the later-executed input of its sum
+            auto self = std::move(prog->nodes.back());
+            prog->nodes.pop_back();
+            prog->nodes.insert(prog->nodes.begin() + position(prog, e), std::move(self));
+        }
         // dependencies: input, input2, weights, bias, wqf, calib, eltw calib
         nf->deps.push_back(c->deps[0]);
         nf->deps.push_back(other);
@@ -611,6 +626,7 @@ static void compile_conv(cldnn_program_impl* prog, node* n)
     d.stride_y = g.sy, d.stride_x = g.sx, d.dilation_y = g.dy, d.dilation_x = g.dx;
     d.pad_y = g.py, d.pad_x = g.px, d.groups = g.groups;
     d.pad_end_delta_y = g.ey, d.pad_end_delta_x = g.ex;
+    d.fully_connected = p.fully_connected ? 1 : 0;
     d.input_quantization_factor = p.iqf;
     d.output_quantization_factor = p.oqf;
     d.bias_dtype = CLDNN_HIP_NO_TYPE;
@@ -771,6 +787,7 @@ std::string describe_node(const node* n)
     s += ",\"size\":" + four(n->out.size.sizes) + ",\"pad_lower\":" + four(n->out.padding.lower_size.sizes) + ",\"pad_upper\":"
          + four(n->out.padding.upper_size.sizes);
     if (p.type == prim_type::convolution || p.type == prim_type::fused_conv_eltwise) {
+        if (p.fully_connected) s += ",\"fully_connected\":true";
         s += ",\"stride\":" + four(p.stride.sizes) + ",\"fused_activation\":" + std::to_string(n->fused_act);
         s += ",\"fused_activation_params\":[" + std::to_string(n->fused_a) + "," + std::to_string(n->fused_b) + "]";
     }

@@ -57,6 +57,21 @@ cldnn_tensor output_size;
 CLDNN_END_PRIMITIVE_DESC(pooling)
 CLDNN_DECLARE_PRIMITIVE_TYPE_ID(pooling);
 
+/* fully_connected (reference api/C/fully_connected.h:33-59): the convolution whose filter covers the whole input
+ * plane; weights [ofm][ifm][y][x] in bfyx.  Quantized (weights_quantization_factors given) it has the epilogue of the
+ * reference's int8 fully_connected kernels, not the convolution's. */
+CLDNN_BEGIN_PRIMITIVE_DESC(fully_connected)
+uint32_t with_activation;
+float activation_negative_slope;
+cldnn_primitive_id weights;
+cldnn_primitive_id bias;
+cldnn_primitive_id weights_quantization_factors;
+cldnn_primitive_id output_calibration_factors;
+float input_quantization_factor;
+float output_quantization_factor;
+CLDNN_END_PRIMITIVE_DESC(fully_connected)
+CLDNN_DECLARE_PRIMITIVE_TYPE_ID(fully_connected);
+
 typedef enum {
     cldnn_eltwise_sum,
     cldnn_eltwise_sub,

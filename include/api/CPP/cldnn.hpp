@@ -586,6 +586,48 @@ private:
     mutable id_list _in;
 };
 
+// fully_connected(id, input, weights, bias, with_activation, slope) and the quantized forms with
+// w_quantization_factor [, output_calibration_factors], i_quantization_factor [, o_quantization_factor]
+// (reference api/CPP/fully_connected.hpp:60-150)
+struct fully_connected : primitive {
+    primitive_id weights, bias, weights_quantization_factors, output_calibration_factors;
+    float input_quantization_factor = 1.0f, output_quantization_factor = 1.0f;
+    bool with_activation;
+    float activation_negative_slope;
+    fully_connected(const primitive_id& id, const primitive_id& input, const primitive_id& weights, const primitive_id& bias = "",
+                    bool with_activation = false, float activation_slp = 0.0f, const padding& output_padding = padding())
+        : primitive(id, {input}, output_padding), weights(weights), bias(bias), with_activation(with_activation),
+          activation_negative_slope(activation_slp) {}
+    fully_connected(const primitive_id& id, const primitive_id& input, const primitive_id& weights, const primitive_id& bias,
+                    const primitive_id& w_quantization_factor, const float i_quantization_factor, const float o_quantization_factor,
+                    bool with_activation = false, float activation_slp = 0.0f, const padding& output_padding = padding())
+        : primitive(id, {input}, output_padding), weights(weights), bias(bias), weights_quantization_factors(w_quantization_factor),
+          input_quantization_factor(i_quantization_factor), output_quantization_factor(o_quantization_factor),
+          with_activation(with_activation), activation_negative_slope(activation_slp) {}
+    fully_connected(const primitive_id& id, const primitive_id& input, const primitive_id& weights, const primitive_id& bias,
+                    const primitive_id& w_quantization_factor, const primitive_id& output_calibration_factors,
+                    const float i_quantization_factor, bool with_activation = false, float activation_slp = 0.0f,
+                    const padding& output_padding = padding())
+        : primitive(id, {input}, output_padding), weights(weights), bias(bias), weights_quantization_factors(w_quantization_factor),
+          output_calibration_factors(output_calibration_factors), input_quantization_factor(i_quantization_factor),
+          with_activation(with_activation), activation_negative_slope(activation_slp) {}
+    CLDNN_CPP_TYPE_ID(fully_connected)
+    const ::cldnn_primitive_desc* get_dto() const override
+    {
+        fill_base(_d, type_id(), _in);
+        _d.with_activation = with_activation, _d.activation_negative_slope = activation_negative_slope;
+        _d.weights = weights.c_str(), _d.bias = bias.c_str();
+        _d.weights_quantization_factors = weights_quantization_factors.c_str();
+        _d.output_calibration_factors = output_calibration_factors.c_str();
+        _d.input_quantization_factor = input_quantization_factor, _d.output_quantization_factor = output_quantization_factor;
+        return reinterpret_cast<const ::cldnn_primitive_desc*>(&_d);
+    }
+
+private:
+    mutable cldnn_fully_connected_desc _d{};
+    mutable id_list _in;
+};
+
 enum class eltwise_mode : int32_t { sum = cldnn_eltwise_sum, sub = cldnn_eltwise_sub, max = cldnn_eltwise_max, prod = cldnn_eltwise_prod };
 
 struct eltwise : primitive {

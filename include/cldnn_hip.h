@@ -240,6 +240,12 @@ typedef struct {
      * padding_above / padding_below of the primitive, which the reference realises with a border primitive
      * (src/graph_optimizer/handle_input_padding.cpp:43-77). */
     int32_t pad_end_delta_y, pad_end_delta_x;
+    /* 1: the epilogue of the reference's quantized fully_connected kernels instead of the convolution's
+     * (kernel_selector/core/cl_kernels/fully_connected_gpu_bfyx_ref.cl:63-84, fully_connected_gpu_MMAD.cl:103-118):
+     * with a bias (char)round(((float)acc * wqf * iqf + bias) * (calib or output factor)), without one the raw
+     * accumulator; conversion to char keeps the low byte; the activation acts on that char.  A fully_connected layer
+     * is the convolution whose filter covers the whole input plane; this flag only matters when has_wqf is set. */
+    int32_t fully_connected;
 } cldnn_hip_conv_desc;
 
 /* Host pointers: weights [ofm][ifm/groups][fy][fx] dense, bias/wqf/calib/eltw_calib [ofm] or NULL.

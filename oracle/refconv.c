@@ -233,6 +233,24 @@ static double epilogue_q(const rc_desc* d, int32_t acc, int f, const void* bias,
     return store_sat(out, d->out_dt, oi, o, 1);
 }
 
+/* quantized fully_connected (see rc_desc.fc) */
+static double epilogue_fc_q(const rc_desc* d, int32_t acc, int f, const void* bias, const float* wqf, const float* calib,
+                            void* out, int64_t oi)
+{
+    int32_t v = acc;
+    if (bias) {
+        float bv = d->bias_dt == RC_F32 ? ((const float*)bias)[f] : (float)((const int32_t*)bias)[f];
+        float x = (float)acc * wqf[f];
+        x = x * d->iqf;
+        x = x + bv;
+        x = x * (d->has_calib ? calib[f] : d->oqf);
+        v = (int32_t)(signed char)(int32_t)rnd(d, x); /* (UNIT_TYPE)round(...) */
+    }
+    signed char c = (signed char)v; /* convert_char: the low byte */
+    c = act_c(d->act, d->act_m, d->act_n, c);
+    return store_sat(out, d->out_dt, oi, c, 0);
+}
+
 /* MODE_FINT: int activation, float only in the last calibration (.cl:35-42, 199-232) */
 static double epilogue_fint(const rc_desc* d, int32_t acc, int f, const void* bias, double eltw_val,
                             const float* eltw_calib, void* out, int64_t oi)
@@ -446,7 +464,9 @@ int rc_conv(const rc_desc* d, const void* in, const void* weights, const void* b
                     if (d->fused)
                         ev = load_val(eltw, d->eltw_dt,
                                       ebase + (int64_t)y * d->esy * d->eltw_p.py + (int64_t)x * d->esx * d->eltw_p.px);
-                    if (mode == MODE_Q) {
+                    if (mode == MODE_Q && d->fc) {
+                        epilogue_fc_q(d, a, f, bias, wqf, calib, out, oi);
+                    } else if (mode == MODE_Q) {
                         epilogue_q(d, a, f, bias, wqf, calib, ev, eltw_calib, out, oi);
                     } else if (mode == MODE_FINT) {
                         epilogue_fint(d, a, f, bias, ev, eltw_calib, out, oi);

@@ -71,6 +71,11 @@ typedef struct {
     rc_pitch in_p, out_p, eltw_p;
     /* 1 = round half to even instead of half away from zero (documented variant, not the reference) */
     int round_even;
+    /* 1 = the epilogue of the reference's quantized fully_connected kernels
+       (fully_connected_gpu_bfyx_ref.cl:63-84, fully_connected_gpu_MMAD.cl:103-118): with a bias
+       (char)round(((float)acc * wqf * iqf + bias) * (calib or oqf)), without one the raw accumulator; converted to
+       char by dropping the upper bits; the activation acts on that char */
+    int fc;
 } rc_desc;
 
 /* Output extent along one axis (sliding_window_utils.h:113-126; degenerate value 1). */

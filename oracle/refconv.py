@@ -36,7 +36,7 @@ class Desc(C.Structure):
         + [("eltw_act", C.c_int), ("eltw_m", C.c_float), ("eltw_n", C.c_float)]
         + [("has_eltw_calib", C.c_int), ("esy", C.c_int), ("esx", C.c_int)]
         + [("in_p", Pitch), ("out_p", Pitch), ("eltw_p", Pitch)]
-        + [("round_even", C.c_int)]
+        + [("round_even", C.c_int), ("fc", C.c_int)]
     )
 
 
@@ -94,7 +94,7 @@ def _dense(F, H, W):
 def conv(x, w, bias=None, wqf=None, calib=None, *, stride=(1, 1), pad=(0, 0), dilation=(1, 1), groups=1,
          out_dt=None, iqf=1.0, oqf=1.0, act="none", act_m=0.0, act_n=0.0,
          eltw=None, non_conv_scale=1.0, eltw_act="none", eltw_m=0.0, eltw_n=0.0, eltw_calib=None,
-         eltw_stride=(1, 1), round_even=False, want_acc=False, nthreads=0, pad_end=None):
+         eltw_stride=(1, 1), round_even=False, want_acc=False, nthreads=0, pad_end=None, fc=False):
     """Reference convolution on dense bfyx numpy arrays.
 
     x [B,IFM,IH,IW]; w [OFM,IFM/groups,FY,FX]; bias/wqf/calib/eltw_calib [OFM];
@@ -140,6 +140,7 @@ def conv(x, w, bias=None, wqf=None, calib=None, *, stride=(1, 1), pad=(0, 0), di
     d.in_p = _dense(IFM, IH, IW)
     d.out_p = _dense(OFM, OH, OW)
     d.round_even = int(round_even)
+    d.fc = int(fc)
     if eltw is not None:
         eltw = np.ascontiguousarray(eltw)
         d.eltw_dt = DT_OF[eltw.dtype]
@@ -200,3 +201,21 @@ def pool(x, mode, size, stride=(1, 1), pad=(0, 0), out_size=None, global_pooling
     if lib().rc_pool(C.byref(d), _ptr(x), _ptr(out)) != 0:
         raise ValueError("unsupported pooling")
     return out
+
+
+def fully_connected(x, w, bias=None, wqf=None, calib=None, *, iqf=1.0, oqf=1.0, act="none", act_m=0.0):
+    """Reference fully_connected: x [B, F, Y, X], w [OFM, F, Y, X] -> [B, OFM, 1, 1] in the input's data type.  Quantized
+    (wqf given) it has its own epilogue, see rc_desc.fc; otherwise it is the convolution whose filter covers the input."""
+    return conv(x, w, bias, wqf=wqf, calib=calib, iqf=iqf, oqf=oqf, act=act, act_m=act_m, fc=wqf is not None)
+
+
+def eltwise_sum(a, b, calib=None, oqf=1.0, relu=False):
+    """Stand-alone element-wise sum of two int8 tensors in its quantized form (reference
+    kernel_selector/core/cl_kernels/generic_eltwise_ref.cl:311-330): int sum, round((float)sum * factor) half away from
+    zero with the factor per feature (calib) or per tensor (oqf), saturation to char, then the activation on the char."""
+    s = a.astype(np.int32) + b.astype(np.int32)
+    f = np.float32(oqf) if calib is None else np.asarray(calib, np.float32).reshape(1, -1, 1, 1)
+    v = s.astype(np.float32) * f
+    r = np.sign(v) * np.floor(np.abs(v) + np.float32(0.5))
+    c = np.clip(r, -128, 127).astype(np.int8)
+    return np.maximum(c, 0) if relu else c

@@ -332,6 +332,24 @@ def test_conv_eltwise_not_fused(kw):
     assert "conv2" in ids and "sum" in ids
 
 
+def test_conv_eltwise_fusing_reaches_every_block_of_a_chain():
+    """three residual blocks in a row: each sum reads the previous (fused) block's output and its own closing 1x1
+    convolution; every one of them fuses (the fused node keeps the sum's place in the execution order)"""
+    w = np.ones((16, 16, 1, 1), np.int8)
+    t = cl.topology(cl.input_layout("in", cl.layout(DT.i8, F.bfyx, cl.tensor(1, 16, 4, 4))), cl.data("w", attach(w)), cl.data("q", vec(16)),
+                    cl.data("c", vec(16)))
+    cur = "in"
+    for i in range(3):
+        t.add(cl.convolution(f"mid{i}", cur, ["w"], None, ["q"], ["c"], with_activation=True),
+              cl.convolution(f"close{i}", f"mid{i}", ["w"], None, ["q"], ["c"]),
+              cl.eltwise(f"sum{i}", cur, f"close{i}", cl.eltwise_mode.sum, with_activation=True))
+        cur = f"sum{i}"
+    t.add(cl.reorder("out", cur, F.bfyx, DT.i8))
+    ids = [n["id"] for n in cl.plan(t, cl.build_options(optimize_data=True))]
+    assert [i for i in ids if "_fused_" in i] == ["close0_fused_sum0", "close1_fused_sum1", "close2_fused_sum2"]
+    assert not any(i.startswith("sum") for i in ids)
+
+
 def test_conv_eltwise_fusing_moves_eltwise_stride_into_the_conv():
     """A strided eltwise after a 1x1 convolution: the convolution takes the stride, the shortcut keeps its own
     (reference src/graph_optimizer/prepare_primitive_fusing.cpp:300-318)."""

@@ -1,0 +1,105 @@
+"""A whole quantized ResNet-50 (53 convolutions, 2 poolings, 16 residual sums, 1 fully_connected) through the clDNN
+API against the CPU oracle run layer by layer, bit for bit, as written and with optimize_data."""
+import numpy as np
+import pytest
+
+from cldnn_amd import resnet50_net as rn
+from oracle import refconv as rc
+
+
+def run_oracle(x, params, fused=(), calibrate=False):
+    """Oracle forward pass, layer by layer.  `fused` names the blocks whose residual sum runs inside the closing
+    convolution (fused_conv_eltwise: the convolution's result is not saturated before the sum); the others use the
+    stand-alone eltwise on the saturated int8 tensor.  With calibrate=True the pass also chooses every layer's factors:
+    the root mean square of its outputs lands at about a quarter of the int8 range (what a calibration tool does), so
+    that few values saturate and no layer dies.  Returns the tensors by primitive id."""
+    t = {"input": x}
+    for step in rn.layer_plan():
+        if step[0] == "conv":
+            _, l, src, relu = step
+            q = params[l["name"]]
+            kw = dict(stride=(l["stride"],) * 2, pad=(l["pad"],) * 2)
+            if calibrate:
+                _, acc = rc.conv(t[src], q["w"], q["bias"], wqf=q["wqf"], calib=np.ones(l["ofm"], np.float32), out_dt="s8", want_acc=True, **kw)
+                full = acc.astype(np.float64) + q["bias"].reshape(1, -1, 1, 1)
+                q["calib"] = (32.0 / (np.sqrt((full * full).mean(axis=(0, 2, 3))) + 1.0)).astype(np.float32)
+            if l["closes_block"] and l["name"][:-9] in fused:
+                continue  # computed together with the residual sum
+            t[l["name"]] = rc.conv(t[src], q["w"], q["bias"], wqf=q["wqf"], calib=q["calib"], out_dt="s8", act="relu" if relu else "none", **kw)
+        elif step[0] == "pool1":
+            t["pool1"] = rc.pool(t["conv1"], "max", (3, 3), (2, 2))
+        elif step[0] == "sum":
+            _, n, shortcut, branch = step
+            if calibrate:
+                params[n] = dict(ecal=np.full(params[branch]["w"].shape[0], 0.6, np.float32))
+            if n in fused:
+                q = params[branch]
+                t[n] = rc.conv(t[n + "_branch2b"], q["w"], q["bias"], wqf=q["wqf"], calib=q["calib"], out_dt="s8", eltw=t[shortcut],
+                               eltw_act="relu", eltw_calib=params[n]["ecal"])
+            else:
+                t[n] = rc.eltwise_sum(t[shortcut], t[branch], calib=params[n]["ecal"], relu=True)
+        elif step[0] == "pool5":
+            t["pool5"] = rc.pool(t["res5c"], "average", None, global_pooling=True)
+        else:
+            q = params["fc1000"]
+            if calibrate:
+                acc = np.einsum("bfyx,ofyx->bo", t["pool5"].astype(np.int64), q["w"].astype(np.int64)).astype(np.float64)
+                q["calib"] = np.full(q["w"].shape[0], 40.0 / (np.sqrt((acc * acc).mean()) + 1.0), np.float32)
+            t["fc1000"] = rc.fully_connected(t["pool5"], q["w"], q["bias"], wqf=q["wqf"], calib=q["calib"])
+    return t
+
+
+BLOCKS = [s[1] for s in rn.layer_plan() if s[0] == "sum"]
+
+
+def test_layer_plan_shape():
+    steps = rn.layer_plan()
+    assert sum(s[0] == "conv" for s in steps) == 53 and sum(s[0] == "sum" for s in steps) == 16
+    assert steps[0][1]["name"] == "conv1" and steps[-1] == ("fc",)
+
+
+def test_fused_and_stand_alone_sum_differ_only_where_the_convolution_saturates():
+    """the property the two oracle forms rest on: (closing convolution, saturated to int8) + stand-alone sum equals the
+    fused primitive wherever the convolution's result fits into int8"""
+    r = np.random.default_rng(1)
+    x = r.integers(0, 128, (1, 64, 6, 6)).astype(np.int8)
+    w = r.integers(-127, 128, (256, 64, 1, 1)).astype(np.int8)
+    bias, one = r.integers(-1000, 1001, 256).astype(np.int32), np.ones(256, np.float32)
+    cal, ecal = np.full(256, 0.003, np.float32), r.uniform(0.4, 0.9, 256).astype(np.float32)
+    sc = r.integers(-128, 128, (1, 256, 6, 6)).astype(np.int8)
+    c = rc.conv(x, w, bias, wqf=one, calib=cal, out_dt="s8")
+    fused = rc.conv(x, w, bias, wqf=one, calib=cal, out_dt="s8", eltw=sc, eltw_act="relu", eltw_calib=ecal)
+    alone = rc.eltwise_sum(sc, c, calib=ecal, relu=True)
+    inside = (c > -128) & (c < 127)
+    assert 0.5 < inside.mean() < 0.999                      # both regions occur
+    np.testing.assert_array_equal(fused[inside], alone[inside])
+    assert (fused[~inside] != alone[~inside]).any()
+
+
+@pytest.mark.gpu
+def test_resnet50_int8_network_matches_the_oracle():
+    from cldnn_amd import api as cl
+    eng = cl.engine()
+    B = 2
+    x = np.random.default_rng(7).integers(0, 256, (B, 3, 224, 224)).astype(np.uint8)
+    params = rn.random_weights(seed=11)
+    run_oracle(x, params, fused=BLOCKS, calibrate=True)
+    topo = rn.topology(cl, eng, params, B)
+    watch = ["pool1", "res2a", "res3d", "res4f", "res5c", "pool5", "fc1000"]
+    for optimize in (True, False):
+        # optimize_data fuses a residual sum into its closing convolution unless the sum is itself an output; the plan says
+        # which ones (node ids <convolution>_fused_<sum>), and the oracle follows it: the two forms differ where the
+        # convolution's own result leaves the int8 range
+        opts = cl.build_options(optimize_data=optimize, outputs=watch)
+        fused = [n["id"].split("_fused_")[1] for n in cl.plan(topo, opts) if "_fused_" in n["id"]]
+        assert sorted(fused) == (sorted(b for b in BLOCKS if b not in watch) if optimize else [])
+        ref = run_oracle(x, params, fused=fused)
+        assert 5 < np.abs(ref["res5c"].astype(np.int32)).mean() < 100 and len(np.unique(ref["fc1000"])) > 50  # alive to the end
+        net = cl.network(eng, topo, opts)
+        net.set_input_data("input", cl.make_memory(eng, x))
+        outs = net.execute()
+        for name in watch:
+            got = outs[name].get_memory().read()
+            assert got.shape == ref[name].shape, name
+            bad = int((got != ref[name]).sum())
+            assert bad == 0, "%s (optimize_data=%s): %d of %d values differ" % (name, optimize, bad, got.size)
