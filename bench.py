@@ -170,6 +170,53 @@ def copy_calibration(args):
                                                            "written_bytes": src.nbytes}}), flush=True)
 
 
+def network_workload(args):
+    """The whole quantized ResNet-50 topology (53 convolutions, 2 poolings, 16 residual sums, fully_connected) built and run
+    through the clDNN API with optimize_data: what an application sees per network.execute(), input already on the device."""
+    from cldnn_amd import api as cl, resnet50_net as rn
+    batch = 32
+    eng = cl.engine()
+    r = np.random.default_rng(1337)
+    params = rn.random_weights()
+    IN_RMS, ECAL = 35.0, 1.0  # keep the signal alive through 16 blocks without a calibration pass
+    for l in workloads.resnet50():  # factors by rule (no calibration pass: timing does not depend on the values)
+        k = l["ifm"] * l["k"] ** 2
+        params[l["name"]]["calib"] = (32.0 / (np.sqrt(k) * IN_RMS * 73.3) * r.uniform(0.7, 1.4, l["ofm"])).astype(np.float32)
+    for step in rn.layer_plan():
+        if step[0] == "sum":
+            params[step[1]] = dict(ecal=np.full(params[step[3]]["w"].shape[0], ECAL, np.float32))
+    params["fc1000"]["calib"] = np.full(1000, 40.0 / (np.sqrt(2048) * 30.0 * 73.3), np.float32)
+    t0 = time.perf_counter()
+    net = cl.network(eng, rn.topology(cl, eng, params, batch), cl.build_options(optimize_data=True))
+    x = r.integers(0, 256, (batch, 3, 224, 224)).astype(np.uint8)
+    net.set_input_data("input", cl.make_memory(eng, x))
+    log("built the network in %.1f s (%d primitives executed per run)" % (time.perf_counter() - t0, len(net.get_executed_primitive_ids())
+                                                                        if hasattr(net, "get_executed_primitive_ids") else -1))
+
+    def run():
+        outs = net.execute()
+        outs["fc1000"].get_event().wait()
+        return outs
+
+    for _ in range(args.warmup):
+        run()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        outs = run()
+    dt = time.perf_counter() - t0
+    logits = outs["fc1000"].get_memory().read()
+    ops = 2.0 * batch * (workloads.macs(workloads.resnet50()) + 2048 * 1000)
+    print(json.dumps({
+        "metric": "ResNet-50 int8 network images/sec @b32 (whole topology through the clDNN API)", "value": batch * args.steps / dt,
+        "unit": "images/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": dt / args.steps * 1e3,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "i8xi8->i32 (f32 requantisation)", "data": "synthetic",
+        "config": {"workload": "resnet50_b32_network", "batch": batch, "primitives": "53 convolution, 2 pooling, 16 eltwise (fused), 1 fully_connected",
+                   "build": "optimize_data"},
+        "roofline": {"bound": "mfma", "achieved": ops * args.steps / dt / 1e12, "peak": PEAK_INT8_OPS / 1e12, "unit": "TOP/s",
+                     "frac": ops * args.steps / dt / PEAK_INT8_OPS, "traffic": None, "kernel": "all kernels of one network.execute()"},
+        "cpu_baseline": None, "distinct_logit_values": int(len(np.unique(logits)))}), flush=True)
+
+
 def measured_traffic(workload):
     """HBM bytes per launch from the committed counter summary of this workload (None when there is none)."""
     path = os.path.join(ROOT, "profiles", "conv_stack_%s_hbm_traffic.txt" % workload)
@@ -189,7 +236,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="resnet50_b32_fused",
                     choices=["resnet50_b32_fused", "resnet50_b32", "resnet50_b1", "vgg16_b16", "mobilenet_v2_b32", "c1",
-                             "copy_256m"])
+                             "copy_256m", "resnet50_b32_network"])
     ap.add_argument("--tile", type=int, default=0, help="force one row (index+1) of the tile table on every layer")
     ap.add_argument("--per-layer", action="store_true", help="time every layer on its own and print a table to stderr")
     ap.add_argument("--tune", action="store_true", help="try every row of the tile table on every layer, print the best")
@@ -209,6 +256,8 @@ def main():
     wl = args.workload
     if wl == "copy_256m":
         return copy_calibration(args)
+    if wl == "resnet50_b32_network":
+        return network_workload(args)
     if wl.startswith("resnet50"):
         layers, batch, fuse = workloads.resnet50(), (1 if wl.endswith("b1") else 32), wl.endswith("fused")
     elif wl == "vgg16_b16":
