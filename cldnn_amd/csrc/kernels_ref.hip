@@ -334,6 +334,34 @@ void launch_conv_ref(hipStream_t s, const ConvProblem& p, const Epilogue& epi, c
     CHIP_CHECK(hipGetLastError());
 }
 
+// 8-bit data from a plain layout into a blocked one (the step in front of the first convolution of a network): one
+// work-item gathers the FSV features of one pixel and writes them with one FSV-byte store; consecutive work-items
+// take consecutive pixels of a row, so the stores of a wavefront are contiguous and the loads run along the rows of
+// FSV feature planes.  Feature padding is written as zero, spatial padding is left untouched.
+template <int FSV>
+__global__ void __launch_bounds__(256) reorder_to_blocked_kernel(ReorderArgs a, const uint8_t* __restrict__ src, uint8_t* __restrict__ dst)
+{
+    const int slices = (a.F + FSV - 1) / FSV;
+    const int64_t total = (int64_t)slices * a.B * a.Y * a.X;
+    const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= total) return;
+    const int x = (int)(idx % a.X);
+    int64_t r = idx / a.X;
+    const int y = (int)(r % a.Y);
+    r /= a.Y;
+    const int fs = (int)(r % slices), b = (int)(r / slices);
+    unsigned w[FSV / 4];
+#pragma unroll
+    for (int i = 0; i < FSV / 4; ++i) w[i] = 0;
+    const int64_t s0 = a.src.at(b, fs * FSV, y, x);
+#pragma unroll
+    for (int c = 0; c < FSV; ++c)
+        if (fs * FSV + c < a.F) w[c >> 2] |= (unsigned)src[s0 + (int64_t)c * a.src.pf] << (8 * (c & 3));
+    uint8_t* o = dst + a.dst.at(b, fs * FSV, y, x);
+    if constexpr (FSV == 4) *reinterpret_cast<unsigned*>(o) = w[0];
+    else *reinterpret_cast<uint4*>(o) = make_uint4(w[0], w[1], w[2], w[3]);
+}
+
 void launch_reorder(hipStream_t s, const cldnn_hip_tensor& st, const void* src, const cldnn_hip_tensor& dt, void* dst)
 {
     CHIP_REQUIRE(st.b == dt.b && st.f == dt.f && st.y == dt.y && st.x == dt.x, CLDNN_HIP_DIMENSION_MISMATCH,
@@ -342,6 +370,19 @@ void launch_reorder(hipStream_t s, const cldnn_hip_tensor& st, const void* src, 
     a.src = make_pitch(st), a.dst = make_pitch(dt);
     a.B = st.b, a.F = st.f, a.Y = st.y, a.X = st.x;
     a.src_dt = st.dtype, a.dst_dt = dt.dtype;
+    const bool bytes = (st.dtype == CLDNN_HIP_S8 || st.dtype == CLDNN_HIP_U8) && st.dtype == dt.dtype;
+    if (bytes && a.src.fsv == 1 && (a.dst.fsv == 4 || a.dst.fsv == 16)) {
+        const int64_t work = (int64_t)((a.F + a.dst.fsv - 1) / a.dst.fsv) * a.B * a.Y * a.X;
+        const int64_t nb = (work + 255) / 256;
+        CHIP_REQUIRE(nb < (1ll << 31), CLDNN_HIP_UNSUPPORTED_SIZE, "tensor too large for the reorder grid");
+        if (a.dst.fsv == 4)
+            hipLaunchKernelGGL(reorder_to_blocked_kernel<4>, dim3((unsigned)nb), dim3(256), 0, s, a, (const uint8_t*)src, (uint8_t*)dst);
+        else
+            hipLaunchKernelGGL(reorder_to_blocked_kernel<16>, dim3((unsigned)nb), dim3(256), 0, s, a, (const uint8_t*)src, (uint8_t*)dst);
+        CHIP_CHECK(hipGetLastError());
+        // feature slices the destination holds beyond ceil(F / fsv) do not exist in these formats
+        return;
+    }
     a.dst_fs_fill = a.dst.fsv > 1 ? a.dst.fs_count * a.dst.fsv - dt.f : 0;
     const int64_t total = (int64_t)a.B * (a.F + a.dst_fs_fill) * a.Y * a.X;
     const int64_t blocks = (total + 255) / 256;
