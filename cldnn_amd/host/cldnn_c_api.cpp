@@ -462,6 +462,7 @@ cldnn_engine cldnn_create_engine(int32_t type, uint32_t engine_num, const cldnn_
         }
         ref<cldnn_engine_impl> e(new cldnn_engine_impl(), false);
         e->profiling = cfg && cfg->enable_profiling;
+        e->memory_pool = !cfg || cfg->enable_memory_pool;
         hip_check(cldnn_hip_engine_create(engine_num, e->profiling ? 1 : 0, &e->h));
         e->retain();
         return e.get();
@@ -617,12 +618,62 @@ cldnn_network cldnn_allocate_network(cldnn_program program, cldnn_status* status
         ref<cldnn_network_impl> net(new cldnn_network_impl(), false);
         net->program = ref<cldnn_program_impl>(program, true);
         cldnn_engine_impl* e = program->engine.get();
-        for (auto& u : program->nodes) {
-            node* n = u.get();
-            if (n->constant) net->mem[n] = on_engine(e, n->p->mem.get());
-            else if (n->p->type == prim_type::input_layout) net->input_set[n->p->id] = false;
-            else if (n->p->type == prim_type::fused_conv_eltwise && n->p->second_input_in_output) net->mem[n] = net->mem[n->deps[1]];
-            else net->mem[n] = allocate(e, n->out);
+        // Memory pool (reference src/memory_pool.cpp, engine option enable_memory_pool): an intermediate tensor takes
+        // over the buffer of an earlier one of exactly the same layout once that one's last consumer has been passed in
+        // execution order -- everything runs in order on one stream.  Same layout only: producers write the logical
+        // elements and never the zero border or the feature padding, so those stay as the allocation left them.
+        // Outputs, inputs and constants keep buffers of their own.
+        std::map<node*, size_t> index, last_use;
+        bool aliasing = false;
+        for (size_t i = 0; i < program->nodes.size(); ++i) {
+            node* n = program->nodes[i].get();
+            index[n] = i;
+            if (n->p->type == prim_type::fused_conv_eltwise && n->p->second_input_in_output) aliasing = true;
+        }
+        for (auto& u : program->nodes)
+            for (node* d : u->deps) last_use[d] = std::max(last_use[d], index[u.get()]);
+        const bool pool = e->memory_pool && !aliasing;
+        std::vector<std::pair<size_t, ref<cldnn_memory_impl>>> in_flight;  // (index of the last consumer, buffer)
+        std::vector<ref<cldnn_memory_impl>> idle;
+        for (size_t i = 0; i < program->nodes.size(); ++i) {
+            node* n = program->nodes[i].get();
+            if (n->constant) {
+                net->mem[n] = on_engine(e, n->p->mem.get());
+                continue;
+            }
+            if (n->p->type == prim_type::input_layout) {
+                net->input_set[n->p->id] = false;
+                continue;
+            }
+            if (n->p->type == prim_type::fused_conv_eltwise && n->p->second_input_in_output) {
+                net->mem[n] = net->mem[n->deps[1]];
+                continue;
+            }
+            // buffers whose tensors nobody reads at or after this primitive become idle
+            for (auto it = in_flight.begin(); it != in_flight.end();) {
+                if (it->first < i) {
+                    idle.push_back(it->second);
+                    it = in_flight.erase(it);
+                } else {
+                    ++it;
+                }
+            }
+            ref<cldnn_memory_impl> m;
+            if (pool && !n->is_output) {
+                for (auto it = idle.begin(); it != idle.end(); ++it)
+                    if (same_layout((*it)->layout, n->out)) {
+                        m = *it;
+                        idle.erase(it);
+                        net->pooled_tensors++;
+                        break;
+                    }
+            }
+            if (!m) {
+                m = allocate(e, n->out);
+                net->allocated_bytes += layout_bytes(n->out);
+            }
+            net->mem[n] = m;
+            if (pool && !n->is_output && last_use.count(n)) in_flight.emplace_back(last_use[n], m);
         }
         net->retain();
         return net.get();

@@ -69,6 +69,7 @@ enum class prim_type { input_layout, data, reorder, activation, eltwise, convolu
 struct cldnn_engine_impl : host::refcounted {
     cldnn_hip_engine h = nullptr;
     bool profiling = false;
+    bool memory_pool = true;  // networks share buffers between intermediate tensors whose lifetimes do not overlap
     ~cldnn_engine_impl() override;
 };
 
@@ -176,4 +177,6 @@ struct cldnn_network_impl : host::refcounted {
     std::map<std::string, bool> input_set;
     std::vector<std::string> executed;
     bool has_run = false;
+    size_t allocated_bytes = 0;  // device bytes of the buffers the network allocated for its primitives' outputs
+    size_t pooled_tensors = 0;   // outputs that reuse the buffer of an earlier, finished tensor
 };

@@ -68,7 +68,7 @@ typedef struct {
     const char* sources_dumps_dir;     /* accepted, no effect */
     int16_t priority_mode;             /* must stay disabled: one stream at default priority */
     int16_t throttle_mode;
-    uint32_t enable_memory_pool;       /* accepted, no effect */
+    uint32_t enable_memory_pool;       /* networks reuse buffers between intermediate tensors of identical layout */
     void* context;                     /* must be NULL */
     const char* tuning_cache_path;     /* accepted, no effect: the tile table is built in */
 } cldnn_engine_configuration;

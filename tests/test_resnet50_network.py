@@ -103,3 +103,27 @@ def test_resnet50_int8_network_matches_the_oracle():
             assert got.shape == ref[name].shape, name
             bad = int((got != ref[name]).sum())
             assert bad == 0, "%s (optimize_data=%s): %d of %d values differ" % (name, optimize, bad, got.size)
+
+
+@pytest.mark.gpu
+def test_memory_pool_shares_buffers_without_changing_results():
+    """engine option enable_memory_pool (reference src/memory_pool.cpp): intermediate tensors of identical layout share
+    buffers once their consumers are done; same results, less device memory"""
+    from cldnn_amd import api as cl
+    B = 2
+    x = np.random.default_rng(3).integers(0, 256, (B, 3, 224, 224)).astype(np.uint8)
+    params = rn.random_weights(seed=5)
+    run_oracle(x, params, fused=BLOCKS, calibrate=True)
+    used, logits = {}, {}
+    for pool in (True, False):
+        eng = cl.engine(enable_memory_pool=pool)
+        base = eng.get_temp_used_device_memory_size()
+        net = cl.network(eng, rn.topology(cl, eng, params, B), cl.build_options(optimize_data=True))
+        net.set_input_data("input", cl.make_memory(eng, x))
+        for _ in range(2):  # a second run reuses the same buffers
+            logits[pool] = net.execute()["fc1000"].get_memory().read()
+        used[pool] = eng.get_temp_used_device_memory_size() - base
+        del net
+    np.testing.assert_array_equal(logits[True], logits[False])
+    np.testing.assert_array_equal(logits[True], run_oracle(x, params, fused=BLOCKS)["fc1000"])
+    assert used[True] < 0.8 * used[False], used
