@@ -42,7 +42,7 @@ class pooling_mode:  # noqa: N801
 
 
 class eltwise_mode:  # noqa: N801
-    sum, sub, max, prod = 0, 1, 2, 3
+    sum, sub, max, prod, div, min, pow, mod = range(8)
 
 
 class build_option_type:  # noqa: N801
@@ -591,11 +591,28 @@ class eltwise(_primitive):  # noqa: N801
     output_calibration_factors / output_quantization_factor (reference api/CPP/eltwise.hpp:78-260)."""
     type_fn = "cldnn_eltwise_type_id"
 
-    def __init__(self, prim_id, inp, inp2, mode=eltwise_mode.sum, with_activation=False, activation_slp=0.0,
+    def __init__(self, prim_id, inp, inp2=None, mode=eltwise_mode.sum, with_activation=False, activation_slp=0.0,
                  output_calibration_factors="", output_quantization_factor=1.0, stride=None, output_padding=None,
-                 output_data_type=None):
+                 output_data_type=None, coefficients=None):
+        """inp may be the list of all inputs (then inp2, if given, is the mode, as in eltwise(id, {inputs}, mode))."""
+        if isinstance(inp, (list, tuple)):
+            inputs = list(inp)
+            if inp2 is not None:
+                mode = inp2
+        else:
+            inputs = [inp, inp2]
+        if coefficients:
+            # reference api/CPP/eltwise.hpp:303-310
+            if mode == eltwise_mode.sum and len(coefficients) != len(inputs):
+                raise ValueError("Invalid eltwise sum coefficients count (should be equal to 0 or input.size)")
+            if mode != eltwise_mode.sum:
+                raise ValueError("Only eltwise sum operation supports blob-wise coefficients")
         d = c_eltwise_desc()
-        self._base(d, prim_id, [inp, inp2], output_padding, output_data_type)
+        self._base(d, prim_id, inputs, output_padding, output_data_type)
+        if coefficients:
+            arr = (C.c_float * len(coefficients))(*coefficients)
+            self._keep.append(arr)
+            d.coefficients = c_float_arr(C.cast(arr, C.POINTER(C.c_float)), len(coefficients))
         _eltw_fields(d, self._keep, output_calibration_factors, output_quantization_factor, mode, with_activation,
                      activation_slp, stride)
 

@@ -400,6 +400,16 @@ cldnn_hip_status cldnn_hip_eltwise_sum(cldnn_hip_engine e, const void* a_dev, co
     });
 }
 
+cldnn_hip_status cldnn_hip_eltwise(cldnn_hip_engine e, const cldnn_hip_eltwise_desc* desc, const void* const* inputs_dev,
+                                   const float* calib_dev, void* output_dev)
+{
+    return guarded([&] {
+        CHIP_REQUIRE(e && desc && inputs_dev && output_dev, CLDNN_HIP_INVALID_ARG, "null argument");
+        e->make_current();
+        launch_eltwise(e->stream, *desc, inputs_dev, calib_dev, output_dev);
+    });
+}
+
 cldnn_hip_status cldnn_hip_pooling(cldnn_hip_engine e, const cldnn_hip_pooling_desc* desc, const void* input_dev, void* output_dev)
 {
     return guarded([&] {

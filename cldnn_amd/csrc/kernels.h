@@ -16,6 +16,7 @@ struct ConvProblem {
 // ---- layout-agnostic kernels (kernels_ref.hip)
 void launch_conv_ref(hipStream_t s, const ConvProblem& p, const Epilogue& epi, const void* in, const void* w,
                      const void* eltw, void* out, int* acc_out);
+void launch_eltwise(hipStream_t s, const cldnn_hip_eltwise_desc& d, const void* const* inputs, const float* calib, void* dst);
 void launch_pooling(hipStream_t s, const cldnn_hip_pooling_desc& d, const void* in, void* out);
 void launch_reorder(hipStream_t s, const cldnn_hip_tensor& st, const void* src, const cldnn_hip_tensor& dt, void* dst);
 // dst = act(a [+ b]); quantized: round((a + b) * (calib[f] or oqf)) saturated to char before the activation

@@ -75,6 +75,18 @@ class PoolingDesc(C.Structure):
         "mode", "divider", "size_y", "size_x", "stride_y", "stride_x", "pad_y", "pad_x")]
 
 
+ELTWISE_MAX_INPUTS = 4
+ELTWISE_MODE = {"sum": 0, "sub": 1, "max": 2, "prod": 3, "div": 4, "min": 5, "pow": 6, "mod": 7}
+
+
+class EltwiseDesc(C.Structure):
+    _fields_ = [("mode", C.c_int32), ("n_inputs", C.c_int32), ("inputs", Tensor * ELTWISE_MAX_INPUTS),
+                ("stride_y", C.c_int32 * ELTWISE_MAX_INPUTS), ("stride_x", C.c_int32 * ELTWISE_MAX_INPUTS),
+                ("has_coefficients", C.c_int32), ("coefficients", C.c_float * ELTWISE_MAX_INPUTS), ("output", Tensor),
+                ("quantized", C.c_int32), ("output_quantization_factor", C.c_float), ("activation", C.c_int32),
+                ("m", C.c_float), ("n", C.c_float)]
+
+
 class ConvInfo(C.Structure):
     _fields_ = [
         ("impl", C.c_int32), ("tile_index", C.c_int32), ("tile_pixels", C.c_int32), ("tile_ofm", C.c_int32),
@@ -139,6 +151,7 @@ SIGNATURES = {
     "cldnn_hip_eltwise_sum": (C.c_int32, [C.c_void_p, C.c_void_p, C.POINTER(Tensor), C.c_void_p, C.POINTER(Tensor),
                                           C.c_void_p, C.POINTER(Tensor), C.c_int32, C.c_void_p, C.c_float, C.c_int32,
                                           C.c_float, C.c_float]),
+    "cldnn_hip_eltwise": (C.c_int32, [C.c_void_p, C.POINTER(EltwiseDesc), C.POINTER(C.c_void_p), C.c_void_p, C.c_void_p]),
     "cldnn_hip_conv_create": (C.c_int32, [C.c_void_p, C.POINTER(ConvDesc), C.c_void_p, C.c_void_p, C.c_void_p,
                                           C.c_void_p, C.c_void_p, C.POINTER(C.c_void_p)]),
     "cldnn_hip_conv_release": (C.c_int32, [C.c_void_p]),
@@ -276,6 +289,45 @@ def pool_forward(engine, x, mode, size, stride=(1, 1), pad=(0, 0), *, fmt="bfyx"
     out.close()
     xin.close()
     return res
+
+
+def eltwise_forward(engine, inputs, mode="sum", strides=None, calib=None, oqf=1.0, relu=False, slope=0.0, coefficients=None, *,
+                    fmt="bfyx", in_pad=(0, 0), out_pad=(0, 0)):
+    """numpy in, numpy out through cldnn_hip_eltwise; arguments as oracle.refconv.eltwise."""
+    L = lib()
+    ins = [np.ascontiguousarray(a) for a in inputs]
+    n = len(ins)
+    strides = [(1, 1)] * n if strides is None else [tuple(s) for s in strides]
+    if any(s != (1, 1) for s in strides):
+        shape = (ins[0].shape[0], ins[0].shape[1], ins[0].shape[2] // strides[0][0], ins[0].shape[3] // strides[0][1])
+    else:
+        shape = tuple(max(a.shape[d] for a in ins) for d in range(4))
+    bufs = [upload(engine, a, fmt, in_pad) for a in ins]
+    d = EltwiseDesc()
+    d.mode, d.n_inputs = ELTWISE_MODE[mode], n
+    for i in range(min(n, ELTWISE_MAX_INPUTS)):
+        d.inputs[i] = bufs[i].tensor
+        d.stride_y[i], d.stride_x[i] = strides[i]
+        d.coefficients[i] = 1.0 if coefficients is None else coefficients[i]
+    d.has_coefficients = coefficients is not None
+    t = bufs[0].tensor
+    d.output = Tensor.make(t.dtype, t.format, shape[0], shape[1], shape[2], shape[3], out_pad[0], out_pad[1])
+    d.quantized = ins[0].dtype != np.float32 and (calib is not None or oqf != 1.0)
+    d.output_quantization_factor = oqf
+    d.activation = ACT_NONE if not relu else (ACT_RELU if slope == 0.0 else ACT_RELU_SLOPE)
+    d.m = slope
+    cal = None
+    if calib is not None:
+        cal = Buffer(engine, Tensor.make(F32, BFYX, 1, 1, 1, len(calib)))
+        cal.write_raw(np.asarray(calib, np.float32))
+    out = Buffer(engine, d.output)
+    ptrs = (C.c_void_p * ELTWISE_MAX_INPUTS)(*[b.ptr for b in bufs[:ELTWISE_MAX_INPUTS]])
+    try:
+        check(L.cldnn_hip_eltwise(engine.h, C.byref(d), ptrs, cal.ptr if cal else None, out.ptr))
+        return download(engine, out)
+    finally:
+        for b in bufs + [out] + ([cal] if cal else []):
+            b.close()
 
 
 def upload(engine, arr, fmt="bfyx", pad=(0, 0)):

@@ -162,18 +162,29 @@ static void execute(cldnn_network_impl* net, cldnn_event* deps, size_t ndeps)
             break;
         }
         case prim_type::eltwise: {
-            HOST_REQUIRE(p.eltw_mode == cldnn_eltwise_sum, CLDNN_INVALID_ARG, "eltwise: only the sum mode is implemented");
-            cldnn_memory_impl* a = mem_of(n->deps[0]);
-            cldnn_memory_impl* b = mem_of(n->deps[1]);
-            const cldnn_hip_tensor at = to_hip(n->deps[0]->out), bt = to_hip(n->deps[1]->out);
+            // reference src/gpu/eltwise_gpu.cpp:58-145: inputs, then the calibration factors
+            const size_t count = p.inputs.size();
+            cldnn_hip_eltwise_desc d{};
+            const void* src[CLDNN_HIP_ELTWISE_MAX_INPUTS] = {};
+            d.mode = p.eltw_mode, d.n_inputs = (int32_t)count;
+            for (size_t i = 0; i < count; ++i) {
+                d.inputs[i] = to_hip(n->deps[i]->out);
+                src[i] = mem_of(n->deps[i])->device_ptr();
+                d.stride_x[i] = p.eltw_stride.empty() ? 1 : p.eltw_stride[i].sizes[2];
+                d.stride_y[i] = p.eltw_stride.empty() ? 1 : p.eltw_stride[i].sizes[3];
+                d.coefficients[i] = p.eltw_coefficients.empty() ? 1.0f : p.eltw_coefficients[i];
+            }
+            d.has_coefficients = !p.eltw_coefficients.empty();
+            d.output = ot;
             const float* calib = nullptr;
-            if (!p.eltw_calib.empty()) calib = (const float*)mem_of(n->deps[2])->device_ptr();
+            if (!p.eltw_calib.empty()) calib = (const float*)mem_of(n->deps[count])->device_ptr();
             const bool int_data = n->deps[0]->out.data_type == cldnn_i8 || n->deps[0]->out.data_type == cldnn_u8;
-            const int quantized = int_data && (calib || p.eltw_oqf != 1.0f);
-            int act = CLDNN_HIP_ACT_NONE;
-            if (p.eltw_with_act) act = p.eltw_slope == 0.0f ? CLDNN_HIP_ACT_RELU : CLDNN_HIP_ACT_RELU_SLOPE;
-            hip_check(cldnn_hip_eltwise_sum(eng->h, a->device_ptr(), &at, b->device_ptr(), &bt, out->device_ptr(), &ot, quantized,
-                                            calib, p.eltw_oqf, act, p.eltw_slope, 0.0f));
+            d.quantized = int_data && (calib || p.eltw_oqf != 1.0f);
+            d.output_quantization_factor = p.eltw_oqf;
+            d.activation = CLDNN_HIP_ACT_NONE;
+            if (p.eltw_with_act) d.activation = p.eltw_slope == 0.0f ? CLDNN_HIP_ACT_RELU : CLDNN_HIP_ACT_RELU_SLOPE;
+            d.m = p.eltw_slope;
+            hip_check(cldnn_hip_eltwise(eng->h, &d, src, calib, out->device_ptr()));
             break;
         }
         case prim_type::convolution:
@@ -348,7 +359,14 @@ void cldnn_add_primitive(cldnn_topology topology, const struct cldnn_primitive_d
             p->eltw_with_act = d->with_activation != 0;
             p->eltw_slope = d->activation_negative_slope;
             for (size_t i = 0; i < d->stride.size; ++i) p->eltw_stride.push_back(d->stride.data[i]);
-            HOST_REQUIRE(d->coefficients.size == 0, CLDNN_INVALID_ARG, "eltwise coefficients are not supported by this library");
+            // reference api/CPP/eltwise.hpp:230-252
+            HOST_REQUIRE(d->mode >= cldnn_eltwise_sum && d->mode <= cldnn_eltwise_mod, CLDNN_INVALID_ARG,
+                         "eltwise: the comparison and logic modes are not supported by this library");
+            for (size_t i = 0; i < d->coefficients.size; ++i) p->eltw_coefficients.push_back(d->coefficients.data[i]);
+            HOST_REQUIRE(d->mode == cldnn_eltwise_sum || p->eltw_coefficients.empty(), CLDNN_INVALID_ARG,
+                         "Only eltwise sum operation supports blob-wise coefficients");
+            HOST_REQUIRE(p->eltw_coefficients.empty() || p->eltw_coefficients.size() == p->inputs.size(), CLDNN_INVALID_ARG,
+                         "Invalid eltwise sum coefficients count (should be equal to 0 or input.size)");
             break;
         }
         case prim_type::convolution: {

@@ -118,6 +118,7 @@ struct prim {
     bool eltw_with_act = false;
     float eltw_slope = 0.f;
     std::vector<cldnn_tensor> eltw_stride;
+    std::vector<float> eltw_coefficients;
     // convolution / fused conv part
     cldnn_tensor input_offset{}, stride{}, dilation{}, output_size{}, padding_above{}, padding_below{};
     bool with_activation = false;

@@ -243,22 +243,35 @@ static void calc_layout(node* n)
         break;
     }
     case prim_type::eltwise: {
-        HOST_REQUIRE(n->deps.size() >= 2, CLDNN_INVALID_ARG, "eltwise needs two inputs");
-        const cldnn_layout &a = n->deps[0]->out, &b = n->deps[1]->out;
+        const size_t count = p.inputs.size();
+        HOST_REQUIRE(count >= 2 && n->deps.size() >= count, CLDNN_INVALID_ARG, "eltwise needs two inputs");
+        HOST_REQUIRE(count <= CLDNN_HIP_ELTWISE_MAX_INPUTS, CLDNN_INVALID_ARG, "eltwise: at most 4 inputs are supported by this library");
+        const cldnn_layout& a = n->deps[0]->out;
+        // reference src/eltwise.cpp:38-46
+        if (is_int8(a.data_type))
+            HOST_REQUIRE(p.eltw_mode != cldnn_eltwise_pow, CLDNN_INVALID_ARG, "Requested eltwise mode is not supported for integer types.");
         n->out = a;
         if (!p.eltw_stride.empty()) {
             // strided inputs: the first input's size divided by its stride (reference src/eltwise.cpp:59-66)
-            HOST_REQUIRE(p.eltw_stride.size() == 2, CLDNN_INVALID_ARG, "eltwise needs one stride per input");
+            HOST_REQUIRE(p.eltw_stride.size() == count, CLDNN_INVALID_ARG, "eltwise needs one stride per input");
             for (int i = 2; i < 4; ++i) {
-                HOST_REQUIRE(p.eltw_stride[0].sizes[i] > 0 && p.eltw_stride[1].sizes[i] > 0, CLDNN_INVALID_ARG, "eltwise stride must be positive");
+                for (size_t k = 0; k < count; ++k)
+                    HOST_REQUIRE(p.eltw_stride[k].sizes[i] > 0, CLDNN_INVALID_ARG, "eltwise stride must be positive");
                 n->out.size.sizes[i] = a.size.sizes[i] / p.eltw_stride[0].sizes[i];
-                HOST_REQUIRE(n->out.size.sizes[i] == b.size.sizes[i] / p.eltw_stride[1].sizes[i], CLDNN_DIMENSION_MISMATCH,
-                             "eltwise inputs differ in size after striding");
+                for (size_t k = 1; k < count; ++k)
+                    HOST_REQUIRE(n->out.size.sizes[i] == n->deps[k]->out.size.sizes[i] / p.eltw_stride[k].sizes[i],
+                                 CLDNN_DIMENSION_MISMATCH, "eltwise inputs differ in size after striding");
             }
         } else {
+            // broadcast: every axis takes the largest size among the inputs (reference src/eltwise.cpp:68-72)
             for (int i = 0; i < 4; ++i)
-                HOST_REQUIRE(a.size.sizes[i] == b.size.sizes[i], CLDNN_DIMENSION_MISMATCH,
-                             "eltwise inputs differ in size (broadcast is not supported)");
+                for (size_t k = 1; k < count; ++k) n->out.size.sizes[i] = std::max(n->out.size.sizes[i], n->deps[k]->out.size.sizes[i]);
+            for (int i = 0; i < 4; ++i)
+                for (size_t k = 0; k < count; ++k) {
+                    const int s = n->deps[k]->out.size.sizes[i];
+                    HOST_REQUIRE(s == n->out.size.sizes[i] || s == 1, CLDNN_DIMENSION_MISMATCH,
+                                 "eltwise inputs differ in size and cannot be broadcast");
+                }
         }
         if (p.out_dt.enabled) n->out.data_type = p.out_dt.data_type;
         break;
@@ -370,6 +383,118 @@ static void fuse_activations(cldnn_program_impl* prog)
         in->p->output_padding = a->p->output_padding;
         for (node* u : std::vector<node*>(a->users)) replace_dep(u, a, in);
         remove_node(prog, a);
+    }
+}
+
+static bool filter_is_1x1(node* conv)
+{
+    node* w = dep_named(conv, conv->p->weights.at(0));
+    return w->out.size.sizes[2] == 1 && w->out.size.sizes[3] == 1;
+}
+
+// An eltwise whose every user is a 1x1 convolution with one and the same stride > 1 computes only the elements those
+// convolutions read: the stride moves into the eltwise and the convolutions become stride 1
+// (reference src/graph_optimizer/eltwise_shrinking.cpp:25-132).
+static void eltwise_shrinking(cldnn_program_impl* prog)
+{
+    for (auto& u : prog->nodes) {
+        node* e = u.get();
+        if (e->p->type != prim_type::eltwise || !e->p->eltw_stride.empty() || e->users.empty() || e->is_output) continue;
+        if (!is_int8(e->out.data_type) && e->out.data_type != cldnn_f32) continue;
+        int sx = 0, sy = 0;
+        bool can_shrink = true;
+        for (node* c : e->users) {
+            if (c->p->type != prim_type::convolution || c->p->fully_connected || c->p->weights.size() != 1 || c->deps[0] != e
+                || std::count(c->deps.begin(), c->deps.end(), e) != 1 || !filter_is_1x1(c)) {
+                can_shrink = false;
+                break;
+            }
+            const int cx = spatial(c->p->stride, 0), cy = spatial(c->p->stride, 1);
+            if (cx <= 1 && cy <= 1) {
+                can_shrink = false;
+                break;
+            }
+            if (sx == 0) sx = cx, sy = cy;
+            // a 1x1 window at offset 0: the convolution reads exactly the elements (y * sy, x * sx)
+            if (cx != sx || cy != sy || spatial(c->p->input_offset, 0) != 0 || spatial(c->p->input_offset, 1) != 0
+                || spatial(c->p->padding_above, 0) != 0 || spatial(c->p->padding_above, 1) != 0
+                || spatial(c->p->padding_below, 0) != 0 || spatial(c->p->padding_below, 1) != 0) {
+                can_shrink = false;
+                break;
+            }
+        }
+        if (!can_shrink) continue;
+        // every convolution keeps the output size it had: the shrunk eltwise must have exactly that size
+        for (node* c : e->users)
+            if (c->out.size.sizes[2] != e->out.size.sizes[2] / sx || c->out.size.sizes[3] != e->out.size.sizes[3] / sy) can_shrink = false;
+        if (!can_shrink) continue;
+        e->p = std::make_shared<prim>(*e->p);
+        cldnn_tensor st = make_tensor(1, 1, sx, sy);
+        e->p->eltw_stride.assign(e->p->inputs.size(), st);
+        calc_layout(e);
+        for (node* c : e->users) {
+            c->p = std::make_shared<prim>(*c->p);
+            c->p->stride.sizes[2] = 1, c->p->stride.sizes[3] = 1;
+            c->p->with_output_size = false;
+            calc_layout(c);
+        }
+    }
+}
+
+// The stride of a strided eltwise input moves up into the convolutions that produce it, so that they no longer compute
+// elements nobody reads: through 1x1 convolutions (which pass it on to their own producer) into the first convolution
+// whose filter is wide enough to take it as its own stride (reference src/graph_optimizer/eltwise_remove_stride.cpp:27-105).
+static bool conv_stride_extend(node* c, cldnn_tensor& st)
+{
+    if (c->users.size() > 1 || c->is_output || c->p->type != prim_type::convolution || c->p->fully_connected || c->p->weights.size() != 1)
+        return false;
+    if (filter_is_1x1(c)) {
+        // only a pointwise convolution of stride 1 without padding commutes with the sub-sampling
+        if (spatial(c->p->stride, 0) != 1 || spatial(c->p->stride, 1) != 1 || spatial(c->p->input_offset, 0) != 0
+            || spatial(c->p->input_offset, 1) != 0)
+            return false;
+        node* d = c->deps[0];
+        if (!conv_stride_extend(d, st)) return false;
+        c->p = std::make_shared<prim>(*c->p);
+        c->p->with_output_size = false;
+        calc_layout(c);
+        return true;
+    }
+    node* w = dep_named(c, c->p->weights.at(0));
+    const int fx = w->out.size.sizes[2], fy = w->out.size.sizes[3];
+    const int cx = spatial(c->p->stride, 0), cy = spatial(c->p->stride, 1), ex = st.sizes[2], ey = st.sizes[3];
+    // reference :54-55; the sub-sampled outputs (y * ey, x * ex) of a stride-(cy, cx) convolution are the outputs of a
+    // convolution of stride (cy * ey, cx * ex) -- the reference adds, which is the same for the stride-1 convolutions
+    // it meets, and a product is what the geometry asks for otherwise
+    if (fx - (cx + (ex - 1)) < 0 || fy - (cy + (ey - 1)) < 0) return false;
+    const cldnn_layout before = c->out;
+    auto p = std::make_shared<prim>(*c->p);
+    p->stride.sizes[2] = cx * ex, p->stride.sizes[3] = cy * ey;
+    p->with_output_size = false;
+    std::shared_ptr<prim> old = c->p;
+    c->p = p;
+    calc_layout(c);
+    if (c->out.size.sizes[2] != before.size.sizes[2] / ex || c->out.size.sizes[3] != before.size.sizes[3] / ey) {
+        c->p = old;  // the strided convolution would not produce exactly the sub-sampled tensor
+        calc_layout(c);
+        return false;
+    }
+    st.sizes[2] = 1, st.sizes[3] = 1;
+    return true;
+}
+
+static void eltwise_remove_stride(cldnn_program_impl* prog)
+{
+    for (auto& u : prog->nodes) {
+        node* e = u.get();
+        if (e->p->type != prim_type::eltwise || e->p->eltw_stride.empty()) continue;
+        for (size_t i = 0; i < e->p->inputs.size(); ++i) {
+            cldnn_tensor& st = e->p->eltw_stride[i];
+            if (st.sizes[2] == 1 && st.sizes[3] == 1) continue;
+            if (std::count(e->deps.begin(), e->deps.end(), e->deps[i]) != 1) continue;
+            conv_stride_extend(e->deps[i], st);
+        }
+        calc_layout(e);
     }
 }
 
@@ -750,6 +875,8 @@ void build_program(cldnn_program_impl* prog, cldnn_topology_impl* topo, const st
 
     if (prog->optimize_data) {
         fuse_activations(prog);
+        eltwise_shrinking(prog);
+        eltwise_remove_stride(prog);
         fuse_conv_eltwise(prog);
         sort_nodes(prog);
         for (auto& u : prog->nodes) u->out.format = cldnn_format_any;
@@ -759,9 +886,6 @@ void build_program(cldnn_program_impl* prog, cldnn_topology_impl* topo, const st
     }
     for (auto& u : prog->nodes) calc_layout(u.get());
     prepare_borders(prog);
-    for (auto& u : prog->nodes)
-        HOST_REQUIRE(u->p->type != prim_type::eltwise || u->p->eltw_stride.empty(), CLDNN_INVALID_ARG,
-                     "eltwise " + u->p->id + ": strides are only supported when the eltwise is fused into a convolution");
     if (!prog->engine) return;  // planning only: the graph is inspected, nothing is compiled
     for (auto& u : prog->nodes) {
         node* n = u.get();
@@ -794,6 +918,11 @@ std::string describe_node(const node* n)
     if (p.type == prim_type::fused_conv_eltwise) {
         s += ",\"eltw_stride\":" + (p.eltw_stride.empty() ? std::string("null") : four(p.eltw_stride[0].sizes));
         s += ",\"eltw_slope\":" + std::to_string(p.eltw_slope) + ",\"eltw_calib\":\"" + p.eltw_calib + "\"";
+    }
+    if (p.type == prim_type::eltwise) {
+        s += ",\"mode\":" + std::to_string(p.eltw_mode) + ",\"strides\":[";
+        for (size_t i = 0; i < p.eltw_stride.size(); ++i) s += (i ? "," : "") + four(p.eltw_stride[i].sizes);
+        s += "]";
     }
     if (n->conv)
         s += std::string(",\"kernel\":\"") + n->conv_info.kernel_name + "\",\"grid\":" + std::to_string(n->conv_info.grid)

@@ -76,8 +76,12 @@ typedef enum {
     cldnn_eltwise_sum,
     cldnn_eltwise_sub,
     cldnn_eltwise_max,
-    cldnn_eltwise_prod
-} cldnn_eltwise_mode; /* only cldnn_eltwise_sum is implemented */
+    cldnn_eltwise_prod,
+    cldnn_eltwise_div,
+    cldnn_eltwise_min,
+    cldnn_eltwise_pow,
+    cldnn_eltwise_mod
+} cldnn_eltwise_mode; /* the reference's comparison and logic modes (eq ... or) are not part of this library */
 
 CLDNN_BEGIN_PRIMITIVE_DESC(eltwise)
 cldnn_primitive_id output_calibration_factors;

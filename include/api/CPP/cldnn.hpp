@@ -628,15 +628,31 @@ private:
     mutable id_list _in;
 };
 
-enum class eltwise_mode : int32_t { sum = cldnn_eltwise_sum, sub = cldnn_eltwise_sub, max = cldnn_eltwise_max, prod = cldnn_eltwise_prod };
+enum class eltwise_mode : int32_t { sum = cldnn_eltwise_sum, sub = cldnn_eltwise_sub, max = cldnn_eltwise_max, prod = cldnn_eltwise_prod,
+                                    div = cldnn_eltwise_div, min = cldnn_eltwise_min, pow = cldnn_eltwise_pow, mod = cldnn_eltwise_mod };
 
 struct eltwise : primitive {
     primitive_id output_calibration_factors;
     float output_quantization_factor = 1.0f;
     eltwise_mode mode;
+    std::vector<float> coefficients;
     std::vector<tensor> stride;
     bool with_activation;
     float activation_negative_slope;
+    // any number of inputs, combined left to right (reference api/CPP/eltwise.hpp:196-225 and 279-311)
+    eltwise(const primitive_id& id, const std::vector<primitive_id>& inputs, eltwise_mode mode, bool with_activation = false,
+            float activation_slp = 0.0f, const padding& output_padding = padding())
+        : primitive(id, inputs, output_padding), mode(mode), with_activation(with_activation), activation_negative_slope(activation_slp) {}
+    eltwise(const primitive_id& id, const std::vector<primitive_id>& inputs, eltwise_mode mode, const std::vector<float>& coefficients,
+            bool with_activation = false, float activation_slp = 0.0f, const padding& output_padding = padding())
+        : primitive(id, inputs, output_padding), mode(mode), coefficients(coefficients), with_activation(with_activation),
+          activation_negative_slope(activation_slp)
+    {
+        if (mode == eltwise_mode::sum && !coefficients.empty() && coefficients.size() != inputs.size())
+            throw std::invalid_argument("Invalid eltwise sum coefficients count (should be equal to 0 or input.size)");
+        if (mode != eltwise_mode::sum && !coefficients.empty())
+            throw std::invalid_argument("Only eltwise sum operation supports blob-wise coefficients");
+    }
     eltwise(const primitive_id& id, const primitive_id& input, const primitive_id& input2, eltwise_mode mode, bool with_activation = false,
             float activation_slp = 0.0f, const padding& output_padding = padding())
         : primitive(id, {input, input2}, output_padding), mode(mode), with_activation(with_activation), activation_negative_slope(activation_slp) {}
@@ -659,7 +675,7 @@ struct eltwise : primitive {
         _d.output_calibration_factors = output_calibration_factors.c_str();
         _d.output_quantization_factor = output_quantization_factor;
         _d.mode = (int32_t)mode;
-        _d.coefficients = cldnn_float_arr{nullptr, 0};
+        _d.coefficients = cldnn_float_arr{coefficients.data(), coefficients.size()};
         _d.with_activation = with_activation;
         _d.activation_negative_slope = activation_negative_slope;
         _strides.assign(stride.begin(), stride.end());

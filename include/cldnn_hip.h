@@ -165,6 +165,37 @@ cldnn_hip_status cldnn_hip_eltwise_sum(cldnn_hip_engine e, const void* a_dev, co
                                        const cldnn_hip_tensor* dst, int32_t quantized, const float* calib_dev,
                                        float output_quantization_factor, int32_t activation, float m, float n);
 
+/* General element-wise primitive: 2..CLDNN_HIP_ELTWISE_MAX_INPUTS inputs combined left to right,
+ * r = op(...op(op(in0, in1), in2)..., inN-1)  (reference src/gpu/eltwise_gpu.cpp:80-140,
+ * kernel_selector/core/actual_kernels/eltwise/eltwise_kernel_base.cpp:236-352,
+ * kernel_selector/core/cl_kernels/generic_eltwise_ref.cl:106-135 and 311-330).
+ * Input i is read at (b % B_i, f % F_i, (y * stride_y[i]) % Y_i, (x * stride_x[i]) % X_i): strides shrink, sizes of
+ * one broadcast.  The arithmetic type follows the first input: float data in float; int8 data in the 8-bit type with
+ * wrap-around after every step, unless `quantized`: then in int, followed by round(r * factor) (calib_dev[f] or
+ * output_quantization_factor), saturation to signed char and the activation.  Integer division and modulo by zero
+ * give 0 here (undefined in the reference).  Coefficients multiply the inputs of a float sum. */
+enum {
+    CLDNN_HIP_ELTWISE_SUM = 0, CLDNN_HIP_ELTWISE_SUB = 1, CLDNN_HIP_ELTWISE_MAX = 2, CLDNN_HIP_ELTWISE_PROD = 3,
+    CLDNN_HIP_ELTWISE_DIV = 4, CLDNN_HIP_ELTWISE_MIN = 5, CLDNN_HIP_ELTWISE_POW = 6, CLDNN_HIP_ELTWISE_MOD = 7
+};  /* the values of cldnn_eltwise_mode (reference api/C/eltwise.h:33-67); POW for float data only */
+#define CLDNN_HIP_ELTWISE_MAX_INPUTS 4
+typedef struct {
+    int32_t mode;                 /* CLDNN_HIP_ELTWISE_* */
+    int32_t n_inputs;
+    cldnn_hip_tensor inputs[CLDNN_HIP_ELTWISE_MAX_INPUTS];
+    int32_t stride_y[CLDNN_HIP_ELTWISE_MAX_INPUTS], stride_x[CLDNN_HIP_ELTWISE_MAX_INPUTS];  /* 0 = 1 */
+    int32_t has_coefficients;     /* float sum only */
+    float coefficients[CLDNN_HIP_ELTWISE_MAX_INPUTS];
+    cldnn_hip_tensor output;
+    int32_t quantized;
+    float output_quantization_factor;
+    int32_t activation;           /* CLDNN_HIP_ACT_* */
+    float m, n;
+} cldnn_hip_eltwise_desc;
+/* asynchronous on the engine stream; device pointers; calib_dev may be NULL */
+cldnn_hip_status cldnn_hip_eltwise(cldnn_hip_engine e, const cldnn_hip_eltwise_desc* desc, const void* const* inputs_dev,
+                                   const float* calib_dev, void* output_dev);
+
 /* ------------------------------------------------------------------ pooling
  * The layers between the convolutions of an int8 network: sliding-window maximum / average.  Replaces the pooling
  * kernels (reference src/gpu/pooling_gpu.cpp:60-160, kernel_selector/core/cl_kernels/pooling_gpu_int8_ref.cl:15-140,

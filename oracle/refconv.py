@@ -209,6 +209,85 @@ def fully_connected(x, w, bias=None, wqf=None, calib=None, *, iqf=1.0, oqf=1.0, 
     return conv(x, w, bias, wqf=wqf, calib=calib, iqf=iqf, oqf=oqf, act=act, act_m=act_m, fc=wqf is not None)
 
 
+def _round_half_away(v):
+    """OpenCL round() of float32 values (exact: the half is added in double)."""
+    v = np.asarray(v, np.float32).astype(np.float64)
+    return np.sign(v) * np.floor(np.abs(v) + 0.5)
+
+
+def eltwise(inputs, mode="sum", strides=None, calib=None, oqf=1.0, relu=False, slope=0.0, coefficients=None):
+    """The reference's stand-alone eltwise on logical [B, F, Y, X] arrays.
+    - output size: input 0 divided by its stride when strides are given, else the per-axis maximum of the inputs
+      (src/eltwise.cpp:57-73);
+    - input i is read at (b % B_i, f % F_i, (y * sy_i) % Y_i, (x * sx_i) % X_i)
+      (kernel_selector/core/cl_kernels/generic_eltwise_ref.cl:106-135);
+    - the inputs are combined left to right, tmp_k = op(tmp_(k-1), input_(k+1))
+      (src/gpu/eltwise_gpu.cpp:80-94), in the first input's type: float, or the 8-bit integer type with wrap-around
+      after every step; with calib / oqf != 1 ("quantized") in int, then round(r * factor), convert_char_sat, and the
+      activation on the char (kernel_selector/core/actual_kernels/eltwise/eltwise_kernel_base.cpp:238-340,
+      generic_eltwise_ref.cl:311-330);
+    - coefficients scale the inputs of a float sum (eltwise_kernel_base.cpp:259-275).
+    Integer division / modulo by zero give 0 (undefined in the reference).  strides: one (sy, sx) per input."""
+    ins = [np.asarray(a) for a in inputs]
+    n = len(ins)
+    strides = [(1, 1)] * n if strides is None else [tuple(s) for s in strides]
+    if any(s != (1, 1) for s in strides):
+        B, F = ins[0].shape[0], ins[0].shape[1]
+        Y, X = ins[0].shape[2] // strides[0][0], ins[0].shape[3] // strides[0][1]
+    else:
+        B, F, Y, X = (max(a.shape[d] for a in ins) for d in range(4))
+
+    def read(i):
+        a, (sy, sx) = ins[i], strides[i]
+        return a[np.ix_(np.arange(B) % a.shape[0], np.arange(F) % a.shape[1], (np.arange(Y) * sy) % a.shape[2],
+                        (np.arange(X) * sx) % a.shape[3])]
+
+    dt = ins[0].dtype
+    quantized = dt != np.float32 and (calib is not None or oqf != 1.0)
+    if dt == np.float32:
+        def op(a, b):
+            with np.errstate(all="ignore"):
+                return {"sum": lambda: a + b, "sub": lambda: a - b, "max": lambda: np.fmax(a, b), "prod": lambda: a * b,
+                        "div": lambda: a / b, "min": lambda: np.fmin(a, b), "pow": lambda: np.power(a, b),
+                        "mod": lambda: np.fmod(a, b)}[mode]().astype(np.float32)
+        v = read(0).astype(np.float32)
+        if coefficients is not None:
+            v = v * np.float32(coefficients[0])
+        for i in range(1, n):
+            w = read(i).astype(np.float32)
+            if coefficients is not None:
+                w = w * np.float32(coefficients[i])
+            v = op(v, w)
+        if relu:
+            v = np.maximum(v, 0) + np.float32(slope) * np.minimum(v, 0)
+        return v.astype(np.float32)
+
+    def trunc_div(a, b):
+        q = np.abs(a) // np.where(b == 0, 1, np.abs(b))
+        return np.where(b == 0, 0, np.sign(a) * np.sign(b) * q)
+
+    def iop(a, b):
+        if mode == "div":
+            return trunc_div(a, b)
+        if mode == "mod":
+            return np.where(b == 0, 0, a - trunc_div(a, b) * b)
+        return {"sum": lambda: a + b, "sub": lambda: a - b, "max": lambda: np.maximum(a, b), "prod": lambda: a * b,
+                "min": lambda: np.minimum(a, b)}[mode]()
+    v = read(0).astype(np.int64)
+    for i in range(1, n):
+        # an operand of another type is cast to the unit type first (float -> char goes toward zero)
+        v = iop(v, np.trunc(read(i)).astype(np.int64).astype(dt).astype(np.int64))
+        # arithmetic in the unit type wraps; the quantized form computes in int (a product of four uint8 values can
+        # leave its range: undefined in C, two's-complement wrap-around on the hardware)
+        v = v.astype(np.int32 if quantized else dt).astype(np.int64)
+    if quantized:
+        f = np.float32(oqf) if calib is None else np.asarray(calib, np.float32).reshape(1, -1, 1, 1)
+        v = np.clip(_round_half_away(v.astype(np.float32) * f), -128, 127).astype(np.int64)
+    if relu:
+        v = np.maximum(v, 0) + int(slope) * np.minimum(v, 0)
+    return v.astype(dt)
+
+
 def eltwise_sum(a, b, calib=None, oqf=1.0, relu=False):
     """Stand-alone element-wise sum of two int8 tensors in its quantized form (reference
     kernel_selector/core/cl_kernels/generic_eltwise_ref.cl:311-330): int sum, round((float)sum * factor) half away from
@@ -216,6 +295,5 @@ def eltwise_sum(a, b, calib=None, oqf=1.0, relu=False):
     s = a.astype(np.int32) + b.astype(np.int32)
     f = np.float32(oqf) if calib is None else np.asarray(calib, np.float32).reshape(1, -1, 1, 1)
     v = s.astype(np.float32) * f
-    r = np.sign(v) * np.floor(np.abs(v) + np.float32(0.5))
-    c = np.clip(r, -128, 127).astype(np.int8)
+    c = np.clip(_round_half_away(v), -128, 127).astype(np.int8)
     return np.maximum(c, 0) if relu else c

@@ -286,6 +286,40 @@ def test_mfma_fused_eltwise(eng, fast, eltw_dt):
     assert_same(ro, go)
 
 
+@pytest.mark.parametrize("shape", [(2, 64, 14, 14, 256, 1, 1, 1), (2, 128, 7, 7, 512, 1, 1, 1), (1, 64, 15, 15, 64, 3, 3, 2),
+                                   (3, 64, 28, 28, 64, 1, 1, 1)],
+                         ids=["closer", "closer_small", "3x3_s2", "narrow"])
+@pytest.mark.parametrize("es", [(2, 2), (1, 3)], ids=["es2x2", "es1x3"])
+def test_fused_eltwise_read_with_stride(eng, shape, es):
+    """the residual operand is a larger tensor read at (y * esy, x * esx): what a shrunk residual sum hands to the
+    convolution it is fused into (reference fused_conv_eltwise_gpu_ref.cl:180-196)"""
+    B, IFM, H, W, OFM, FY, FX, st = shape
+    x, w, bias, wqf, calib = problem(41, B, IFM, H, W, OFM, FY, FX)
+    pad = (FY // 2, FX // 2)
+    OH, OW = (H + 2 * pad[0] - FY) // st + 1, (W + 2 * pad[1] - FX) // st + 1
+    r = np.random.default_rng(6)
+    e = r.integers(-128, 128, (B, OFM, OH * es[0] + 1, OW * es[1])).astype(np.int8)
+    ecal = r.uniform(0.3, 1.2, OFM).astype(np.float32)
+    kw = dict(stride=(st, st), pad=pad, out_dt="s8", act="none", eltw=e, eltw_act="relu", eltw_calib=ecal, eltw_stride=es)
+    ref = rc.conv(x, w, bias, wqf=wqf, calib=calib, **kw)
+    # the operand really is sub-sampled
+    plain = rc.conv(x, w, bias, wqf=wqf, calib=calib, **dict(kw, eltw=np.ascontiguousarray(e[:, :, ::es[0], ::es[1]][:, :, :OH, :OW]),
+                                                             eltw_stride=(1, 1)))
+    np.testing.assert_array_equal(ref, plain)
+    for fmt, impl in (("bfyx", hip.IMPL_REF), ("fs_b_yx_fsv16", hip.IMPL_AUTO)):
+        assert_same(ref, hip.conv_forward(eng, x, w, bias, wqf, calib, fmt=fmt, impl=impl, **kw))
+    seen = set()
+    for tile in [t for t in tiles() if not tile_names()[t - 1].startswith("stem")]:
+        try:
+            got, info = hip.conv_forward(eng, x, w, bias, wqf, calib, fmt="fs_b_yx_fsv16", tile=tile, want_info=True,
+                                         in_pad=(pad[0] + (1 if FY > 1 else 0), pad[1]), **kw)
+        except hip.HipError:  # a kernel family that does not take this shape refuses it
+            continue
+        seen.add(info.kernel_name.decode().split("<")[0])
+        assert_same(ref, got)
+    assert len(seen) >= 3, seen
+
+
 def test_mfma_padded_buffers(eng):
     # physical zero borders on input and output (what a following 3x3 layer asks of its producer)
     x, w, bias, wqf, calib = problem(16, 2, 64, 14, 14, 64, 3, 3)

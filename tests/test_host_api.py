@@ -332,6 +332,63 @@ def test_conv_eltwise_not_fused(kw):
     assert "conv2" in ids and "sum" in ids
 
 
+def downsampling_junction(size=8, user_stride=(2, 2), second_user="conv", mid_filter=3):
+    """the place where a Caffe-form ResNet halves its resolution: a residual sum whose users are the two stride-2 1x1
+    convolutions of the next block"""
+    Cn = 16
+    w1, w3 = attach(np.ones((Cn, Cn, 1, 1), np.int8)), attach(np.ones((Cn, Cn, mid_filter, mid_filter), np.int8))
+    conv = lambda i, src, w, **kw: cl.convolution(i, src, [w], None, ["q"], ["c"], **kw)  # noqa: E731
+    t = cl.topology(cl.input_layout("in", cl.layout(DT.i8, F.bfyx, cl.tensor(1, Cn, size, size))), cl.data("w1", w1), cl.data("w3", w3),
+                    cl.data("q", vec(Cn)), cl.data("c", vec(Cn)),
+                    conv("a", "in", "w1", with_activation=True),
+                    conv("b", "a", "w3", with_activation=True, input_offset=cl.tensor(0, 0, -(mid_filter // 2), -(mid_filter // 2), 0)),
+                    conv("c_", "b", "w1"),
+                    cl.eltwise("res", "in", "c_", cl.eltwise_mode.sum, True, 0.0, output_calibration_factors="c"),
+                    conv("down1", "res", "w1", stride=cl.tensor(1, 1, 2, 2)))
+    if second_user == "conv":
+        t.add(conv("down2", "res", "w1", stride=cl.tensor(1, 1, user_stride[0], user_stride[1])))
+    elif second_user == "pool":
+        t.add(cl.pooling("down2", "res", cl.pooling_mode.max, cl.tensor(1, 1, 2, 2), cl.tensor(1, 1, 2, 2)))
+    return t
+
+
+def conv_node(nodes, i):
+    """an output convolution of the blocked path is followed by a reorder that takes over its id"""
+    return nodes.get(i + "_fsv16", nodes[i])
+
+
+def test_eltwise_shrinking_and_stride_removal():
+    """reference src/graph_optimizer/eltwise_shrinking.cpp, eltwise_remove_stride.cpp: the sum computes only what the
+    stride-2 users read, and the branch before it shrinks back to the first convolution that can take the stride"""
+    plain = by_id(cl.plan(downsampling_junction()))
+    assert plain["res"]["size"][2:] == [8, 8] and plain["b"]["stride"][2:] == [1, 1] and plain["down1"]["stride"][2:] == [2, 2]
+    opt = by_id(cl.plan(downsampling_junction(), cl.build_options(optimize_data=True)))
+    f = opt["c__fused_res"]
+    assert f["size"][2:] == [4, 4] and f["stride"][2:] == [1, 1] and f["eltw_stride"][2:] == [2, 2]
+    assert opt["b"]["stride"][2:] == [2, 2] and opt["b"]["size"][2:] == [4, 4]
+    assert opt["a"]["size"][2:] == [8, 8]
+    assert conv_node(opt, "down1")["stride"][2:] == [1, 1] and conv_node(opt, "down2")["stride"][2:] == [1, 1]
+    assert opt["down1"]["size"] == plain["down1"]["size"] and opt["down2"]["size"] == plain["down2"]["size"]
+
+
+@pytest.mark.parametrize("kw", [dict(user_stride=(1, 1)), dict(user_stride=(2, 1)), dict(second_user="pool"), dict(size=7)],
+                         ids=["a_user_of_stride_1", "users_differ", "a_user_is_no_convolution", "odd_size"])
+def test_eltwise_not_shrunk(kw):
+    opt = by_id(cl.plan(downsampling_junction(**kw), cl.build_options(optimize_data=True)))
+    f = opt["c__fused_res"]
+    assert f["size"][2:] == [kw.get("size", 8)] * 2 and f["eltw_stride"] is None
+    assert conv_node(opt, "down1")["stride"][2:] == [2, 2] and opt["b"]["stride"][2:] == [1, 1]
+
+
+def test_eltwise_stride_stays_where_no_convolution_takes_it():
+    """a 1x1 convolution in the middle of the branch cannot absorb the stride: the sum stays strided on that input
+    and the closing convolution takes the stride when the two are fused"""
+    opt = by_id(cl.plan(downsampling_junction(mid_filter=1), cl.build_options(optimize_data=True)))
+    f = opt["c__fused_res"]
+    assert f["size"][2:] == [4, 4] and f["stride"][2:] == [2, 2] and f["eltw_stride"][2:] == [2, 2]
+    assert opt["b"]["size"][2:] == [8, 8] and conv_node(opt, "down1")["stride"][2:] == [1, 1]
+
+
 def test_conv_eltwise_fusing_reaches_every_block_of_a_chain():
     """three residual blocks in a row: each sum reads the previous (fused) block's output and its own closing 1x1
     convolution; every one of them fuses (the fused node keeps the sum's place in the execution order)"""
@@ -365,9 +422,8 @@ def test_conv_eltwise_fusing_moves_eltwise_stride_into_the_conv():
     f = by_id(nodes)["conv_fused_sum"]
     assert f["stride"][2:] == [2, 2] and f["eltw_stride"][2:] == [2, 2]
     assert f["size"] == [1, 16, 4, 4]
-    with pytest.raises(cl.error) as e:  # left unfused, a strided eltwise is refused: only the fused form is served
-        cl.plan(t)
-    assert "fused into a convolution" in str(e.value)
+    unfused = by_id(cl.plan(t))  # left unfused, the stand-alone eltwise does the sub-sampling
+    assert unfused["sum"]["type"] == "eltwise" and unfused["sum"]["size"] == [1, 16, 4, 4] and unfused["conv"]["size"] == [1, 16, 8, 8]
 
 
 # ------------------------------------------------------------------------------------------ layout rule

@@ -85,14 +85,23 @@ def test_resnet50_int8_network_matches_the_oracle():
     params = rn.random_weights(seed=11)
     run_oracle(x, params, fused=BLOCKS, calibrate=True)
     topo = rn.topology(cl, eng, params, B)
-    watch = ["pool1", "res2a", "res3d", "res4f", "res5c", "pool5", "fc1000"]
-    for optimize in (True, False):
+    # a watched sum is an output: it is neither fused nor shrunk.  The first list leaves the junction behind res2c to the
+    # eltwise_shrinking / eltwise_remove_stride passes, the second one those behind res3d and res4f.
+    for optimize, watch in ((True, ["pool1", "res2a", "res3d", "res4f", "res5c", "pool5", "fc1000"]),
+                            (True, ["res2c", "res3a", "res4b", "res5a", "fc1000"]),
+                            (False, ["pool1", "res2a", "res3d", "res4f", "res5c", "pool5", "fc1000"])):
         # optimize_data fuses a residual sum into its closing convolution unless the sum is itself an output; the plan says
         # which ones (node ids <convolution>_fused_<sum>), and the oracle follows it: the two forms differ where the
         # convolution's own result leaves the int8 range
         opts = cl.build_options(optimize_data=optimize, outputs=watch)
-        fused = [n["id"].split("_fused_")[1] for n in cl.plan(topo, opts) if "_fused_" in n["id"]]
+        plan = {n["id"]: n for n in cl.plan(topo, opts)}
+        fused = [i.split("_fused_")[1] for i in plan if "_fused_" in i]
         assert sorted(fused) == (sorted(b for b in BLOCKS if b not in watch) if optimize else [])
+        for junction, size in (("res2c", 28), ("res3d", 14), ("res4f", 7)):
+            name = "%s_branch2c_fused_%s" % (junction, junction)
+            if name in plan:  # the sum and the 3x3 convolution before it produce only what the stride-2 block behind them reads
+                assert plan[name]["size"][2:] == [size, size] and plan[name]["eltw_stride"][2:] == [2, 2]
+                assert plan[junction + "_branch2b"]["stride"][2:] == [2, 2]
         ref = run_oracle(x, params, fused=fused)
         assert 5 < np.abs(ref["res5c"].astype(np.int32)).mean() < 100 and len(np.unique(ref["fc1000"])) > 50  # alive to the end
         net = cl.network(eng, topo, opts)
@@ -126,4 +135,4 @@ def test_memory_pool_shares_buffers_without_changing_results():
         del net
     np.testing.assert_array_equal(logits[True], logits[False])
     np.testing.assert_array_equal(logits[True], run_oracle(x, params, fused=BLOCKS)["fc1000"])
-    assert used[True] < 0.8 * used[False], used
+    assert used[True] < 0.9 * used[False], used
