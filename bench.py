@@ -188,6 +188,14 @@ def network_workload(args):
     params["fc1000"]["calib"] = np.full(1000, 40.0 / (np.sqrt(2048) * 30.0 * 73.3), np.float32)
     t0 = time.perf_counter()
     topo, opts = rn.topology(cl, eng, params, batch), cl.build_options(optimize_data=True)
+    if args.tuning_cache:
+        # measure what the cache file does not hold yet (needs an engine with profiling), then run from the file
+        tuner = cl.engine(enable_profiling=True)
+        t0 = time.perf_counter()
+        cl.network(tuner, rn.topology(cl, tuner, params, batch),
+                   cl.build_options(optimize_data=True, tuning_config=(cl.tuning_mode.tuning_tune_and_cache, args.tuning_cache)))
+        log("tuning pass over %s: %.1f s" % (args.tuning_cache, time.perf_counter() - t0))
+        opts = cl.build_options(optimize_data=True, tuning_config=(cl.tuning_mode.tuning_use_cache, args.tuning_cache))
     net = cl.network(eng, topo, opts)
     x = r.integers(0, 256, (batch, 3, 224, 224)).astype(np.uint8)
     net.set_input_data("input", cl.make_memory(eng, x))
@@ -220,7 +228,7 @@ def network_workload(args):
         "unit": "images/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": dt / args.steps * 1e3,
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "i8xi8->i32 (f32 requantisation)", "data": "synthetic",
         "config": {"workload": "resnet50_b32_network", "batch": batch, "primitives": "53 convolution, 2 pooling, 16 eltwise (fused), 1 fully_connected",
-                   "build": "optimize_data", "executed_ops_per_step": ops, "nominal_ops_per_step": nominal},
+                   "build": "optimize_data" + (", tuning cache" if args.tuning_cache else ""), "executed_ops_per_step": ops, "nominal_ops_per_step": nominal},
         "roofline": {"bound": "mfma", "achieved": ops * args.steps / dt / 1e12, "peak": PEAK_INT8_OPS / 1e12, "unit": "TOP/s",
                      "frac": ops * args.steps / dt / PEAK_INT8_OPS, "traffic": None, "kernel": "all kernels of one network.execute()"},
         "cpu_baseline": None, "distinct_logit_values": int(len(np.unique(logits)))}), flush=True)
@@ -251,6 +259,8 @@ def main():
     ap.add_argument("--tune", action="store_true", help="try every row of the tile table on every layer, print the best")
     ap.add_argument("--only", default="", help="comma-separated layer names: run just these layers of the workload "
                                                "(same buffers every step, so their tensors stay cache-resident)")
+    ap.add_argument("--tuning-cache", default="", help="resnet50_b32_network only: tune what this cache file lacks "
+                                                       "(build option tuning_config, tune_and_cache), then run from it")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline / full-size check")
     ap.add_argument("--host-io", action="store_true",
                     help="also report the rate with the first layer's input crossing PCIe into the device and the last "

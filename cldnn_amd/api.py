@@ -591,16 +591,27 @@ class eltwise(_primitive):  # noqa: N801
     output_calibration_factors / output_quantization_factor (reference api/CPP/eltwise.hpp:78-260)."""
     type_fn = "cldnn_eltwise_type_id"
 
-    def __init__(self, prim_id, inp, inp2=None, mode=eltwise_mode.sum, with_activation=False, activation_slp=0.0,
-                 output_calibration_factors="", output_quantization_factor=1.0, stride=None, output_padding=None,
-                 output_data_type=None, coefficients=None):
-        """inp may be the list of all inputs (then inp2, if given, is the mode, as in eltwise(id, {inputs}, mode))."""
-        if isinstance(inp, (list, tuple)):
-            inputs = list(inp)
-            if inp2 is not None:
-                mode = inp2
-        else:
-            inputs = [inp, inp2]
+    def __init__(self, prim_id, inp, *args, **kw):
+        """eltwise(id, input, input2, mode, with_activation, activation_slp, ...) or, with the list of all inputs,
+        eltwise(id, [inputs], mode, with_activation, activation_slp, ...); keywords: output_calibration_factors,
+        output_quantization_factor, stride (one tensor per input), coefficients, output_padding, output_data_type."""
+        several = isinstance(inp, (list, tuple))
+        names = ([] if several else ["inp2"]) + ["mode", "with_activation", "activation_slp", "output_calibration_factors",
+                                                 "output_quantization_factor", "stride", "output_padding", "output_data_type", "coefficients"]
+        if len(args) > len(names):
+            raise TypeError("eltwise: too many positional arguments")
+        for k, v in zip(names, args):
+            if k in kw:
+                raise TypeError("eltwise: argument %s given twice" % k)
+            kw[k] = v
+        unknown = set(kw) - set(names) - {"inp2"}
+        if unknown:
+            raise TypeError("eltwise: unknown argument(s) %s" % sorted(unknown))
+        inputs = list(inp) if several else [inp, kw["inp2"]]
+        mode, with_activation, activation_slp = kw.get("mode", eltwise_mode.sum), kw.get("with_activation", False), kw.get("activation_slp", 0.0)
+        output_calibration_factors, output_quantization_factor = kw.get("output_calibration_factors", ""), kw.get("output_quantization_factor", 1.0)
+        stride, output_padding, output_data_type = kw.get("stride"), kw.get("output_padding"), kw.get("output_data_type")
+        coefficients = kw.get("coefficients")
         if coefficients:
             # reference api/CPP/eltwise.hpp:303-310
             if mode == eltwise_mode.sum and len(coefficients) != len(inputs):
@@ -707,10 +718,21 @@ class topology:  # noqa: N801
             self.h = None
 
 
+class tuning_mode:  # noqa: N801
+    tuning_disabled, tuning_use_cache, tuning_tune_and_cache = range(3)
+
+
+class c_tuning_config(C.Structure):
+    _fields_ = [("mode", C.c_int32), ("cache_file_path", C.c_char_p)]
+
+
 class build_options:  # noqa: N801
-    def __init__(self, optimize_data=False, outputs=None):
+    """optimize_data, outputs, tuning_config=(tuning_mode, cache file path) (reference api/CPP/program.hpp:68-135)"""
+
+    def __init__(self, optimize_data=False, outputs=None, tuning_config=None):
         self.optimize_data = optimize_data
         self.outputs = outputs
+        self.tuning_config = tuning_config
 
     def _c(self):
         keep, opts = [], []
@@ -720,6 +742,10 @@ class build_options:  # noqa: N801
             arr = _ids(self.outputs, keep)
             keep.append(arr)
             opts.append(c_build_option(build_option_type.outputs, C.cast(C.pointer(arr), C.c_void_p)))
+        if self.tuning_config is not None:
+            t = c_tuning_config(self.tuning_config[0], (self.tuning_config[1] or "").encode())
+            keep.append(t)
+            opts.append(c_build_option(build_option_type.tuning_config, C.cast(C.pointer(t), C.c_void_p)))
         carr = (c_build_option * max(len(opts), 1))(*opts)
         return carr, len(opts), keep
 

@@ -350,6 +350,105 @@ cldnn_hip_status cldnn_hip_conv_enqueue(cldnn_hip_conv c, const void* input_dev,
     return guarded([&] { run(c, input_dev, output_dev, eltw_dev, nullptr); });
 }
 
+// One candidate of the tuner: microseconds per launch, or a negative value when the row refuses the convolution.
+static float time_candidate(cldnn_hip_engine e, cldnn_hip_conv_desc d, int tile_override, const void* weights, const void* bias,
+                            const float* wqf, const float* calib, const float* eltw_calib, const void* in, void* out,
+                            const void* eltw, int runs)
+{
+    d.tile_override = tile_override;
+    cldnn_hip_conv c = nullptr;
+    if (cldnn_hip_conv_create(e, &d, weights, bias, wqf, calib, eltw_calib, &c) != CLDNN_HIP_SUCCESS) return -1.0f;
+    if (tile_override && c->impl != CLDNN_HIP_IMPL_MFMA) {
+        cldnn_hip_conv_release(c);
+        return -1.0f;
+    }
+    float best = -1.0f;
+    hipEvent_t t0 = nullptr, t1 = nullptr;
+    try {
+        CHIP_CHECK(hipEventCreate(&t0));
+        CHIP_CHECK(hipEventCreate(&t1));
+        for (int i = 0; i < 3; ++i) run(c, in, out, eltw, nullptr);
+        for (int batch = 0; batch < 3; ++batch) {
+            CHIP_CHECK(hipEventRecord(t0, e->stream));
+            for (int i = 0; i < runs; ++i) run(c, in, out, eltw, nullptr);
+            CHIP_CHECK(hipEventRecord(t1, e->stream));
+            CHIP_CHECK(hipEventSynchronize(t1));
+            float ms = 0.0f;
+            CHIP_CHECK(hipEventElapsedTime(&ms, t0, t1));
+            const float us = ms * 1000.0f / (float)runs;
+            if (best < 0.0f || us < best) best = us;
+        }
+    } catch (...) {
+        if (t0) (void)hipEventDestroy(t0);
+        if (t1) (void)hipEventDestroy(t1);
+        cldnn_hip_conv_release(c);
+        throw;
+    }
+    (void)hipEventDestroy(t0);
+    (void)hipEventDestroy(t1);
+    cldnn_hip_conv_release(c);
+    return best;
+}
+
+cldnn_hip_status cldnn_hip_conv_tune(cldnn_hip_engine e, const cldnn_hip_conv_desc* desc, const void* weights, const void* bias,
+                                     const float* wqf, const float* calib, const float* eltw_calib, int32_t runs,
+                                     int32_t* best_tile_index, float* best_us, float* default_us, float* row_us)
+{
+    return guarded([&] {
+        CHIP_REQUIRE(e && desc && weights && best_tile_index && best_us, CLDNN_HIP_INVALID_ARG, "null argument");
+        CHIP_REQUIRE(runs >= 1 && runs <= 10000, CLDNN_HIP_INVALID_ARG, "tuning runs must be between 1 and 10000");
+        e->make_current();
+        const size_t in_bytes = tensor_elems(desc->input) * dtype_size(desc->input.dtype);
+        const size_t out_bytes = tensor_elems(desc->output) * dtype_size(desc->output.dtype);
+        const bool separate_eltw = desc->fused && !desc->second_input_in_output;
+        const size_t el_bytes = separate_eltw ? tensor_elems(desc->eltw) * dtype_size(desc->eltw.dtype) : 0;
+        void *in = nullptr, *out = nullptr, *eltw = nullptr;
+        auto release = [&] {
+            (void)hipStreamSynchronize(e->stream);
+            if (in) (void)hipFree(in);
+            if (out) (void)hipFree(out);
+            if (eltw) (void)hipFree(eltw);
+        };
+        try {
+            CHIP_CHECK(hipMalloc(&in, in_bytes ? in_bytes : 1));
+            CHIP_CHECK(hipMalloc(&out, out_bytes ? out_bytes : 1));
+            if (separate_eltw) CHIP_CHECK(hipMalloc(&eltw, el_bytes ? el_bytes : 1));
+            // pseudo-random bytes; a float tensor gets small integers so that no NaN patterns are timed
+            std::vector<uint8_t> host(std::max(in_bytes, el_bytes));
+            uint32_t state = 1337u;
+            for (auto& b : host) {
+                state = state * 1664525u + 1013904223u;
+                b = (uint8_t)(state >> 24);
+            }
+            if (desc->input.dtype == CLDNN_HIP_F32)
+                for (size_t i = 0; i + 4 <= in_bytes; i += 4) {
+                    const float v = (float)(int8_t)host[i];
+                    std::memcpy(&host[i], &v, 4);
+                }
+            CHIP_CHECK(hipMemcpy(in, host.data(), in_bytes, hipMemcpyHostToDevice));
+            if (separate_eltw) CHIP_CHECK(hipMemcpy(eltw, host.data(), el_bytes, hipMemcpyHostToDevice));
+            CHIP_CHECK(hipMemset(out, 0, out_bytes));
+            const float base = time_candidate(e, *desc, 0, weights, bias, wqf, calib, eltw_calib, in, out, eltw, runs);
+            CHIP_REQUIRE(base >= 0.0f, CLDNN_HIP_ERROR, std::string("the convolution cannot be created: ") + cldnn_hip_last_error());
+            *best_tile_index = -1, *best_us = base;
+            if (default_us) *default_us = base;
+            const int rows = cldnn_hip_tile_config_count();
+            for (int r = 0; r < rows; ++r) {
+                const float us = desc->impl == CLDNN_HIP_IMPL_AUTO || desc->impl == CLDNN_HIP_IMPL_MFMA
+                                     ? time_candidate(e, *desc, r + 1, weights, bias, wqf, calib, eltw_calib, in, out, eltw, runs)
+                                     : -1.0f;
+                if (row_us) row_us[r] = us;
+                // a row has to win by more than the noise of the measurement to replace the table's choice
+                if (us >= 0.0f && us < *best_us * 0.98f) *best_us = us, *best_tile_index = r;
+            }
+        } catch (...) {
+            release();
+            throw;
+        }
+        release();
+    });
+}
+
 cldnn_hip_status cldnn_hip_conv_accumulators(cldnn_hip_conv c, const void* input_dev, int32_t* acc_dev)
 {
     return guarded([&] {

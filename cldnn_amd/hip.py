@@ -154,6 +154,9 @@ SIGNATURES = {
     "cldnn_hip_eltwise": (C.c_int32, [C.c_void_p, C.POINTER(EltwiseDesc), C.POINTER(C.c_void_p), C.c_void_p, C.c_void_p]),
     "cldnn_hip_conv_create": (C.c_int32, [C.c_void_p, C.POINTER(ConvDesc), C.c_void_p, C.c_void_p, C.c_void_p,
                                           C.c_void_p, C.c_void_p, C.POINTER(C.c_void_p)]),
+    "cldnn_hip_conv_tune": (C.c_int32, [C.c_void_p, C.POINTER(ConvDesc), C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,
+                                        C.c_int32, C.POINTER(C.c_int32), C.POINTER(C.c_float), C.POINTER(C.c_float),
+                                        C.POINTER(C.c_float)]),
     "cldnn_hip_conv_release": (C.c_int32, [C.c_void_p]),
     "cldnn_hip_conv_enqueue": (C.c_int32, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p]),
     "cldnn_hip_conv_accumulators": (C.c_int32, [C.c_void_p, C.c_void_p, C.c_void_p]),
@@ -407,6 +410,18 @@ class Conv:
             self.close()
         except Exception:
             pass
+
+
+def conv_tune(engine, desc, w, bias=None, wqf=None, calib=None, eltw_calib=None, runs=20):
+    """cldnn_hip_conv_tune: -> (best row or -1, its microseconds, microseconds of the table's own choice, per-row list)"""
+    L = lib()
+    keep = [np.ascontiguousarray(w)] + [None if a is None else np.ascontiguousarray(a) for a in (bias, wqf, calib, eltw_calib)]
+    ptr = [None if a is None else a.ctypes.data_as(C.c_void_p) for a in keep]
+    best, best_us, default_us = C.c_int32(-1), C.c_float(0), C.c_float(0)
+    rows = (C.c_float * L.cldnn_hip_tile_config_count())()
+    check(L.cldnn_hip_conv_tune(engine.h, C.byref(desc), ptr[0], ptr[1], ptr[2], ptr[3], ptr[4], runs, C.byref(best), C.byref(best_us),
+                                C.byref(default_us), rows))
+    return best.value, best_us.value, default_us.value, list(rows)
 
 
 def conv_desc(x_t, w_shape, out_dt, *, stride=(1, 1), pad=(0, 0), dilation=(1, 1), groups=1, out_fmt=None,

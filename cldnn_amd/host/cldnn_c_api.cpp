@@ -480,6 +480,7 @@ cldnn_engine cldnn_create_engine(int32_t type, uint32_t engine_num, const cldnn_
         }
         ref<cldnn_engine_impl> e(new cldnn_engine_impl(), false);
         e->profiling = cfg && cfg->enable_profiling;
+        if (cfg && cfg->tuning_cache_path && cfg->tuning_cache_path[0]) e->tuning_cache_path = cfg->tuning_cache_path;
         e->memory_pool = !cfg || cfg->enable_memory_pool;
         hip_check(cldnn_hip_engine_create(engine_num, e->profiling ? 1 : 0, &e->h));
         e->retain();
@@ -600,7 +601,21 @@ static cldnn_program build(cldnn_engine engine, cldnn_topology topology, cldnn_b
         case cldnn_build_option_outputs:
             if (options[i].data) outputs = ids_of(*reinterpret_cast<const cldnn_primitive_id_arr*>(options[i].data));
             break;
-        default: break;  // fusing, debug, tuning_config, graph_dumps_dir, learning_config: accepted, no effect here
+        case cldnn_build_option_tuning_config:
+            if (options[i].data) {
+                auto* t = reinterpret_cast<const cldnn_tuning_config*>(options[i].data);
+                HOST_REQUIRE(t->mode >= cldnn_tuning_disabled && t->mode <= cldnn_tuning_tune_and_cache, CLDNN_INVALID_ARG, "unknown tuning mode");
+                if (t->mode != cldnn_tuning_disabled) {
+                    // reference src/program.cpp:305-309
+                    HOST_REQUIRE(t->mode != cldnn_tuning_tune_and_cache || !engine || engine->profiling, CLDNN_INVALID_ARG,
+                                 "Engine must be created with profiling enabled in tune_and_cache mode!");
+                    std::string path = t->cache_file_path ? t->cache_file_path : "";
+                    if (path.empty()) path = engine ? engine->tuning_cache_path : "cache.json";
+                    prog->tuning.load(path, t->mode);  // planning without an engine still reads (and so validates) the file
+                }
+            }
+            break;
+        default: break;  // fusing, debug, graph_dumps_dir, learning_config: accepted, no effect here
         }
     }
     build_program(prog.get(), topology, outputs);

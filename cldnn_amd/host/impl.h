@@ -64,11 +64,25 @@ struct ref {  // owning smart pointer for refcounted objects
 
 enum class prim_type { input_layout, data, reorder, activation, eltwise, convolution, fused_conv_eltwise, pooling };
 
+// which row of the tile-config table a convolution runs on, measured once and kept in a JSON file (tuning_cache.cpp)
+struct tuning_cache {
+    std::string path;
+    int mode = cldnn_tuning_disabled;
+    std::map<std::string, std::map<std::string, std::pair<std::string, int>>> entries;  // compute units -> signature -> (row name, row)
+    bool dirty = false;
+    void load(const std::string& file, int tuning_mode);
+    bool find(uint32_t compute_units, const std::string& key, std::string* name, int* index) const;
+    void store(uint32_t compute_units, const std::string& key, const std::string& name, int index);
+    void save();
+};
+std::string conv_signature(const cldnn_hip_conv_desc& d);
+
 }  // namespace host
 
 struct cldnn_engine_impl : host::refcounted {
     cldnn_hip_engine h = nullptr;
     bool profiling = false;
+    std::string tuning_cache_path = "cache.json";  // engine configuration; a tuning_config without a path of its own uses it
     bool memory_pool = true;  // networks share buffers between intermediate tensors whose lifetimes do not overlap
     ~cldnn_engine_impl() override;
 };
@@ -167,6 +181,8 @@ struct cldnn_program_impl : host::refcounted {
     std::vector<std::unique_ptr<host::node>> nodes;  // execution order
     std::map<std::string, host::node*> by_id;
     bool optimize_data = false;
+    host::tuning_cache tuning;       // build option tuning_config
+    size_t tuned_now = 0, tuned_from_cache = 0;
     std::vector<std::string> all_org_ids;
     ~cldnn_program_impl() override;
 };

@@ -828,6 +828,29 @@ static void compile_conv(cldnn_program_impl* prog, node* n)
         }
     }
     d.impl = CLDNN_HIP_IMPL_AUTO;
+    const void* bias_ptr = bv.empty() ? nullptr : bv.data();
+    const float* wqf_ptr = qv.empty() ? nullptr : (const float*)qv.data();
+    const float* calib_ptr = cv.empty() ? nullptr : (const float*)cv.data();
+    if (prog->tuning.mode != cldnn_tuning_disabled) {
+        // reference src/gpu/convolution_gpu.cpp:147-154, kernel_selector/core/kernel_selector.cpp GetAutoTuneBestKernel: take
+        // the cached choice; in tune_and_cache mode measure what the cache does not hold and add it
+        cldnn_hip_engine_info info{};
+        hip_check(cldnn_hip_engine_get_info(prog->engine->h, &info));
+        const std::string key = conv_signature(d);
+        std::string name;
+        int row = -1;
+        if (prog->tuning.find(info.cores_count, key, &name, &row)) {
+            if (row >= 0 && row < cldnn_hip_tile_config_count() && name == cldnn_hip_tile_config_name(row)) d.tile_override = row + 1;
+            ++prog->tuned_from_cache;
+        } else if (prog->tuning.mode == cldnn_tuning_tune_and_cache) {
+            float best_us = 0.0f;
+            hip_check(cldnn_hip_conv_tune(prog->engine->h, &d, wv.data(), bias_ptr, wqf_ptr, calib_ptr, (const float*)eltw_calib, 20, &row,
+                                          &best_us, nullptr, nullptr));
+            prog->tuning.store(info.cores_count, key, row >= 0 ? cldnn_hip_tile_config_name(row) : "table", row);
+            if (row >= 0) d.tile_override = row + 1;
+            ++prog->tuned_now;
+        }
+    }
     hip_check(cldnn_hip_conv_create(prog->engine->h, &d, wv.data(), bv.empty() ? nullptr : bv.data(),
                                     qv.empty() ? nullptr : (const float*)qv.data(), cv.empty() ? nullptr : (const float*)cv.data(),
                                     (const float*)eltw_calib, &n->conv));
@@ -891,6 +914,7 @@ void build_program(cldnn_program_impl* prog, cldnn_topology_impl* topo, const st
         node* n = u.get();
         if (n->p->type == prim_type::convolution || n->p->type == prim_type::fused_conv_eltwise) compile_conv(prog, n);
     }
+    prog->tuning.save();
 }
 
 // ------------------------------------------------------------------------------------------ inspection

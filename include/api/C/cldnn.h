@@ -70,7 +70,7 @@ typedef struct {
     int16_t throttle_mode;
     uint32_t enable_memory_pool;       /* networks reuse buffers between intermediate tensors of identical layout */
     void* context;                     /* must be NULL */
-    const char* tuning_cache_path;     /* accepted, no effect: the tile table is built in */
+    const char* tuning_cache_path;     /* tuning cache file of a tuning_config that names none (default "cache.json") */
 } cldnn_engine_configuration;
 
 typedef struct {

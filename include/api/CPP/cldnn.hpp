@@ -952,10 +952,26 @@ enum class build_option_type : int32_t {
     learning_config = cldnn_build_option_learning_config
 };
 
+// reference api/CPP/program.hpp:68-93
+enum class tuning_mode : int32_t {
+    tuning_disabled = cldnn_tuning_disabled,
+    tuning_use_cache = cldnn_tuning_use_cache,
+    tuning_tune_and_cache = cldnn_tuning_tune_and_cache
+};
+struct tuning_config_options {
+    tuning_mode mode = tuning_mode::tuning_disabled;
+    std::string cache_file_path;
+};
+
 struct build_option {
     build_option_type type;
     bool enabled = true;
     std::vector<primitive_id> ids;
+    tuning_config_options tuning;
+    static build_option tuning_config(const tuning_config_options& config = tuning_config_options())
+    {
+        return {build_option_type::tuning_config, true, {}, config};
+    }
     static build_option fusing(bool enable = false) { return {build_option_type::fusing, enable, {}}; }
     static build_option optimize_data(bool enable = false) { return {build_option_type::optimize_data, enable, {}}; }
     static build_option debug(bool enable = false) { return {build_option_type::debug, enable, {}}; }
@@ -984,15 +1000,20 @@ struct build_options {
         std::vector<cldnn_build_option> opts;
         std::vector<std::vector<const char*>> ptrs;
         std::vector<cldnn_primitive_id_arr> arrs;
+        std::vector<cldnn_tuning_config> tuning;
     };
     std::unique_ptr<c_view> get_refs() const
     {
         std::unique_ptr<c_view> v(new c_view());
         v->ptrs.reserve(_opts.size());
         v->arrs.reserve(_opts.size());
+        v->tuning.reserve(_opts.size());
         for (auto& o : _opts) {
             if (!o.enabled) continue;
-            if (o.type == build_option_type::outputs) {
+            if (o.type == build_option_type::tuning_config) {
+                v->tuning.push_back(cldnn_tuning_config{(int32_t)o.tuning.mode, o.tuning.cache_file_path.c_str()});
+                v->opts.push_back(cldnn_build_option{(int32_t)o.type, &v->tuning.back()});
+            } else if (o.type == build_option_type::outputs) {
                 v->ptrs.emplace_back();
                 for (auto& s : o.ids) v->ptrs.back().push_back(s.c_str());
                 v->arrs.push_back(cldnn_primitive_id_arr{v->ptrs.back().data(), v->ptrs.back().size()});

@@ -306,6 +306,19 @@ cldnn_hip_status cldnn_hip_conv_get_info(cldnn_hip_conv c, cldnn_hip_conv_info* 
 /* computed output extent along one axis (reference src/include/sliding_window_utils.h:90-129) */
 int32_t cldnn_hip_conv_out_extent(int32_t in, int32_t pad, int32_t filt, int32_t dil, int32_t stride);
 
+/* Kernel runner for tuning: times the table's own choice and every row of the tile-config table that accepts this
+ * convolution, on scratch tensors of the descriptor's shapes filled with pseudo-random bytes, and reports the fastest.
+ * Replaces the reference's kernel_runner (src/gpu/kernel_runner.cpp:106-190, used by tuning_mode tune_and_cache through
+ * kernel_selector/core/kernel_selector.cpp GetAutoTuneBestKernel): each candidate is created, warmed up and run
+ * `runs` times back to back on the engine's stream between two events; the best of three such batches counts.
+ * best_tile_index = -1 when the table's own choice is the fastest (or no row applies: depthwise, plain layouts).
+ * row_us (may be NULL) receives cldnn_hip_tile_config_count() entries, negative where a row does not apply.
+ * Blocks until done; allocates and frees its scratch tensors. */
+cldnn_hip_status cldnn_hip_conv_tune(cldnn_hip_engine e, const cldnn_hip_conv_desc* desc, const void* weights,
+                                     const void* bias, const float* wqf, const float* calib, const float* eltw_calib,
+                                     int32_t runs, int32_t* best_tile_index, float* best_us, float* default_us,
+                                     float* row_us);
+
 /* number of rows of the gfx950 tile-config table and a printable description of one row */
 int32_t cldnn_hip_tile_config_count(void);
 const char* cldnn_hip_tile_config_name(int32_t index);

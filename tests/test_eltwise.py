@@ -217,3 +217,66 @@ def test_api_argument_checks():
     with pytest.raises(cl.error, match="at most 4 inputs"):
         build(f, ["a", "b", "a", "b", "a"], cl.eltwise_mode.sum)
     assert build(f, ["a", "b", "a", "b"], cl.eltwise_mode.sum) is not None
+
+
+def _ramp(shape, add=0):
+    """the reference's test data: element i of the bfyx buffer is (char)(i + add)"""
+    n = int(np.prod(shape))
+    return ((np.arange(n, dtype=np.int64) + add) & 255).astype(np.uint8).view(np.int8).reshape(shape)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("b,f,size", [(1, 256, 56), (4, 512, 28), (16, 1024, 14), (32, 2048, 14)])
+def test_api_b_fs_yx_fsv4_with_calibration(b, f, size):
+    """reference tests/test_cases/eltwise_gpu_test.cpp:1833-1971: the quantized sum with per-feature calibration (every
+    seventh factor negative) in bfyx and through b_fs_yx_fsv4 reorders; both must equal the oracle"""
+    from cldnn_amd import api as cl
+    eng = cl.engine()
+    x = _ramp((b, f, size, size))
+    cal, sign = np.empty(f, np.float32), np.float32(1)
+    for i in range(f):
+        cal[i] = sign if (i + 1) % 7 else -sign
+        sign = np.float32(sign * np.float32(1.0123))
+    exp = rc.eltwise([x, x], "sum", calib=cal, relu=True)
+    assert 0.2 < (exp > 0).mean() < 0.6 and (exp == 127).any()
+    lay = cl.layout(cl.data_types.i8, cl.format.bfyx, cl.tensor(b, f, size, size))
+    blocked = cl.layout(cl.data_types.i8, cl.format.b_fs_yx_fsv4, cl.tensor(b, f, size, size))
+    common = [cl.input_layout("input1", lay), cl.input_layout("input2", lay),
+              cl.data("callib", cl.make_memory(eng, cal.reshape(1, 1, 1, -1)))]
+    gold = cl.topology(*common, cl.eltwise("eltw_GOLD", "input1", "input2", cl.eltwise_mode.sum, True, output_calibration_factors="callib"))
+    imad = cl.topology(*common, cl.reorder("reorder1_Swizzelled", "input1", blocked), cl.reorder("reorder2_Swizzelled", "input2", blocked),
+                       cl.eltwise("eltw_IMAD", "reorder1_Swizzelled", "reorder2_Swizzelled", cl.eltwise_mode.sum, True,
+                                  output_calibration_factors="callib"),
+                       cl.reorder("reorder_UnSwizzelled", "eltw_IMAD", lay))
+    m = cl.make_memory(eng, x)
+    for topo, out in ((gold, "eltw_GOLD"), (imad, "reorder_UnSwizzelled")):
+        net = cl.network(eng, topo, cl.build_options())
+        net.set_input_data("input1", m)
+        net.set_input_data("input2", m)
+        got = net.execute()[out].get_memory().read()
+        assert np.array_equal(got, exp), out
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("mode", ["min", "max", "sum"])
+def test_api_b_fs_yx_fsv4_three_inputs(mode):
+    """reference tests/test_cases/eltwise_gpu_test.cpp:1973-2119: three int8 inputs, no calibration (8-bit wrap-around)"""
+    from cldnn_amd import api as cl
+    eng = cl.engine()
+    shape = (1, 256, 56, 56)
+    ins = [_ramp(shape, k) for k in (1, 2, 3)]
+    exp = rc.eltwise(ins, mode, relu=True)
+    lay = cl.layout(cl.data_types.i8, cl.format.bfyx, cl.tensor(1, 256, 56, 56))
+    blocked = cl.layout(cl.data_types.i8, cl.format.b_fs_yx_fsv4, cl.tensor(1, 256, 56, 56))
+    names = ["input1", "input2", "input3"]
+    common = [cl.input_layout(n, lay) for n in names]
+    gold = cl.topology(*common, cl.eltwise("eltw_GOLD", names, getattr(cl.eltwise_mode, mode), True))
+    imad = cl.topology(*common, *[cl.reorder("r" + n, n, blocked) for n in names],
+                       cl.eltwise("eltw_IMAD", ["r" + n for n in names], getattr(cl.eltwise_mode, mode), True),
+                       cl.reorder("reorder_UnSwizzelled", "eltw_IMAD", lay))
+    for topo, out in ((gold, "eltw_GOLD"), (imad, "reorder_UnSwizzelled")):
+        net = cl.network(eng, topo, cl.build_options())
+        for n, a in zip(names, ins):
+            net.set_input_data(n, cl.make_memory(eng, a))
+        got = net.execute()[out].get_memory().read()
+        assert np.array_equal(got, exp), out
