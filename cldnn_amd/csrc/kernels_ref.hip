@@ -362,6 +362,39 @@ __global__ void __launch_bounds__(256) reorder_to_blocked_kernel(ReorderArgs a, 
     else *reinterpret_cast<uint4*>(o) = make_uint4(w[0], w[1], w[2], w[3]);
 }
 
+// The same for FSV = 4 when rows are whole dwords (X % 4 == 0, 4-byte aligned planes): one lane = 4 consecutive pixels
+// of a row: one dword load per feature plane, a 4x4 byte transpose in registers, one 16-byte store.
+template <bool ALIGNED16>
+__global__ void __launch_bounds__(256) reorder_to_fsv4_x4_kernel(ReorderArgs a, const uint8_t* __restrict__ src, uint8_t* __restrict__ dst)
+{
+    const int slices = (a.F + 3) / 4, xq = a.X / 4;
+    const unsigned total = (unsigned)slices * a.B * a.Y * xq;
+    const unsigned idx = blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= total) return;
+    const int x = (int)(idx % xq) * 4;
+    unsigned r = idx / xq;
+    const int y = (int)(r % a.Y);
+    r /= a.Y;
+    const int fs = (int)(r % slices), b = (int)(r / slices);
+    const int64_t s0 = a.src.at(b, fs * 4, y, x);
+    unsigned p[4] = {0, 0, 0, 0};
+#pragma unroll
+    for (int c = 0; c < 4; ++c)
+        if (fs * 4 + c < a.F) p[c] = *reinterpret_cast<const unsigned*>(src + s0 + (int64_t)c * a.src.pf);
+    unsigned w[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)  // pixel i: byte i of every plane
+        w[i] = ((p[0] >> (8 * i)) & 255u) | (((p[1] >> (8 * i)) & 255u) << 8) | (((p[2] >> (8 * i)) & 255u) << 16)
+               | (((p[3] >> (8 * i)) & 255u) << 24);
+    uint8_t* o = dst + a.dst.at(b, fs * 4, y, x);
+    if constexpr (ALIGNED16) {
+        *reinterpret_cast<uint4*>(o) = make_uint4(w[0], w[1], w[2], w[3]);
+    } else {  // a left border whose width is not a multiple of 4 pixels
+#pragma unroll
+        for (int i = 0; i < 4; ++i) reinterpret_cast<unsigned*>(o)[i] = w[i];
+    }
+}
+
 void launch_reorder(hipStream_t s, const cldnn_hip_tensor& st, const void* src, const cldnn_hip_tensor& dt, void* dst)
 {
     CHIP_REQUIRE(st.b == dt.b && st.f == dt.f && st.y == dt.y && st.x == dt.x, CLDNN_HIP_DIMENSION_MISMATCH,
@@ -375,7 +408,16 @@ void launch_reorder(hipStream_t s, const cldnn_hip_tensor& st, const void* src, 
         const int64_t work = (int64_t)((a.F + a.dst.fsv - 1) / a.dst.fsv) * a.B * a.Y * a.X;
         const int64_t nb = (work + 255) / 256;
         CHIP_REQUIRE(nb < (1ll << 31), CLDNN_HIP_UNSUPPORTED_SIZE, "tensor too large for the reorder grid");
-        if (a.dst.fsv == 4)
+        // dword path: every row of every plane starts on a 4-byte boundary on both sides
+        const bool dwords = a.dst.fsv == 4 && a.X % 4 == 0 && a.src.px == 1 && a.src.off % 4 == 0 && a.src.py % 4 == 0 && a.src.pf % 4 == 0
+                            && a.src.pb % 4 == 0 && (uintptr_t)src % 4 == 0 && (uintptr_t)dst % 4 == 0 && work / 4 < (1ll << 31);
+        const bool aligned16 = a.dst.off % 16 == 0 && a.dst.py % 16 == 0 && a.dst.pf % 16 == 0 && a.dst.pb % 16 == 0 && (uintptr_t)dst % 16 == 0;
+        const dim3 grid4((unsigned)((work / 4 + 255) / 256));
+        if (dwords && aligned16)
+            hipLaunchKernelGGL(reorder_to_fsv4_x4_kernel<true>, grid4, dim3(256), 0, s, a, (const uint8_t*)src, (uint8_t*)dst);
+        else if (dwords)
+            hipLaunchKernelGGL(reorder_to_fsv4_x4_kernel<false>, grid4, dim3(256), 0, s, a, (const uint8_t*)src, (uint8_t*)dst);
+        else if (a.dst.fsv == 4)
             hipLaunchKernelGGL(reorder_to_blocked_kernel<4>, dim3((unsigned)nb), dim3(256), 0, s, a, (const uint8_t*)src, (uint8_t*)dst);
         else
             hipLaunchKernelGGL(reorder_to_blocked_kernel<16>, dim3((unsigned)nb), dim3(256), 0, s, a, (const uint8_t*)src, (uint8_t*)dst);

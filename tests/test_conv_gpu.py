@@ -420,6 +420,26 @@ def test_reorder_round_trip_and_layout_independence(eng, fmt):
     np.testing.assert_array_equal(a, b_)
 
 
+@pytest.mark.parametrize("shape", [(2, 3, 6, 8), (1, 4, 5, 12), (2, 7, 3, 16), (1, 3, 4, 6)], ids=lambda s: "x".join(map(str, s)))
+@pytest.mark.parametrize("pad", [(0, 0), (3, 3), (1, 4)], ids=lambda p: "pad%dx%d" % p)
+@pytest.mark.parametrize("fmt", ["b_fs_yx_fsv4", "fs_b_yx_fsv16"])
+def test_reorder_into_blocked_layouts(eng, shape, pad, fmt):
+    """the byte paths of the reorder (row widths that are and are not whole dwords, borders that do and do not keep the
+    16-byte alignment): every element where the layout formula says, feature padding zero, borders untouched"""
+    import ctypes as C
+    r = np.random.default_rng(21)
+    x = r.integers(1, 256, shape).astype(np.uint8)
+    buf = hip.upload(eng, x, fmt, pad)
+    np.testing.assert_array_equal(hip.download(eng, buf), x)
+    raw = buf.read_raw()
+    L = hip.lib()
+    expect = np.zeros_like(raw)
+    for idx in np.ndindex(*shape):
+        expect[L.cldnn_hip_tensor_offset(C.byref(buf.tensor), *[int(i) for i in idx])] = x[idx]
+    np.testing.assert_array_equal(raw, expect)
+    buf.close()
+
+
 def test_reorder_f32_to_int8_goes_towards_zero_and_saturates(eng):
     """the reference's reorder converts with convert_char (jitter.cpp:483): towards zero; its pooling test relies on
     9.5 -> 9 (pooling_gpu_test.cpp:264-309).  Out-of-range values saturate here."""
