@@ -210,9 +210,10 @@ void build(cldnn_hip_conv c, const void* weights, const void* bias, const float*
     // can the short epilogue reproduce the long one?  (an int32 bias is folded into the start values, a float one is not)
     {
         Epilogue probe = e;
-        probe.bias = bias && d.bias_dtype == CLDNN_HIP_F32 ? (const void*)weights : nullptr;
+        probe.bias = bias && (d.bias_dtype == CLDNN_HIP_F32 || e.fc) ? (const void*)weights : nullptr;
         c->fast = mfma_fast_epilogue(p, probe, calib_on ? calib : nullptr, eltw_calib, wqf, &c->fe);
     }
+    if (impl == CLDNN_HIP_IMPL_DEPTHWISE && e.fc) c->fast = false;  // the depthwise kernels have no short fully_connected form
     const bool dw_fast = impl == CLDNN_HIP_IMPL_DEPTHWISE && dw_fast_applies(p, c->fast);
     const bool xor_u8 = (impl == CLDNN_HIP_IMPL_MFMA || dw_fast) && p.in_dt == CLDNN_HIP_U8;
     for (int f = 0; f < p.OFM; ++f) {
@@ -221,12 +222,13 @@ void build(cldnn_hip_conv c, const void* weights, const void* bias, const float*
             for (size_t i = 0; i < (size_t)ifm_g * p.FY * p.FX; ++i) s += w8[(size_t)f * ifm_g * p.FY * p.FX + i];
         uint32_t v = (uint32_t)(int32_t)(128 * s);
         init_raw[f] = impl == CLDNN_HIP_IMPL_MFMA ? (int32_t)v : 0;  // the accumulator probe of the depthwise path never flips signs
-        if (bias && d.bias_dtype == CLDNN_HIP_I32 && !e.bias_after) v += (uint32_t)((const int32_t*)bias)[f];
+        // (the fully_connected form adds its bias as a float after the dequantisation, whatever its type)
+        if (bias && d.bias_dtype == CLDNN_HIP_I32 && !e.bias_after && !e.fc) v += (uint32_t)((const int32_t*)bias)[f];
         init[f] = (int32_t)v;
     }
     c->acc_init = upload(c, init.data(), ofm_pad * 4);
     c->acc_init_raw = upload(c, init_raw.data(), ofm_pad * 4);
-    if (bias && d.bias_dtype == CLDNN_HIP_F32) {
+    if (bias && (d.bias_dtype == CLDNN_HIP_F32 || e.fc)) {
         c->bias = upload(c, bias, p.OFM * 4, ofm_pad * 4);
         e.bias = c->bias;
     } else {

@@ -317,8 +317,15 @@ bool mfma_fast_epilogue(const ConvProblem& p, const Epilogue& e, const float* ca
                         FastEpi* out)
 {
     FastEpi F{};
-    if (e.mode != MODE_Q || e.round_even || e.fc) return false;
-    if (e.bias) return false;  // an int32 bias is folded into the accumulator start; a float bias takes the long path
+    if (e.mode != MODE_Q || e.round_even) return false;
+    if (e.fc) {
+        // the fully_connected form has a short version for a float bias and no / relu activation
+        if (!e.bias || e.bias_dt != CLDNN_HIP_F32 || e.fused || e.out_dt != CLDNN_HIP_S8) return false;
+        if (!(e.act == CLDNN_HIP_ACT_NONE || e.act == CLDNN_HIP_ACT_RELU)) return false;
+        F.fc = 1;
+    } else if (e.bias) {
+        return false;  // an int32 bias is folded into the accumulator start; a float bias takes the long path
+    }
     if (!(e.out_dt == CLDNN_HIP_S8 || e.out_dt == CLDNN_HIP_U8)) return false;
     if (!(e.act == CLDNN_HIP_ACT_NONE || e.act == CLDNN_HIP_ACT_RELU || e.act == CLDNN_HIP_ACT_CLAMP)) return false;
     if (e.act == CLDNN_HIP_ACT_CLAMP && !(e.act_m <= e.act_n)) return false;  // the median form needs ordered bounds
@@ -419,7 +426,7 @@ void launch_conv_mfma(hipStream_t s, const ConvProblem& p, const MfmaPlan& pl, c
         a.fe = *fast;
         kind = EPI_KIND_FAST;
         // the branch-free forms
-        if (!fast->has_wqf && epi.calib) {
+        if (!fast->has_wqf && epi.calib && !fast->fc) {
             if (!fast->fused && fast->relu_folded) kind = EPI_KIND_RELU;
             if (!fast->fused && fast->act == CLDNN_HIP_ACT_NONE) kind = EPI_KIND_LINEAR;
             if (fast->fused && fast->act == CLDNN_HIP_ACT_NONE && fast->eltw_relu_folded && epi.eltw_calib) kind = EPI_KIND_FUSED;

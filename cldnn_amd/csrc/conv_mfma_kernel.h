@@ -253,7 +253,24 @@ __device__ __forceinline__ v4i epilogue_fast16(const Args& a, const v4i (&acc)[4
     }
     v4i packed;
     bool finished = false;
-    if (F.relu_folded) {
+    if (F.fc) {
+        // reference fully_connected_gpu_bfyx_ref.cl:63-84: (char)round((acc * wqf * iqf + bias) * factor), then the
+        // activation on the char; ecal[] holds the bias
+#pragma unroll
+        for (int d = 0; d < 4; ++d) {
+            unsigned word = 0;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int c = d * 4 + i;
+                float x = v[c] + ecal[c];
+                x = x * cal[c];
+                int q = (int)(signed char)(int)rha(x);
+                if (F.act == CLDNN_HIP_ACT_RELU) q = q > 0 ? q : 0;
+                word |= ((unsigned)q & 255u) << (8 * i);
+            }
+            packed[d] = (int)word;
+        }
+    } else if (F.relu_folded) {
 #pragma unroll
         for (int c = 0; c < 16; ++c) v[c] = med3(v[c] * cal[c], 0.0f, F.hi) + 0.49999997f;
 #pragma unroll
@@ -347,6 +364,7 @@ __device__ __forceinline__ void load_scales(const Args& a, int f0, LaneScales& s
             else if (e.oqf_on) c4 = make_float4(e.oqf, e.oqf, e.oqf, e.oqf);
             if (a.fe.has_wqf) w4 = *reinterpret_cast<const float4*>(e.wqf + f0 + d * 4);
             if (a.fe.has_ecal) e4 = *reinterpret_cast<const float4*>(e.eltw_calib + f0 + d * 4);
+            if (a.fe.fc) e4 = *reinterpret_cast<const float4*>((const float*)e.bias + f0 + d * 4);  // never fused: the slot is free
             sc.cal[d * 4 + 0] = c4.x, sc.cal[d * 4 + 1] = c4.y, sc.cal[d * 4 + 2] = c4.z, sc.cal[d * 4 + 3] = c4.w;
             sc.wq[d * 4 + 0] = w4.x, sc.wq[d * 4 + 1] = w4.y, sc.wq[d * 4 + 2] = w4.z, sc.wq[d * 4 + 3] = w4.w;
             sc.ecal[d * 4 + 0] = e4.x, sc.ecal[d * 4 + 1] = e4.y, sc.ecal[d * 4 + 2] = e4.z, sc.ecal[d * 4 + 3] = e4.w;

@@ -82,6 +82,7 @@ struct FastEpi {
     int32_t eltw_u8;
     float lo, hi;         // saturation bounds of the output type
     float iqf;
+    int32_t fc;           // the fully_connected form: float bias after the dequantisation, conversion to char keeps the low byte
 };
 // true (and *out filled) when the short epilogue reproduces the long one bit for bit
 bool mfma_fast_epilogue(const ConvProblem& p, const Epilogue& e, const float* calib, const float* ecal, const float* wqf,

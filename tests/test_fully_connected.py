@@ -147,6 +147,33 @@ def test_gpu_quantized_matches_oracle(eng, fmt, kw):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("act", ["relu", "none"])
+@pytest.mark.parametrize("bias_dt", [np.float32, np.int32], ids=["f32_bias", "i32_bias"])
+@pytest.mark.parametrize("shape", [dict(F=2048, H=1, W=1, OFM=1000, B=32), dict(F=64, H=3, W=3, OFM=70, B=5), dict(F=128, H=1, W=1, OFM=64, B=2)],
+                         ids=["resnet_fc1000_b32", "3x3_plane", "small"])
+def test_gpu_quantized_blocked_kernels(eng, shape, bias_dt, act):
+    """every matrix-core kernel family that takes the shape, short and long epilogue (a float bias takes the short
+    form, an int32 bias the long one; both add the bias as a float after the dequantisation)"""
+    from cldnn_amd import hip
+    x, w, b, q, c = quantized_problem(10, **shape)
+    b = (b * 3).astype(bias_dt)
+    ref = rc.fully_connected(x, w, b, wqf=q, calib=c, iqf=0.5, act=act)
+    assert len(np.unique(ref)) > 30 and (act == "none") == bool((ref < 0).any())
+    L = hip.lib()
+    seen = set()
+    for tile in range(0, L.cldnn_hip_tile_config_count() + 1):
+        try:
+            out, info = hip.conv_forward(eng, x, w, b, q, c, fmt="fs_b_yx_fsv16", fc=True, iqf=0.5, act=act, tile=tile, want_info=True)
+        except hip.HipError:
+            continue  # a row that does not take this shape refuses it
+        name = info.kernel_name.decode()
+        assert ("fast" in name) == (bias_dt == np.float32), name
+        seen.add(name.split("<")[0])
+        np.testing.assert_array_equal(out, ref, err_msg=name)
+    assert len(seen) >= 2, seen
+
+
+@pytest.mark.gpu
 def test_api_known_answers_and_quantized_network():
     from cldnn_amd import api as cl
     e = cl.engine()
