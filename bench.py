@@ -171,36 +171,52 @@ def copy_calibration(args):
 
 
 def network_workload(args):
-    """The whole quantized ResNet-50 topology (53 convolutions, 2 poolings, 16 residual sums, fully_connected) built and run
-    through the clDNN API with optimize_data: what an application sees per network.execute(), input already on the device."""
-    from cldnn_amd import api as cl, resnet50_net as rn
+    """A whole quantized network built and run through the clDNN API with optimize_data: what an application sees per
+    network.execute(), input already on the device.  resnet50_b32_network: 53 convolutions, 2 poolings, 16 residual sums,
+    fully_connected; mobilenet_v2_b32_network: 52 convolutions (17 depthwise), 35 clamps, 10 residual sums, pooling,
+    fully_connected."""
+    from cldnn_amd import api as cl
     batch = 32
     eng = cl.engine()
     r = np.random.default_rng(1337)
-    params = rn.random_weights()
-    IN_RMS, ECAL = 35.0, 1.0  # keep the signal alive through 16 blocks without a calibration pass
-    for l in workloads.resnet50():  # factors by rule (no calibration pass: timing does not depend on the values)
-        k = l["ifm"] * l["k"] ** 2
-        params[l["name"]]["calib"] = (32.0 / (np.sqrt(k) * IN_RMS * 73.3) * r.uniform(0.7, 1.4, l["ofm"])).astype(np.float32)
-    for step in rn.layer_plan():
+    resnet = args.workload.startswith("resnet50")
+    if resnet:
+        from cldnn_amd import resnet50_net as net_def
+        layers, classes_in = workloads.resnet50(), 2048
+        primitives = "53 convolution, 2 pooling, 16 eltwise (fused), 1 fully_connected"
+    else:
+        from cldnn_amd import mobilenet_v2_net as net_def
+        layers, classes_in = workloads.mobilenet_v2(), 1280
+        primitives = "52 convolution (17 depthwise), 35 activation clamp (folded), 10 eltwise, 1 pooling, 1 fully_connected"
+    params = net_def.random_weights()
+    IN_RMS, ECAL = 35.0, 1.0  # keep the signal alive through the blocks without a calibration pass
+    for l in layers:  # factors by rule (no calibration pass: timing does not depend on the values)
+        k = (l["ifm"] // l["groups"]) * l["k"] ** 2
+        q = params[l["name"]]
+        if l["act"] == "relu6":  # the clamp acts on the dequantised value: scale it into range, requantise with 127 / 6
+            q["wqf"] = (3.0 / (np.sqrt(k) * IN_RMS * 73.3) * r.uniform(0.7, 1.4, l["ofm"])).astype(np.float32)
+            q["calib"] = np.full(l["ofm"], 127.0 / 6.0, np.float32)
+        else:
+            q.setdefault("wqf", np.ones(l["ofm"], np.float32))
+            q["calib"] = (32.0 / (np.sqrt(k) * IN_RMS * 73.3) * r.uniform(0.7, 1.4, l["ofm"])).astype(np.float32)
+    for step in net_def.layer_plan():
         if step[0] == "sum":
-            params[step[1]] = dict(ecal=np.full(params[step[3]]["w"].shape[0], ECAL, np.float32))
-    params["fc1000"]["calib"] = np.full(1000, 40.0 / (np.sqrt(2048) * 30.0 * 73.3), np.float32)
+            params[step[1]] = dict(ecal=np.full(params[step[3]]["w"].shape[0], ECAL if resnet else 0.75, np.float32))
+    params["fc1000"]["calib"] = np.full(1000, 40.0 / (np.sqrt(classes_in) * 30.0 * 73.3), np.float32)
     t0 = time.perf_counter()
-    topo, opts = rn.topology(cl, eng, params, batch), cl.build_options(optimize_data=True)
+    topo, opts = net_def.topology(cl, eng, params, batch), cl.build_options(optimize_data=True)
     if args.tuning_cache:
         # measure what the cache file does not hold yet (needs an engine with profiling), then run from the file
         tuner = cl.engine(enable_profiling=True)
         t0 = time.perf_counter()
-        cl.network(tuner, rn.topology(cl, tuner, params, batch),
+        cl.network(tuner, net_def.topology(cl, tuner, params, batch),
                    cl.build_options(optimize_data=True, tuning_config=(cl.tuning_mode.tuning_tune_and_cache, args.tuning_cache)))
         log("tuning pass over %s: %.1f s" % (args.tuning_cache, time.perf_counter() - t0))
         opts = cl.build_options(optimize_data=True, tuning_config=(cl.tuning_mode.tuning_use_cache, args.tuning_cache))
     net = cl.network(eng, topo, opts)
     x = r.integers(0, 256, (batch, 3, 224, 224)).astype(np.uint8)
     net.set_input_data("input", cl.make_memory(eng, x))
-    log("built the network in %.1f s (%d primitives executed per run)" % (time.perf_counter() - t0, len(net.get_executed_primitive_ids())
-                                                                        if hasattr(net, "get_executed_primitive_ids") else -1))
+    log("built the network in %.1f s" % (time.perf_counter() - t0))
 
     def run():
         outs = net.execute()
@@ -215,20 +231,22 @@ def network_workload(args):
     dt = time.perf_counter() - t0
     logits = outs["fc1000"].get_memory().read()
     # multiply-adds the kernels execute: the graph passes let the layers in front of a stride-2 block compute only what
-    # that block reads, so this is less than the model's nominal count
-    nominal = 2.0 * batch * (workloads.macs(workloads.resnet50()) + 2048 * 1000)
+    # that block reads, so this can be less than the model's nominal count
+    nominal = 2.0 * batch * (workloads.macs(layers) + classes_in * 1000)
     plan = {n["id"]: n for n in cl.plan(topo, opts)}
     ops = 0.0
     for n in plan.values():
         if n["type"] in ("convolution", "fused_conv_eltwise"):
             ofm, ifm, fx, fy = plan[n["deps"][1 if n["type"] == "convolution" else 2]]["size"]
             ops += 2.0 * np.prod(n["size"]) * ifm * fx * fy
+    name = "ResNet-50" if resnet else "MobileNet-v2"
     print(json.dumps({
-        "metric": "ResNet-50 int8 network images/sec @b32 (whole topology through the clDNN API)", "value": batch * args.steps / dt,
+        "metric": "%s int8 network images/sec @b32 (whole topology through the clDNN API)" % name, "value": batch * args.steps / dt,
         "unit": "images/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": dt / args.steps * 1e3,
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "i8xi8->i32 (f32 requantisation)", "data": "synthetic",
-        "config": {"workload": "resnet50_b32_network", "batch": batch, "primitives": "53 convolution, 2 pooling, 16 eltwise (fused), 1 fully_connected",
-                   "build": "optimize_data" + (", tuning cache" if args.tuning_cache else ""), "executed_ops_per_step": ops, "nominal_ops_per_step": nominal},
+        "config": {"workload": args.workload, "batch": batch, "primitives": primitives,
+                   "build": "optimize_data" + (", tuning cache" if args.tuning_cache else ""), "kernels_per_execute": len([n for n in plan.values() if n["type"] not in ("data", "input_layout")]),
+                   "executed_ops_per_step": ops, "nominal_ops_per_step": nominal},
         "roofline": {"bound": "mfma", "achieved": ops * args.steps / dt / 1e12, "peak": PEAK_INT8_OPS / 1e12, "unit": "TOP/s",
                      "frac": ops * args.steps / dt / PEAK_INT8_OPS, "traffic": None, "kernel": "all kernels of one network.execute()"},
         "cpu_baseline": None, "distinct_logit_values": int(len(np.unique(logits)))}), flush=True)
@@ -253,13 +271,13 @@ def main():
     ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--workload", default="resnet50_b32_fused",
                     choices=["resnet50_b32_fused", "resnet50_b32", "resnet50_b1", "vgg16_b16", "mobilenet_v2_b32", "c1",
-                             "copy_256m", "resnet50_b32_network"])
+                             "copy_256m", "resnet50_b32_network", "mobilenet_v2_b32_network"])
     ap.add_argument("--tile", type=int, default=0, help="force one row (index+1) of the tile table on every layer")
     ap.add_argument("--per-layer", action="store_true", help="time every layer on its own and print a table to stderr")
     ap.add_argument("--tune", action="store_true", help="try every row of the tile table on every layer, print the best")
     ap.add_argument("--only", default="", help="comma-separated layer names: run just these layers of the workload "
                                                "(same buffers every step, so their tensors stay cache-resident)")
-    ap.add_argument("--tuning-cache", default="", help="resnet50_b32_network only: tune what this cache file lacks "
+    ap.add_argument("--tuning-cache", default="", help="network workloads only: tune what this cache file lacks "
                                                        "(build option tuning_config, tune_and_cache), then run from it")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline / full-size check")
     ap.add_argument("--host-io", action="store_true",
@@ -275,7 +293,7 @@ def main():
     wl = args.workload
     if wl == "copy_256m":
         return copy_calibration(args)
-    if wl == "resnet50_b32_network":
+    if wl.endswith("_network"):
         return network_workload(args)
     if wl.startswith("resnet50"):
         layers, batch, fuse = workloads.resnet50(), (1 if wl.endswith("b1") else 32), wl.endswith("fused")

@@ -121,6 +121,121 @@ __global__ void __launch_bounds__(256) eltwise_kernel(EltwiseArgs p, void* __res
     store_out(dst, p.dst_dt, p.dst.at(bi, f, y, x), o);
 }
 
+// The form a quantized network meets between its convolutions: every operand 8-bit in fs_b_yx_fsv16, same logical size
+// (strides allowed, no broadcast).  One lane = one pixel of one 16-feature slice: a 16-byte load per input, the same
+// arithmetic as above on 16 values, one 16-byte store; the padding features of the last slice are written as zero.
+struct EltwiseBlockedArgs {
+    const uint8_t* src[CLDNN_HIP_ELTWISE_MAX_INPUTS];
+    int off[CLDNN_HIP_ELTWISE_MAX_INPUTS], pb[CLDNN_HIP_ELTWISE_MAX_INPUTS], pf[CLDNN_HIP_ELTWISE_MAX_INPUTS],
+        py[CLDNN_HIP_ELTWISE_MAX_INPUTS], px[CLDNN_HIP_ELTWISE_MAX_INPUTS];  // bytes; the strides are folded into py / px
+    int is_u8[CLDNN_HIP_ELTWISE_MAX_INPUTS];
+    int count, mode;
+    int doff, dpb, dpf, dpy;
+    int B, F, Y, X, slices;
+    int quantized, calib_vec4;
+    const float* calib;
+    float oqf;
+    int act;
+    float m, n;
+};
+
+__global__ void __launch_bounds__(256) eltwise_blocked_kernel(EltwiseBlockedArgs p, uint8_t* __restrict__ dst)
+{
+    // grid: x over the pixels of a plane, y = batch, z = feature slice
+    const unsigned pixel = blockIdx.x * blockDim.x + threadIdx.x;
+    if (pixel >= (unsigned)(p.Y * p.X)) return;
+    const int y = (int)(pixel / (unsigned)p.X), x = (int)(pixel - (unsigned)y * p.X);
+    const int b = (int)blockIdx.y, fs = (int)blockIdx.z;
+    int v[16];
+    {
+        const uint4 w = *reinterpret_cast<const uint4*>(p.src[0] + p.off[0] + b * p.pb[0] + fs * p.pf[0] + y * p.py[0] + x * p.px[0]);
+        const unsigned ww[4] = {w.x, w.y, w.z, w.w};
+#pragma unroll
+        for (int c = 0; c < 16; ++c) {
+            const unsigned byte = (ww[c >> 2] >> (8 * (c & 3))) & 255u;
+            v[c] = p.is_u8[0] ? (int)byte : (int)(signed char)byte;
+        }
+    }
+    const bool wrap_unsigned = p.is_u8[0] != 0;
+    for (int i = 1; i < p.count; ++i) {
+        const uint4 w = *reinterpret_cast<const uint4*>(p.src[i] + p.off[i] + b * p.pb[i] + fs * p.pf[i] + y * p.py[i] + x * p.px[i]);
+        const unsigned ww[4] = {w.x, w.y, w.z, w.w};
+#pragma unroll
+        for (int c = 0; c < 16; ++c) {
+            const unsigned byte = (ww[c >> 2] >> (8 * (c & 3))) & 255u;
+            int o = p.is_u8[i] ? (int)byte : (int)(signed char)byte;
+            // an operand of the other 8-bit type is cast to the first input's type first
+            if (p.is_u8[i] != p.is_u8[0]) o = wrap_unsigned ? (int)(unsigned char)o : (int)(signed char)o;
+            int t = eltwise_op_int(p.mode, v[c], o);
+            if (!p.quantized) t = wrap_unsigned ? (int)(unsigned char)t : (int)(signed char)t;
+            v[c] = t;
+        }
+    }
+    unsigned out[4] = {0, 0, 0, 0};
+    const int f0 = fs * 16;
+    float scale[16];
+    if (p.quantized) {
+        if (p.calib && p.calib_vec4) {  // whole slices and an aligned vector: four 16-byte loads
+#pragma unroll
+            for (int d4 = 0; d4 < 4; ++d4) {
+                const float4 c4 = *reinterpret_cast<const float4*>(p.calib + f0 + d4 * 4);
+                scale[d4 * 4 + 0] = c4.x, scale[d4 * 4 + 1] = c4.y, scale[d4 * 4 + 2] = c4.z, scale[d4 * 4 + 3] = c4.w;
+            }
+        } else {
+#pragma unroll
+            for (int c = 0; c < 16; ++c) scale[c] = p.calib ? p.calib[f0 + c < p.F ? f0 + c : 0] : p.oqf;
+        }
+    }
+#pragma unroll
+    for (int c = 0; c < 16; ++c) {
+        int t = v[c];
+        if (p.quantized) {
+            const float s = scale[c];
+            t = (int)round_half_away((float)t * s);
+            t = t < -128 ? -128 : (t > 127 ? 127 : t);
+        }
+        t = act_i(p.act, p.m, p.n, t);
+        if (f0 + c < p.F) out[c >> 2] |= ((unsigned)t & 255u) << (8 * (c & 3));
+    }
+    *reinterpret_cast<uint4*>(dst + p.doff + b * p.dpb + fs * p.dpf + y * p.dpy + x * 16) = make_uint4(out[0], out[1], out[2], out[3]);
+}
+
+// true when the blocked kernel was launched
+static bool launch_eltwise_blocked(hipStream_t s, const cldnn_hip_eltwise_desc& d, const void* const* inputs, const float* calib, void* dst)
+{
+    const cldnn_hip_tensor& o = d.output;
+    auto byte_type = [](int dt) { return dt == CLDNN_HIP_S8 || dt == CLDNN_HIP_U8; };
+    if (o.format != CLDNN_HIP_FMT_FS_B_YX_FSV16 || !byte_type(o.dtype) || d.has_coefficients) return false;
+    if (tensor_elems(o) >= (1ull << 31)) return false;
+    EltwiseBlockedArgs p{};
+    for (int i = 0; i < d.n_inputs; ++i) {
+        const cldnn_hip_tensor& t = d.inputs[i];
+        const int sy = d.stride_y[i] > 0 ? d.stride_y[i] : 1, sx = d.stride_x[i] > 0 ? d.stride_x[i] : 1;
+        if (!inputs[i] || t.format != CLDNN_HIP_FMT_FS_B_YX_FSV16 || !byte_type(t.dtype) || tensor_elems(t) >= (1ull << 31)) return false;
+        // same features and batch, spatial size covered exactly: nothing wraps around
+        if (t.b != o.b || t.f != o.f || t.y / sy != o.y || t.x / sx != o.x) return false;
+        const Pitch q = make_pitch(t);
+        p.src[i] = (const uint8_t*)inputs[i];
+        p.off[i] = (int)q.off, p.pb[i] = (int)q.pb, p.pf[i] = (int)q.pf, p.py[i] = (int)q.py * sy, p.px[i] = (int)q.px * sx;
+        p.is_u8[i] = t.dtype == CLDNN_HIP_U8;
+    }
+    const Pitch q = make_pitch(o);
+    p.count = d.n_inputs, p.mode = d.mode;
+    p.doff = (int)q.off, p.dpb = (int)q.pb, p.dpf = (int)q.pf, p.dpy = (int)q.py;
+    p.B = o.b, p.F = o.f, p.Y = o.y, p.X = o.x, p.slices = (o.f + 15) / 16;
+    // (the stored value is the low byte of the result for either output type: conversion between the 8-bit types wraps)
+    p.quantized = d.quantized, p.calib = calib, p.oqf = d.output_quantization_factor;
+    p.act = d.activation, p.m = d.m, p.n = d.n;
+    p.calib_vec4 = calib && o.f % 16 == 0 && (uintptr_t)calib % 16 == 0;
+    const int64_t plane = (int64_t)p.Y * p.X;
+    if (plane == 0 || p.B == 0) return true;
+    if (p.B > 65535 || p.slices > 65535) return false;
+    hipLaunchKernelGGL(eltwise_blocked_kernel, dim3((unsigned)((plane + 255) / 256), (unsigned)p.B, (unsigned)p.slices), dim3(256), 0, s, p,
+                       (uint8_t*)dst);
+    CHIP_CHECK(hipGetLastError());
+    return true;
+}
+
 void launch_eltwise(hipStream_t s, const cldnn_hip_eltwise_desc& d, const void* const* inputs, const float* calib, void* dst)
 {
     CHIP_REQUIRE(d.n_inputs >= 2 && d.n_inputs <= CLDNN_HIP_ELTWISE_MAX_INPUTS, CLDNN_HIP_INVALID_ARG,
@@ -136,9 +251,10 @@ void launch_eltwise(hipStream_t s, const cldnn_hip_eltwise_desc& d, const void* 
     CHIP_REQUIRE(!d.quantized || int_data, CLDNN_HIP_INVALID_ARG, "eltwise: the quantized form needs int8 inputs");
     CHIP_REQUIRE(!d.has_coefficients || (!int_data && d.mode == CLDNN_HIP_ELTWISE_SUM), CLDNN_HIP_INVALID_ARG,
                  "eltwise: coefficients belong to a float sum");
+    const cldnn_hip_tensor& o = d.output;
+    if (int_data && launch_eltwise_blocked(s, d, inputs, calib, dst)) return;
     EltwiseArgs p{};
     p.count = d.n_inputs, p.mode = d.mode, p.has_coef = d.has_coefficients;
-    const cldnn_hip_tensor& o = d.output;
     for (int i = 0; i < d.n_inputs; ++i) {
         const cldnn_hip_tensor& t = d.inputs[i];
         CHIP_REQUIRE(inputs[i], CLDNN_HIP_INVALID_ARG, "eltwise: null input");

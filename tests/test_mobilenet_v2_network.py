@@ -1,0 +1,98 @@
+"""A whole quantized MobileNet-v2 (52 convolutions of which 17 depthwise, ReLU6 as clamp activations, 10 residual sums
+that stay stand-alone eltwise primitives, global average pooling, fully_connected) through the clDNN API against the CPU
+oracle run layer by layer, bit for bit."""
+import numpy as np
+import pytest
+
+from cldnn_amd import mobilenet_v2_net as mn
+from oracle import refconv as rc
+
+
+def run_oracle(x, params, folded=True, calibrate=False):
+    """Oracle forward pass.  folded: the clamp{0, 6} behind a convolution acts inside it on the dequantised value, before
+    the calibration (what optimize_data makes of the pair, as the reference's prepare_primitive_fusing does); otherwise
+    it is a primitive of its own and clamps the convolution's int8 output.  calibrate=True also chooses the factors:
+    the dequantised values of a ReLU6 layer get a root mean square of 3 and are requantised with 127 / 6; a linear
+    layer's outputs a root mean square of 30."""
+    t = {"input": x}
+    last = None
+    for step in mn.layer_plan():
+        if step[0] == "conv":
+            _, l, src = step
+            q, n = params[l["name"]], l["name"]
+            relu6 = l["act"] == "relu6"
+            kw = dict(stride=(l["stride"],) * 2, pad=(l["pad"],) * 2, groups=l["groups"], out_dt="s8")
+            if calibrate:
+                one = np.ones(l["ofm"], np.float32)
+                _, acc = rc.conv(t[src], q["w"], q["bias"], wqf=one, calib=one, want_acc=True, **kw)
+                full = acc.astype(np.float64) + q["bias"].reshape(1, -1, 1, 1)
+                rms = np.sqrt((full * full).mean(axis=(0, 2, 3))) + 1.0
+                q["wqf"] = ((3.0 if relu6 else 30.0) / rms).astype(np.float32)
+                q["calib"] = np.full(l["ofm"], 127.0 / 6.0 if relu6 else 1.0, np.float32)
+            if relu6 and folded:
+                t[n + "_relu6"] = rc.conv(t[src], q["w"], q["bias"], wqf=q["wqf"], calib=q["calib"], act="clamp", act_m=0.0, act_n=6.0, **kw)
+            else:
+                t[n] = rc.conv(t[src], q["w"], q["bias"], wqf=q["wqf"], calib=q["calib"], **kw)
+                if relu6:
+                    t[n + "_relu6"] = np.clip(t[n], 0, 6)  # the stand-alone activation clamps the int8 values themselves
+            last = n + ("_relu6" if relu6 else "")
+        elif step[0] == "sum":
+            _, n, shortcut, branch = step
+            if calibrate:
+                params[n] = dict(ecal=np.full(t[branch].shape[1], 0.75, np.float32))
+            t[n] = rc.eltwise([t[shortcut], t[branch]], "sum", calib=params[n]["ecal"])
+            last = n
+        elif step[0] == "pool":
+            t["pool"] = rc.pool(t[last], "average", None, global_pooling=True)
+        else:
+            q = params["fc1000"]
+            if calibrate:
+                acc = np.einsum("bfyx,ofyx->bo", t["pool"].astype(np.int64), q["w"].astype(np.int64)).astype(np.float64)
+                q["calib"] = np.full(q["w"].shape[0], 40.0 / (np.sqrt((acc * acc).mean()) + 1.0), np.float32)
+            t["fc1000"] = rc.fully_connected(t["pool"], q["w"], q["bias"], wqf=q["wqf"], calib=q["calib"])
+    return t
+
+
+def test_layer_plan_shape():
+    steps = mn.layer_plan()
+    assert [s[0] for s in steps].count("conv") == 52 and [s[0] for s in steps].count("sum") == 10
+    assert steps[-2:] == [("pool",), ("fc",)]
+    sums = [s for s in steps if s[0] == "sum"]
+    assert sums[0][1:] == ("b3", "b2_project", "b3_project") and sums[1][1:] == ("b5", "b4_project", "b5_project")
+    assert sums[2][1:] == ("b6", "b5", "b6_project")  # the second sum of a group reads the first one
+
+
+@pytest.mark.gpu
+def test_mobilenet_v2_int8_network_matches_the_oracle():
+    from cldnn_amd import api as cl
+    eng = cl.engine()
+    B = 2
+    x = np.random.default_rng(17).integers(0, 256, (B, 3, 224, 224)).astype(np.uint8)
+    params = mn.random_weights(seed=23)
+    run_oracle(x, params, calibrate=True)
+    topo = mn.topology(cl, eng, params, B)
+    # linear points only: a watched clamp would stay a primitive of its own also in the optimised build
+    watch = ["b1_project", "b3", "b7_project", "b10", "b14_project", "b17_project", "pool", "fc1000"]
+    for optimize in (True, False):
+        opts = cl.build_options(optimize_data=optimize, outputs=watch)
+        plan = {n["id"]: n for n in cl.plan(topo, opts)}
+        folded = [i for i, n in plan.items() if n["type"] == "convolution" and n.get("fused_activation") == cl.activation_func.clamp]
+        if optimize:
+            # every clamp is folded into the convolution before it; the residual sums have no activation and stay
+            # stand-alone; every convolution up to the classifier runs in the blocked layout
+            assert len(folded) == 35 and not any(n["type"] == "activation" for n in plan.values())
+            assert sum(n["type"] == "eltwise" for n in plan.values()) == 10 and not any("_fused_" in i for i in plan)
+            assert all(n["format"] == cl.format.fs_b_yx_fsv16 for n in plan.values() if n["type"] == "convolution" and not n.get("fully_connected"))
+        else:
+            assert folded == [] and sum(n["type"] == "activation" for n in plan.values()) == 35
+        ref = run_oracle(x, params, folded=optimize)
+        if optimize:
+            assert 3 < np.abs(ref["b17_project"].astype(np.int32)).mean() < 100 and len(np.unique(ref["fc1000"])) > 50  # alive to the end
+        net = cl.network(eng, topo, opts)
+        net.set_input_data("input", cl.make_memory(eng, x))
+        outs = net.execute()
+        for name in watch:
+            got = outs[name].get_memory().read()
+            assert got.shape == ref[name].shape, name
+            bad = int((got != ref[name]).sum())
+            assert bad == 0, "%s (optimize_data=%s): %d of %d values differ" % (name, optimize, bad, got.size)
