@@ -115,6 +115,7 @@ static int spatial(const cldnn_tensor& t, int i) { return t.sizes[2 + i]; }
 struct conv_geom {
     int B, IFM, IH, IW, OFM, FY, FX, sy, sx, dy, dx, py, px, OH, OW, groups;
     int ey, ex;  // zero padding on the high side minus the padding on the low side (asymmetric padding_above / below)
+    int vy, vx;  // positive input offset: the input is the view that leaves this many elements out on both sides (IH / IW are the view's)
 };
 
 // output extent with `lo` zeros in front of and `hi` behind the input (reference sliding_window_utils.h:113-126)
@@ -152,7 +153,13 @@ static conv_geom conv_geometry(const prim& p, const cldnn_layout& in, const cldn
     HOST_REQUIRE(p.input_offset.sizes[0] == 0 && p.input_offset.sizes[1] == 0, CLDNN_INVALID_ARG,
                  "input offset in batch / feature is not supported");
     int ox = spatial(p.input_offset, 0), oy = spatial(p.input_offset, 1);
-    HOST_REQUIRE(ox <= 0 && oy <= 0, CLDNN_INVALID_ARG, "positive input offsets are not supported");
+    // a positive offset moves the origin of the input into the data: the convolution runs on the view that leaves
+    // `offset` elements out on both sides (reference src/gpu/convolution_gpu.cpp:94-98 with the size rule of
+    // sliding_window_utils.h:113-126, input - 2 * offset)
+    g.vx = std::max(ox, 0), g.vy = std::max(oy, 0);
+    HOST_REQUIRE(2 * g.vx < g.IW && 2 * g.vy < g.IH, CLDNN_INVALID_ARG, "input offset is greater than the input data range");
+    g.IW -= 2 * g.vx, g.IH -= 2 * g.vy;
+    ox = std::min(ox, 0), oy = std::min(oy, 0);
     // padding_above / padding_below: zeros in front of / behind the input.  The reference folds the symmetric case
     // into the offset and puts a zero border primitive in front of the convolution otherwise
     // (handle_input_padding.cpp:27-92); here both are padding of the convolution itself.
@@ -161,6 +168,8 @@ static conv_geom conv_geometry(const prim& p, const cldnn_layout& in, const cldn
     HOST_REQUIRE(p.padding_above.sizes[0] == 0 && p.padding_above.sizes[1] == 0 && p.padding_below.sizes[0] == 0
                      && p.padding_below.sizes[1] == 0, CLDNN_INVALID_ARG, "padding above / below in batch or feature is not supported");
     HOST_REQUIRE(pax >= 0 && pay >= 0 && pbx >= 0 && pby >= 0, CLDNN_INVALID_ARG, "padding above / below cannot be negative");
+    HOST_REQUIRE((g.vx == 0 || (pax == 0 && pbx == 0)) && (g.vy == 0 || (pay == 0 && pby == 0)), CLDNN_INVALID_ARG,
+                 "a positive input offset together with padding above / below on the same axis is not supported");
     g.px = -ox + pax, g.py = -oy + pay;
     g.ex = pbx - pax, g.ey = pby - pay;
     const int ow = window_extent(g.IW, g.px, g.px + g.ex, g.FX, g.dx, g.sx);
@@ -744,6 +753,9 @@ static void compile_conv(cldnn_program_impl* prog, node* n)
 
     cldnn_hip_conv_desc d{};
     d.input = to_hip(in->out);
+    // a positive input offset: the same buffer, seen as the smaller tensor with what is left out counted as border
+    d.input.y = g.IH, d.input.x = g.IW;
+    d.input.pad_lo_y += g.vy, d.input.pad_hi_y += g.vy, d.input.pad_lo_x += g.vx, d.input.pad_hi_x += g.vx;
     d.output = to_hip(n->out);
     d.weights_dtype = hip_dtype(w->out.data_type);
     HOST_REQUIRE(d.weights_dtype == CLDNN_HIP_S8 || d.weights_dtype == CLDNN_HIP_F32, CLDNN_INVALID_ARG, "weights must be i8 or f32");

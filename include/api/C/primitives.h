@@ -95,7 +95,7 @@ CLDNN_END_PRIMITIVE_DESC(eltwise)
 CLDNN_DECLARE_PRIMITIVE_TYPE_ID(eltwise);
 
 CLDNN_BEGIN_PRIMITIVE_DESC(convolution)
-cldnn_tensor input_offset;   /* negative spatial values = zero padding */
+cldnn_tensor input_offset;   /* negative spatial values = zero padding; positive = that many elements left out on both sides */
 cldnn_tensor stride;
 cldnn_tensor dilation;
 uint32_t with_activation;

@@ -259,6 +259,32 @@ def test_with_output_size_same_input(eng):
     np.testing.assert_allclose(o1[:, :4], rc.conv(x, w1[:4], None, stride=(2, 2), pad=(3, 3)), rtol=1e-4, atol=1e-3)
 
 
+@pytest.mark.parametrize("optimize", OPT, ids=["plain", "optimize_data"])
+@pytest.mark.parametrize("offset,stride", [((1, 2), 1), ((2, 0), 2), ((1, -1), 1)], ids=["x1y2", "x2_s2", "x1_ypad1"])
+def test_positive_input_offset(eng, offset, stride, optimize):
+    """a positive input offset moves the origin into the data: the convolution runs on the view that leaves `offset`
+    elements out on both sides (reference src/gpu/convolution_gpu.cpp:94-98, sliding_window_utils.h:113-126)"""
+    r = np.random.default_rng(31)
+    B, Cn, H, W, OFM = 2, 64, 11, 14, 64
+    x = r.integers(-128, 128, (B, Cn, H, W)).astype(np.int8)
+    w = r.integers(-127, 128, (OFM, Cn, 3, 3)).astype(np.int8)
+    cal = r.uniform(2e-4, 8e-4, OFM).astype(np.float32)
+    ox, oy = offset
+    t = cl.topology(cl.input_layout("input", cl.layout(DT.i8, F.bfyx, cl.tensor(B, Cn, W, H))), cl.data("w", cl.make_memory(eng, w)),
+                    cl.data("q", vec_mem(eng, np.ones(OFM, np.float32))), cl.data("c", vec_mem(eng, cal)),
+                    cl.convolution("conv", "input", ["w"], None, ["q"], ["c"], stride=cl.tensor(1, 1, stride, stride),
+                                   input_offset=cl.tensor(0, 0, ox, oy, 0), with_activation=True))
+    net, outs = run(eng, t, {"input": cl.make_memory(eng, x)}, optimize)
+    vy, vx = max(oy, 0), max(ox, 0)
+    view = x[:, :, vy:H - vy, vx:W - vx]
+    ref = rc.conv(view, w, None, wqf=np.ones(OFM, np.float32), calib=cal, stride=(stride, stride), pad=(max(-oy, 0), max(-ox, 0)), act="relu")
+    got = outs["conv"].get_memory().read()
+    assert got.shape == ref.shape
+    np.testing.assert_array_equal(got, ref)
+    # the view must not be the whole tensor shifted: the last rows / columns are left out as well
+    assert ref.shape[3] == (W - 2 * vx + 2 * max(-ox, 0) - 3) // stride + 1
+
+
 # ------------------------------------------------------------------------------------------ networks vs the oracle
 def rand_layer(r, ofm, ifm, k, in_u8=True):
     w = r.integers(-127, 128, (ofm, ifm, k, k)).astype(np.int8)
