@@ -367,7 +367,17 @@ bool mfma_fast_epilogue(const ConvProblem& p, const Epilogue& e, const float* ca
             for (int f = 0; f < p.OFM && nonneg; ++f) nonneg = calib[f] >= 0.0f;
         else if (e.oqf_on) nonneg = e.oqf >= 0.0f;
         F.relu_folded = nonneg ? 1 : 0;
+    } else if (e.act == CLDNN_HIP_ACT_CLAMP && !F.fc && e.act_m >= 0.0f) {
+        // x in [m, n], factor >= 0: 0 <= x * factor <= n * factor (rounding is monotonic), so if n * factor is inside the
+        // output range the second clamp does nothing and the value rounds like a non-negative number
+        bool inside = true;
+        auto ok = [&](float factor) { return factor >= 0.0f && e.act_n * factor <= F.hi; };
+        if (calib)
+            for (int f = 0; f < p.OFM && inside; ++f) inside = ok(calib[f]);
+        else inside = ok(e.oqf_on ? e.oqf : 1.0f);
+        F.clamp_folded = inside ? 1 : 0;
     }
+    F.iqf_one = e.iqf == 1.0f ? 1 : 0;
     *out = F;
     return true;
 }

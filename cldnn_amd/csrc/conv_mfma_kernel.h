@@ -245,15 +245,27 @@ __device__ __forceinline__ v4i epilogue_fast16(const Args& a, const v4i (&acc)[4
         return packed;
     }
     if (F.has_wqf) {
+        if (F.iqf_one) {
 #pragma unroll
-        for (int c = 0; c < 16; ++c) {
-            v[c] = v[c] * wq[c];
-            v[c] = v[c] * F.iqf;
+            for (int c = 0; c < 16; ++c) v[c] = v[c] * wq[c];
+        } else {
+#pragma unroll
+            for (int c = 0; c < 16; ++c) {
+                v[c] = v[c] * wq[c];
+                v[c] = v[c] * F.iqf;
+            }
         }
     }
     v4i packed;
     bool finished = false;
-    if (F.fc) {
+    if (F.clamp_folded) {
+        // clamp{m, n} on the dequantised value (ReLU6), then the calibration: the result lies in [0, n * factor], which
+        // the host has checked to be inside the output range
+#pragma unroll
+        for (int c = 0; c < 16; ++c) v[c] = med3(v[c], F.act_m, F.act_n) * cal[c] + 0.49999997f;
+#pragma unroll
+        for (int d = 0; d < 4; ++d) packed[d] = pack_nonneg(v + d * 4);
+    } else if (F.fc) {
         // reference fully_connected_gpu_bfyx_ref.cl:63-84: (char)round((acc * wqf * iqf + bias) * factor), then the
         // activation on the char; ecal[] holds the bias
 #pragma unroll

@@ -82,6 +82,9 @@ struct FastEpi {
     int32_t eltw_u8;
     float lo, hi;         // saturation bounds of the output type
     float iqf;
+    int32_t iqf_one;      // iqf == 1: the multiplication is left out (x * 1.0f == x)
+    int32_t clamp_folded; // clamp{m, n} with 0 <= m <= n, factors >= 0 and n * factor inside the output range: the result
+                          // needs no second clamp and rounds like a non-negative number
     int32_t fc;           // the fully_connected form: float bias after the dequantisation, conversion to char keeps the low byte
 };
 // true (and *out filled) when the short epilogue reproduces the long one bit for bit
