@@ -174,19 +174,25 @@ def network_workload(args):
     """A whole quantized network built and run through the clDNN API with optimize_data: what an application sees per
     network.execute(), input already on the device.  resnet50_b32_network: 53 convolutions, 2 poolings, 16 residual sums,
     fully_connected; mobilenet_v2_b32_network: 52 convolutions (17 depthwise), 35 clamps, 10 residual sums, pooling,
-    fully_connected."""
+    fully_connected; vgg16_b16_network: 13 convolutions, 5 poolings, 3 fully_connected (the first over a 7x7 plane)."""
     from cldnn_amd import api as cl
     batch = 32
     eng = cl.engine()
     r = np.random.default_rng(1337)
-    resnet = args.workload.startswith("resnet50")
+    resnet, vgg = args.workload.startswith("resnet50"), args.workload.startswith("vgg16")
+    out_id, fcs = "fc1000", []
     if resnet:
         from cldnn_amd import resnet50_net as net_def
-        layers, classes_in = workloads.resnet50(), 2048
+        layers, fcs = workloads.resnet50(), [("fc1000", 2048, 1000)]
         primitives = "53 convolution, 2 pooling, 16 eltwise (fused), 1 fully_connected"
+    elif vgg:
+        from cldnn_amd import vgg16_net as net_def
+        batch, out_id = 16, "fc8"
+        layers, fcs = workloads.vgg16(), [("fc6", 25088, 4096), ("fc7", 4096, 4096), ("fc8", 4096, 1000)]
+        primitives = "13 convolution, 5 pooling, 3 fully_connected"
     else:
         from cldnn_amd import mobilenet_v2_net as net_def
-        layers, classes_in = workloads.mobilenet_v2(), 1280
+        layers, fcs = workloads.mobilenet_v2(), [("fc1000", 1280, 1000)]
         primitives = "52 convolution (17 depthwise), 35 activation clamp (folded), 10 eltwise, 1 pooling, 1 fully_connected"
     params = net_def.random_weights()
     IN_RMS, ECAL = 35.0, 1.0  # keep the signal alive through the blocks without a calibration pass
@@ -202,7 +208,8 @@ def network_workload(args):
     for step in net_def.layer_plan():
         if step[0] == "sum":
             params[step[1]] = dict(ecal=np.full(params[step[3]]["w"].shape[0], ECAL if resnet else 0.75, np.float32))
-    params["fc1000"]["calib"] = np.full(1000, 40.0 / (np.sqrt(classes_in) * 30.0 * 73.3), np.float32)
+    for name, k, ofm in fcs:
+        params[name]["calib"] = np.full(ofm, 40.0 / (np.sqrt(k) * 30.0 * 73.3), np.float32)
     t0 = time.perf_counter()
     topo, opts = net_def.topology(cl, eng, params, batch), cl.build_options(optimize_data=True)
     if args.tuning_cache:
@@ -220,7 +227,7 @@ def network_workload(args):
 
     def run():
         outs = net.execute()
-        outs["fc1000"].get_event().wait()
+        outs[out_id].get_event().wait()
         return outs
 
     for _ in range(args.warmup):
@@ -229,19 +236,19 @@ def network_workload(args):
     for _ in range(args.steps):
         outs = run()
     dt = time.perf_counter() - t0
-    logits = outs["fc1000"].get_memory().read()
+    logits = outs[out_id].get_memory().read()
     # multiply-adds the kernels execute: the graph passes let the layers in front of a stride-2 block compute only what
     # that block reads, so this can be less than the model's nominal count
-    nominal = 2.0 * batch * (workloads.macs(layers) + classes_in * 1000)
+    nominal = 2.0 * batch * (workloads.macs(layers) + sum(k * ofm for _, k, ofm in fcs))
     plan = {n["id"]: n for n in cl.plan(topo, opts)}
     ops = 0.0
     for n in plan.values():
         if n["type"] in ("convolution", "fused_conv_eltwise"):
             ofm, ifm, fx, fy = plan[n["deps"][1 if n["type"] == "convolution" else 2]]["size"]
             ops += 2.0 * np.prod(n["size"]) * ifm * fx * fy
-    name = "ResNet-50" if resnet else "MobileNet-v2"
+    name = "ResNet-50" if resnet else ("VGG-16" if vgg else "MobileNet-v2")
     print(json.dumps({
-        "metric": "%s int8 network images/sec @b32 (whole topology through the clDNN API)" % name, "value": batch * args.steps / dt,
+        "metric": "%s int8 network images/sec @b%d (whole topology through the clDNN API)" % (name, batch), "value": batch * args.steps / dt,
         "unit": "images/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": dt / args.steps * 1e3,
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "i8xi8->i32 (f32 requantisation)", "data": "synthetic",
         "config": {"workload": args.workload, "batch": batch, "primitives": primitives,
@@ -271,7 +278,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--workload", default="resnet50_b32_fused",
                     choices=["resnet50_b32_fused", "resnet50_b32", "resnet50_b1", "vgg16_b16", "mobilenet_v2_b32", "c1",
-                             "copy_256m", "resnet50_b32_network", "mobilenet_v2_b32_network"])
+                             "copy_256m", "resnet50_b32_network", "mobilenet_v2_b32_network", "vgg16_b16_network"])
     ap.add_argument("--tile", type=int, default=0, help="force one row (index+1) of the tile table on every layer")
     ap.add_argument("--per-layer", action="store_true", help="time every layer on its own and print a table to stderr")
     ap.add_argument("--tune", action="store_true", help="try every row of the tile table on every layer, print the best")

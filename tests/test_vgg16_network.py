@@ -1,0 +1,67 @@
+"""A whole quantized VGG-16 (13 convolutions, 5 max poolings, 3 fully_connected layers of which the first reads a 7x7
+plane: K = 25088) through the clDNN API against the CPU oracle run layer by layer, bit for bit."""
+import numpy as np
+import pytest
+
+from cldnn_amd import vgg16_net as vg
+from oracle import refconv as rc
+
+
+def run_oracle(x, params, calibrate=False):
+    """Oracle forward pass; calibrate=True also chooses every layer's factors (root mean square of the outputs at about a
+    quarter of the int8 range)."""
+    t = {"input": x}
+    for step in vg.layer_plan():
+        if step[0] == "conv":
+            _, l, src = step
+            q = params[l["name"]]
+            if calibrate:
+                _, acc = rc.conv(t[src], q["w"], q["bias"], wqf=q["wqf"], calib=np.ones(l["ofm"], np.float32), pad=(1, 1), out_dt="s8", want_acc=True)
+                full = acc.astype(np.float64) + q["bias"].reshape(1, -1, 1, 1)
+                q["calib"] = (32.0 / (np.sqrt((full * full).mean(axis=(0, 2, 3))) + 1.0)).astype(np.float32)
+            t[l["name"]] = rc.conv(t[src], q["w"], q["bias"], wqf=q["wqf"], calib=q["calib"], pad=(1, 1), out_dt="s8", act="relu")
+        elif step[0] == "pool":
+            _, n, src = step
+            t[n] = rc.pool(t[src], "max", (2, 2), (2, 2))
+        else:
+            _, n, src, ifm, plane, ofm, relu = step
+            q = params[n]
+            xin = t[src].reshape(x.shape[0], ifm, plane, plane)
+            if calibrate:
+                acc = np.einsum("bfyx,ofyx->bo", xin.astype(np.int64), q["w"].astype(np.int64)).astype(np.float64)
+                q["calib"] = np.full(ofm, 40.0 / (np.sqrt((acc * acc).mean()) + 1.0), np.float32)
+            t[n] = rc.fully_connected(xin, q["w"], q["bias"], wqf=q["wqf"], calib=q["calib"], act="relu" if relu else "none")
+    return t
+
+
+def test_layer_plan_shape():
+    steps = vg.layer_plan()
+    assert [s[0] for s in steps].count("conv") == 13 and [s[0] for s in steps].count("pool") == 5
+    assert [s[1] for s in steps if s[0] == "fc"] == ["fc6", "fc7", "fc8"] and steps[-3][3:6] == (512, 7, 4096)
+
+
+@pytest.mark.gpu
+def test_vgg16_int8_network_matches_the_oracle():
+    from cldnn_amd import api as cl
+    eng = cl.engine()
+    B = 2
+    x = np.random.default_rng(41).integers(0, 256, (B, 3, 224, 224)).astype(np.uint8)
+    params = vg.random_weights(seed=43)
+    ref = run_oracle(x, params, calibrate=True)
+    assert 5 < np.abs(ref["pool5"].astype(np.int32)).mean() < 100 and len(np.unique(ref["fc8"])) > 50  # alive to the end
+    topo = vg.topology(cl, eng, params, B)
+    watch = ["pool1", "conv5", "pool3", "pool5", "fc6", "fc7", "fc8"]
+    for optimize in (True, False):
+        opts = cl.build_options(optimize_data=optimize, outputs=watch)
+        if optimize:
+            plan = {n["id"]: n for n in cl.plan(topo, opts)}
+            # the pooling layers stay in the blocked layout between the convolutions
+            assert all(plan[i]["format"] == cl.format.fs_b_yx_fsv16 for i in ("pool2", "pool4", "conv6", "conv12"))
+        net = cl.network(eng, topo, opts)
+        net.set_input_data("input", cl.make_memory(eng, x))
+        outs = net.execute()
+        for name in watch:
+            got = outs[name].get_memory().read()
+            assert got.reshape(ref[name].shape).shape == ref[name].shape, name
+            bad = int((got.reshape(ref[name].shape) != ref[name]).sum())
+            assert bad == 0, "%s (optimize_data=%s): %d of %d values differ" % (name, optimize, bad, got.size)
