@@ -61,3 +61,12 @@ def test_no_device_fails_loudly():
         hip.Engine()
     assert ei.value.status == -4
     assert "no HIP device" in str(ei.value)
+
+
+def test_bench_refuses_more_than_one_gpu():
+    """bench.py measures one GPU; asking for more ends with a message and a non-zero status before anything is loaded"""
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    r = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"], capture_output=True, text=True, timeout=120)
+    assert r.returncode != 0 and "one GPU" in r.stderr and r.stdout.strip() == ""
