@@ -2,6 +2,10 @@
 
 TEST INFRASTRUCTURE ONLY: imported by tests/, by __graft_entry__.smoke() and by
 bench.py's cpu_baseline leg, never by the product package.
+
+Pinned by the reference's own known-answer tables (tests/golden/*.json): conv / fused conv / pooling /
+fully_connected in refconv.c, eltwise() here.  Parity unpinned (no table of the reference covers them): float pow and
+mod of eltwise(); integer division and modulo by zero (0 here, undefined in the reference).
 """
 import ctypes as C
 import os
