@@ -286,6 +286,10 @@ def main():
                                                "(same buffers every step, so their tensors stay cache-resident)")
     ap.add_argument("--tuning-cache", default="", help="network workloads only: tune what this cache file lacks "
                                                        "(build option tuning_config, tune_and_cache), then run from it")
+    ap.add_argument("--in-flight", type=int, default=2,
+                    help="after the headline measurement also time this many independent requests of the same workload in "
+                         "flight at once, one engine (HIP stream) and one host thread each; reported under "
+                         "requests_in_flight, never as the headline value (0 or 1 = skip)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline / full-size check")
     ap.add_argument("--host-io", action="store_true",
                     help="also report the rate with the first layer's input crossing PCIe into the device and the last "
@@ -343,6 +347,39 @@ def main():
     ms_per_step = t_wall / args.steps * 1e3
     value = batch * args.steps / t_wall
 
+    in_flight = None
+    if args.in_flight > 1 and not args.only:
+        # What an application gets that keeps several requests going (the reference's users run one network per request
+        # and thread): every request has an engine = stream of its own; kernels of different requests overlap on the
+        # device and fill what one request's kernels leave idle.
+        import threading
+        engines = [eng] + [hip.Engine(0, profiling=False) for _ in range(args.in_flight - 1)]
+        stacks = [stack] + [build_stack(e, layers, batch, fuse, seed=1337 + 1000 * (k + 1), tile=args.tile) for k, e in enumerate(engines[1:])]
+
+        def request_loop(k, count):
+            for _ in range(count):
+                run_step(stacks[k])
+            engines[k].finish()
+        for k in range(len(engines)):
+            request_loop(k, 5)
+        threads = [threading.Thread(target=request_loop, args=(k, args.steps)) for k in range(len(engines))]
+        t0 = time.perf_counter()
+        for t in threads:
+            t.start()
+        for t in threads:
+            t.join()
+        dt = time.perf_counter() - t0
+        in_flight = {"requests": len(engines), "steps_per_request": args.steps, "images_per_s": len(engines) * batch * args.steps / dt,
+                     "ms_per_request_step": dt / args.steps * 1e3, "tops": len(engines) * ops * args.steps / dt / 1e12,
+                     "frac_of_int8_peak": len(engines) * ops * args.steps / dt / PEAK_INT8_OPS,
+                     "what": "independent requests of this workload, one engine (HIP stream at default priority) and one host thread each"}
+        for L in [L for st in stacks[1:] for L in st]:
+            L.conv.close(), L.out.close(), L.xin.close()
+            if L.ein is not None:
+                L.ein.close()
+        del stacks
+        for e in engines[1:]:
+            e.close()
     host_io = None
     if args.host_io:
         # what a caller holding host tensors pays: bfyx input host -> device, device reorder into the blocked layout
@@ -457,6 +494,8 @@ def main():
     }
     if host_io:
         res["pcie_inclusive"] = host_io
+    if in_flight:
+        res["requests_in_flight"] = in_flight
 
     if not args.no_cpu:
         cb = cpu_baseline_and_check(eng, stack, batch, args.cpu_seconds)
