@@ -440,6 +440,35 @@ def test_reorder_into_blocked_layouts(eng, shape, pad, fmt):
     buf.close()
 
 
+def test_two_engines_from_two_threads():
+    """one engine (= stream) and one host thread per request: the C-ABI keeps no state that two requests could share
+    (the last error message is per thread)"""
+    import threading
+    results, errors = {}, []
+    probs = {k: problem(50 + k, 2, 64, 14, 14, 128, 3, 3) for k in range(2)}
+    refs = {k: rc.conv(p[0], p[1], p[2], wqf=p[3], calib=p[4], pad=(1, 1), out_dt="s8", act="relu") for k, p in probs.items()}
+
+    def request(k):
+        try:
+            e = hip.Engine(0)
+            x, w, bias, wqf, calib = probs[k]
+            for _ in range(20):
+                results[k] = hip.conv_forward(e, x, w, bias, wqf, calib, pad=(1, 1), out_dt="s8", act="relu", fmt="fs_b_yx_fsv16")
+            with pytest.raises(hip.HipError, match="tile_override out of range"):
+                hip.conv_forward(e, x, w, bias, wqf, calib, pad=(1, 1), out_dt="s8", fmt="fs_b_yx_fsv16", tile=10 ** 6)
+            e.close()
+        except Exception as err:  # noqa: BLE001 - reported by the main thread
+            errors.append(err)
+    threads = [threading.Thread(target=request, args=(k,)) for k in range(2)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert not errors, errors
+    for k in range(2):
+        assert_same(refs[k], results[k])
+
+
 def test_reorder_f32_to_int8_goes_towards_zero_and_saturates(eng):
     """the reference's reorder converts with convert_char (jitter.cpp:483): towards zero; its pooling test relies on
     9.5 -> 9 (pooling_gpu_test.cpp:264-309).  Out-of-range values saturate here."""
