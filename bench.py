@@ -177,7 +177,7 @@ def network_workload(args):
     fully_connected; vgg16_b16_network: 13 convolutions, 5 poolings, 3 fully_connected (the first over a 7x7 plane)."""
     from cldnn_amd import api as cl
     batch = 32
-    eng = cl.engine()
+    eng = cl.engine(enable_parallelisation=args.second_stream)
     r = np.random.default_rng(1337)
     resnet, vgg = args.workload.startswith("resnet50"), args.workload.startswith("vgg16")
     out_id, fcs = "fc1000", []
@@ -252,7 +252,7 @@ def network_workload(args):
         "unit": "images/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": dt / args.steps * 1e3,
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "i8xi8->i32 (f32 requantisation)", "data": "synthetic",
         "config": {"workload": args.workload, "batch": batch, "primitives": primitives,
-                   "build": "optimize_data" + (", tuning cache" if args.tuning_cache else ""), "kernels_per_execute": len([n for n in plan.values() if n["type"] not in ("data", "input_layout")]),
+                   "build": "optimize_data" + (", tuning cache" if args.tuning_cache else "") + (", second stream" if args.second_stream else ""), "kernels_per_execute": len([n for n in plan.values() if n["type"] not in ("data", "input_layout")]),
                    "executed_ops_per_step": ops, "nominal_ops_per_step": nominal},
         "roofline": {"bound": "mfma", "achieved": ops * args.steps / dt / 1e12, "peak": PEAK_INT8_OPS / 1e12, "unit": "TOP/s",
                      "frac": ops * args.steps / dt / PEAK_INT8_OPS, "traffic": None, "kernel": "all kernels of one network.execute()"},
@@ -286,6 +286,8 @@ def main():
                                                "(same buffers every step, so their tensors stay cache-resident)")
     ap.add_argument("--tuning-cache", default="", help="network workloads only: tune what this cache file lacks "
                                                        "(build option tuning_config, tune_and_cache), then run from it")
+    ap.add_argument("--second-stream", action="store_true", help="network workloads only: engine option enable_parallelisation "
+                    "(shortcut convolutions run on a second stream beside the branch)")
     ap.add_argument("--in-flight", type=int, default=2,
                     help="after the headline measurement also time this many independent requests of the same workload in "
                          "flight at once, one engine (HIP stream) and one host thread each; reported under "

@@ -334,13 +334,14 @@ def _layout_shape(l):
 class engine:  # noqa: N801
     """cldnn::engine (reference api/CPP/engine.hpp:96-190)."""
 
-    def __init__(self, engine_num=0, enable_profiling=False, enable_memory_pool=True, _handle=None):
+    def __init__(self, engine_num=0, enable_profiling=False, enable_memory_pool=True, enable_parallelisation=False, _handle=None):
         if _handle is not None:
             self.h = _handle
             return
         cfg = c_engine_configuration()
         cfg.enable_profiling = 1 if enable_profiling else 0
         cfg.enable_memory_pool = 1 if enable_memory_pool else 0  # the reference's default is on (api/CPP/engine.hpp:66)
+        cfg.enable_parallelisation = 1 if enable_parallelisation else 0  # independent branches on a second stream
         self.h = _call("cldnn_create_engine", 0, engine_num, C.byref(cfg))
 
     @staticmethod

@@ -123,6 +123,9 @@ static void execute(cldnn_network_impl* net, cldnn_event* deps, size_t ndeps)
     }
     net->executed.clear();
     net->events.clear();
+    for (cldnn_hip_event ev : net->stream_events) cldnn_hip_event_release(ev);  // the previous run's; it has been waited for
+    net->stream_events.clear();
+    std::map<node*, cldnn_hip_event> joins;  // completion of the primitives on the second stream
     for (auto& u : prog->nodes) {
         node* n = u.get();
         prim& p = *n->p;
@@ -138,8 +141,22 @@ static void execute(cldnn_network_impl* net, cldnn_event* deps, size_t ndeps)
             return it->second.get();
         };
         cldnn_memory_impl* out = mem_of(n);
+        // a primitive on the second stream starts when everything issued before it on the first has finished (its
+        // inputs, and whatever used its output buffer before); its user waits for it
+        cldnn_hip_engine where = eng->h;
+        if (n->side_stream) {
+            where = eng->side;
+            cldnn_hip_event fork = nullptr;
+            hip_check(cldnn_hip_event_record(eng->h, &fork));
+            net->stream_events.push_back(fork);
+            hip_check(cldnn_hip_engine_wait_events(eng->side, &fork, 1));
+        }
+        for (node* d : n->deps) {
+            auto j = joins.find(d);
+            if (j != joins.end()) hip_check(cldnn_hip_engine_wait_events(eng->h, &j->second, 1));
+        }
         cldnn_hip_event pev = nullptr;
-        if (eng->profiling) hip_check(cldnn_hip_event_record_begin(eng->h, &pev));
+        if (eng->profiling) hip_check(cldnn_hip_event_record_begin(where, &pev));
         const cldnn_hip_tensor ot = to_hip(n->out);
         switch (p.type) {
         case prim_type::reorder: {
@@ -197,6 +214,12 @@ static void execute(cldnn_network_impl* net, cldnn_event* deps, size_t ndeps)
         }
         default: break;
         }
+        if (n->side_stream) {
+            cldnn_hip_event join = nullptr;
+            hip_check(cldnn_hip_event_record(eng->side, &join));
+            net->stream_events.push_back(join);
+            joins[n] = join;
+        }
         if (pev) {
             hip_check(cldnn_hip_event_record_end(pev));
             ref<cldnn_event_impl> ev(new cldnn_event_impl(), false);
@@ -218,6 +241,7 @@ static void execute(cldnn_network_impl* net, cldnn_event* deps, size_t ndeps)
         }
         net->events[n] = marker;
     }
+    if (eng->side) hip_check(cldnn_hip_engine_flush(eng->side));
     hip_check(cldnn_hip_engine_flush(eng->h));
     net->has_run = true;
 }
@@ -228,6 +252,7 @@ using namespace host;
 
 cldnn_engine_impl::~cldnn_engine_impl()
 {
+    if (side) cldnn_hip_engine_release(side);
     if (h) cldnn_hip_engine_release(h);
 }
 cldnn_memory_impl::~cldnn_memory_impl()
@@ -237,6 +262,10 @@ cldnn_memory_impl::~cldnn_memory_impl()
 cldnn_event_impl::~cldnn_event_impl()
 {
     if (h) cldnn_hip_event_release(h);
+}
+cldnn_network_impl::~cldnn_network_impl()
+{
+    for (cldnn_hip_event ev : stream_events) cldnn_hip_event_release(ev);
 }
 cldnn_program_impl::~cldnn_program_impl()
 {
@@ -480,9 +509,11 @@ cldnn_engine cldnn_create_engine(int32_t type, uint32_t engine_num, const cldnn_
         }
         ref<cldnn_engine_impl> e(new cldnn_engine_impl(), false);
         e->profiling = cfg && cfg->enable_profiling;
+        const bool parallel = cfg && cfg->enable_parallelisation;
         if (cfg && cfg->tuning_cache_path && cfg->tuning_cache_path[0]) e->tuning_cache_path = cfg->tuning_cache_path;
         e->memory_pool = !cfg || cfg->enable_memory_pool;
         hip_check(cldnn_hip_engine_create(engine_num, e->profiling ? 1 : 0, &e->h));
+        if (parallel) hip_check(cldnn_hip_engine_create(engine_num, e->profiling ? 1 : 0, &e->side));
         e->retain();
         return e.get();
     });
@@ -665,6 +696,11 @@ cldnn_network cldnn_allocate_network(cldnn_program program, cldnn_status* status
         }
         for (auto& u : program->nodes)
             for (node* d : u->deps) last_use[d] = std::max(last_use[d], index[u.get()]);
+        // a primitive on the second stream may still read its inputs while the first stream moves on: they stay
+        // reserved until the primitive that waits for it
+        for (auto& u : program->nodes)
+            if (u->side_stream)
+                for (node* d : u->deps) last_use[d] = std::max(last_use[d], index[u->users.at(0)]);
         const bool pool = e->memory_pool && !aliasing;
         std::vector<std::pair<size_t, ref<cldnn_memory_impl>>> in_flight;  // (index of the last consumer, buffer)
         std::vector<ref<cldnn_memory_impl>> idle;

@@ -81,6 +81,7 @@ std::string conv_signature(const cldnn_hip_conv_desc& d);
 
 struct cldnn_engine_impl : host::refcounted {
     cldnn_hip_engine h = nullptr;
+    cldnn_hip_engine side = nullptr;  // second stream for primitives nothing waits for yet (enable_parallelisation)
     bool profiling = false;
     std::string tuning_cache_path = "cache.json";  // engine configuration; a tuning_config without a path of its own uses it
     bool memory_pool = true;  // networks share buffers between intermediate tensors whose lifetimes do not overlap
@@ -160,6 +161,7 @@ struct node {
     std::string org_id;             // id in the user's topology ("" for inserted nodes)
     std::vector<node*> deps;        // data dependencies in primitive order (input, [input2], weights, bias, wqf, calib, [eltw calib])
     std::vector<node*> users;
+    bool side_stream = false;       // runs on the engine's second stream, joined before its only user
     cldnn_layout out{};             // output layout incl. physical padding
     int32_t user_format = cldnn_format_any;  // output format before the layout pass (what the topology implies)
     bool is_output = false;
@@ -193,7 +195,9 @@ struct cldnn_network_impl : host::refcounted {
     std::map<host::node*, host::ref<cldnn_event_impl>> events;
     std::map<std::string, bool> input_set;
     std::vector<std::string> executed;
+    std::vector<cldnn_hip_event> stream_events;  // fork / join events between the two streams of the last run
     bool has_run = false;
     size_t allocated_bytes = 0;  // device bytes of the buffers the network allocated for its primitives' outputs
     size_t pooled_tensors = 0;   // outputs that reuse the buffer of an earlier, finished tensor
+    ~cldnn_network_impl() override;
 };

@@ -863,10 +863,34 @@ static void compile_conv(cldnn_program_impl* prog, node* n)
             ++prog->tuned_now;
         }
     }
-    hip_check(cldnn_hip_conv_create(prog->engine->h, &d, wv.data(), bv.empty() ? nullptr : bv.data(),
+    hip_check(cldnn_hip_conv_create(n->side_stream ? prog->engine->side : prog->engine->h, &d, wv.data(), bv.empty() ? nullptr : bv.data(),
                                     qv.empty() ? nullptr : (const float*)qv.data(), cv.empty() ? nullptr : (const float*)cv.data(),
                                     (const float*)eltw_calib, &n->conv));
     hip_check(cldnn_hip_conv_get_info(n->conv, &n->conv_info));
+}
+
+// enable_parallelisation (reference api/C/cldnn.h:152, "parallel execution of primitives which don't depend on each
+// other"): a convolution whose only user comes at least two primitives later in execution order -- the projection
+// shortcut of a residual block -- runs on the engine's second stream while the primitives in between run on the
+// first; the user waits for it.
+static void assign_streams(cldnn_program_impl* prog)
+{
+    for (size_t i = 0; i < prog->nodes.size(); ++i) {
+        node* x = prog->nodes[i].get();
+        if (x->constant || x->is_output || x->users.size() != 1) continue;
+        if (x->p->type != prim_type::convolution || x->p->fully_connected) continue;
+        bool plain_deps = true;
+        for (node* d : x->deps) plain_deps = plain_deps && !d->side_stream;
+        if (!plain_deps) continue;
+        node* user = x->users[0];
+        if (user->p->type == prim_type::fused_conv_eltwise && user->p->second_input_in_output) continue;
+        size_t between = 0;  // primitives that execute between the two
+        const size_t pu = position(prog, user);
+        for (size_t k = i + 1; k < pu; ++k)
+            if (!prog->nodes[k]->constant && prog->nodes[k]->p->type != prim_type::input_layout) ++between;
+        if (pu == (size_t)-1 || pu <= i || between == 0) continue;
+        x->side_stream = true;
+    }
 }
 
 // ------------------------------------------------------------------------------------------ build
@@ -922,6 +946,7 @@ void build_program(cldnn_program_impl* prog, cldnn_topology_impl* topo, const st
     for (auto& u : prog->nodes) calc_layout(u.get());
     prepare_borders(prog);
     if (!prog->engine) return;  // planning only: the graph is inspected, nothing is compiled
+    if (prog->engine->side) assign_streams(prog);
     for (auto& u : prog->nodes) {
         node* n = u.get();
         if (n->p->type == prim_type::convolution || n->p->type == prim_type::fused_conv_eltwise) compile_conv(prog, n);
@@ -960,6 +985,7 @@ std::string describe_node(const node* n)
         for (size_t i = 0; i < p.eltw_stride.size(); ++i) s += (i ? "," : "") + four(p.eltw_stride[i].sizes);
         s += "]";
     }
+    if (n->side_stream) s += ",\"stream\":1";
     if (n->conv)
         s += std::string(",\"kernel\":\"") + n->conv_info.kernel_name + "\",\"grid\":" + std::to_string(n->conv_info.grid)
              + ",\"ops\":" + std::to_string(n->conv_info.ops) + ",\"bytes\":" + std::to_string(n->conv_info.bytes);

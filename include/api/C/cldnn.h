@@ -63,7 +63,7 @@ typedef struct {
     uint32_t dump_custom_program;      /* accepted, no effect */
     const char* compiler_options;      /* accepted, no effect */
     const char* single_kernel_name;    /* accepted, no effect */
-    uint32_t enable_parallelisation;   /* accepted, no effect: one in-order stream */
+    uint32_t enable_parallelisation;   /* a second stream runs convolutions whose only user comes later (shortcut branches) */
     const char* engine_log;            /* accepted, no effect */
     const char* sources_dumps_dir;     /* accepted, no effect */
     int16_t priority_mode;             /* must stay disabled: one stream at default priority */

@@ -264,7 +264,9 @@ struct engine_configuration {
     std::string tuning_cache_path;
     engine_configuration(bool profiling = false, bool decorate_kernel_names = false, bool dump_custom_program = false,
                          const std::string& options = std::string(), const std::string& single_kernel = std::string(),
-                         bool primitives_parallelisation = true, const std::string& engine_log = std::string(),
+                         bool primitives_parallelisation = false /* the reference's default is true; here the second stream costs more
+                                                                    in cross-stream waits than it hides, so it is opt-in */,
+                         const std::string& engine_log = std::string(),
                          const std::string& sources_dumps_dir = std::string(),
                          priority_mode_types priority_mode = priority_mode_types::disabled,
                          throttle_mode_types throttle_mode = throttle_mode_types::disabled, bool memory_pool = true,

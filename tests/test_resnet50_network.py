@@ -136,3 +136,32 @@ def test_memory_pool_shares_buffers_without_changing_results():
     np.testing.assert_array_equal(logits[True], logits[False])
     np.testing.assert_array_equal(logits[True], run_oracle(x, params, fused=BLOCKS)["fc1000"])
     assert used[True] < 0.9 * used[False], used
+
+
+@pytest.mark.gpu
+def test_shortcut_convolutions_on_the_second_stream():
+    """engine option enable_parallelisation: a convolution whose only user comes later in the order (the projection
+    shortcut of res2a / res3a / res4a / res5a) runs on the engine's second stream beside the branch; same results, with
+    and without the memory pool, run after run"""
+    from cldnn_amd import api as cl
+    B = 2
+    params = rn.random_weights(seed=13)
+    run_oracle(np.random.default_rng(1).integers(0, 256, (B, 3, 224, 224)).astype(np.uint8), params, fused=BLOCKS, calibrate=True)
+    watch = ["res2a", "res3b", "res5a", "fc1000"]
+    xs = [np.random.default_rng(seed).integers(0, 256, (B, 3, 224, 224)).astype(np.uint8) for seed in (2, 3)]
+    refs = None
+    for pool in (True, False):
+        eng = cl.engine(enable_parallelisation=True, enable_memory_pool=pool)
+        topo = rn.topology(cl, eng, params, B)
+        opts = cl.build_options(optimize_data=True, outputs=watch)
+        if refs is None:
+            fused = [n["id"].split("_fused_")[1] for n in cl.plan(topo, opts) if "_fused_" in n["id"]]
+            refs = [run_oracle(x, params, fused=fused) for x in xs]
+        net = cl.network(eng, topo, opts)
+        side = [i for i in net.get_all_primitive_ids() if "_branch" in i and net.get_primitive_info(i).get("stream") == 1]
+        assert side == ["res2a_branch1", "res3a_branch1", "res4a_branch1", "res5a_branch1"]
+        for k in (0, 1, 0):
+            net.set_input_data("input", cl.make_memory(eng, xs[k]))
+            outs = net.execute()
+            for name in watch:
+                np.testing.assert_array_equal(outs[name].get_memory().read(), refs[k][name], err_msg="%s pool=%s input %d" % (name, pool, k))
