@@ -24,6 +24,7 @@ struct cldnn_hip_conv_s {
     void* w_packed = nullptr; // MFMA / depthwise operand stream
     void* w_masked = nullptr; // depthwise 3x3 kernel: one weight byte per dword
     void* ktab = nullptr;
+    void* gather = nullptr;   // scratch of the small-batch kernel (activations in fragment order)
     void* acc_init = nullptr;      // int32: offset correction + int32 bias
     void* acc_init_raw = nullptr;  // int32: offset correction only (accumulator probe)
     void* bias = nullptr;
@@ -245,11 +246,12 @@ void build(cldnn_hip_conv c, const void* weights, const void* bias, const float*
         mfma_pack_weights(p, c->mplan, w8, packed.data(), ktab.data());
         c->w_packed = upload(c, packed.data(), packed.size());
         c->ktab = upload(c, ktab.data(), ktab.size() * 4);
+        if (const size_t g = mfma_gather_bytes(p, c->mplan)) c->gather = upload(c, nullptr, 0, g);
         const TileConfig& tc = tile_config(tile);
         inf.tile_index = tile, inf.tile_pixels = tc.tile_pixels, inf.tile_ofm = tc.tile_ofm;
-        inf.grid = c->mplan.grid, inf.block = 256, inf.lds_bytes = c->mplan.lds_bytes;
-        std::snprintf(inf.kernel_name, sizeof(inf.kernel_name), "conv_%s<%s,%s,%s>", c->mplan.stream ? "stream" : (c->mplan.bdir ? "bdir" : (c->mplan.wsl ? "wsl" : "mfma")),
-                      tc.name, c->mplan.checked ? "checked" : "border", c->fast ? "fast" : "generic");
+        inf.grid = c->mplan.grid, inf.block = c->mplan.gemv ? 64 * c->mplan.gemv_waves : 256, inf.lds_bytes = c->mplan.lds_bytes;
+        std::snprintf(inf.kernel_name, sizeof(inf.kernel_name), "conv_%s<%s,%s,%s>", c->mplan.gemv ? "gemv" : c->mplan.stream ? "stream" : (c->mplan.bdir ? "bdir" : (c->mplan.wsl ? "wsl" : "mfma")),
+                      tc.name, c->mplan.checked ? "checked" : "border", c->fast && !c->mplan.gemv ? "fast" : "generic");
     } else {
         c->dplan = dw_plan(p);
         std::vector<int8_t> packed(c->dplan.packed_bytes);
@@ -330,7 +332,7 @@ static void run(cldnn_hip_conv c, const void* in, void* out, const void* eltw, i
         launch_conv_ref(s, p, c->epi, in, c->w_raw, eltw, out, raw);
         break;
     case CLDNN_HIP_IMPL_MFMA: {
-        MfmaBuffers wb{(const int8_t*)c->w_packed, (const int32_t*)c->ktab};
+        MfmaBuffers wb{(const int8_t*)c->w_packed, (const int32_t*)c->ktab, c->gather};
         if (raw)
             launch_conv_mfma(s, p, c->mplan, wb, (const int32_t*)c->acc_init_raw, c->epi, nullptr, in, nullptr, nullptr, raw);
         else

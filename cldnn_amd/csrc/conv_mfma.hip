@@ -16,6 +16,8 @@ void launch_bdir_f64(hipStream_t s, const MfmaArgs& a, int nt, int grid, int lds
 void launch_bdir_f128(hipStream_t s, const MfmaArgs& a, int nt, int grid, int lds, int epi);
 void launch_bdir_k2(hipStream_t s, const MfmaArgs& a, int nt, int grid, int lds, int epi);
 void launch_bdir_k4(hipStream_t s, const MfmaArgs& a, int nt, int grid, int lds, int epi);
+void launch_gemv(hipStream_t s, const MfmaArgs& a, int grid, int waves, int mtiles);
+size_t gemv_gather_bytes(int mtiles, int ksteps);
 #define DECL_WSL(d) void launch_wsl_d##d(hipStream_t s, const MfmaArgs& a, int nt, int grid, int lds, int epi);
 DECL_WSL(1) DECL_WSL(2) DECL_WSL(3) DECL_WSL(4) DECL_WSL(6) DECL_WSL(8)
 #undef DECL_WSL
@@ -51,8 +53,11 @@ static const TileConfig g_tiles[] = {
     // first layers (at most 4 input features) read b_fs_yx_fsv4: a 16-byte fragment is 4 horizontal taps x 4 features;
     // streaming kernel
     {"stem_p32", 32, 64, 32},
+    // few pixels, long K (fully_connected): a workgroup owns one 16-feature fragment of a 64-feature tile and 16
+    // pixels; its waves split K and stream both operands straight from global memory
+    {"gemv_p16_f16", 16, 64, 16},
 };
-enum { FIRST_STREAM_ROW = 6, FIRST_BDIR_ROW = 8, FIRST_WSL_ROW = 14, FIRST_BDIRK_ROW = 17, STEM_ROW = 20 };
+enum { FIRST_STREAM_ROW = 6, FIRST_BDIR_ROW = 8, FIRST_WSL_ROW = 14, FIRST_BDIRK_ROW = 17, STEM_ROW = 20, GEMV_ROW = 21 };
 enum { WSL_MAX_LDS = 160 * 1024 };
 enum { MFMA_SLACK_STEPS = 40 };  // >= weight look-ahead + activation look-ahead + 3
 static const tile_launcher g_launch[] = {launch_mfma_tile_0, launch_mfma_tile_1, launch_mfma_tile_2, launch_mfma_tile_3,
@@ -97,7 +102,7 @@ enum {
     ROW_STREAM_P16 = 6, ROW_STREAM_P32 = 7,
     ROW_BDIR_P64_F64 = 8, ROW_BDIR_P128_F64 = 9, ROW_BDIR_P256_F64 = 10, ROW_BDIR_P64_F128 = 11, ROW_BDIR_P128_F128 = 12,
     ROW_BDIR_P256_F128 = 13, ROW_WSL_P64 = 14, ROW_WSL_P128 = 15, ROW_WSL_P256 = 16,
-    ROW_BDIR_K2_P64_F64 = 17, ROW_BDIR_K4_P64_F64 = 18, ROW_BDIR_K2_P128_F64 = 19, ROW_STEM_P32 = 20
+    ROW_BDIR_K2_P64_F64 = 17, ROW_BDIR_K4_P64_F64 = 18, ROW_BDIR_K2_P128_F64 = 19, ROW_STEM_P32 = 20, ROW_GEMV = 21
 };
 
 static int choose_lds_tile(const ConvProblem& p, int64_t m, int cus)
@@ -129,6 +134,9 @@ int mfma_choose(const ConvProblem& p, int cus)
     const bool stream_fits = border && ksteps <= 8 && stream_waves * 2 >= 4ll * cus;
     const int stream_row = stream_waves >= 4ll * cus ? ROW_STREAM_P32 : ROW_STREAM_P16;
 
+    // a fragment or two of pixels and a long K (fully_connected): the weights are the traffic and the tile kernels
+    // would occupy one workgroup per 64 features
+    if (direct && m <= 32 && ksteps >= 16) return ROW_GEMV;
     if (ksteps <= 2 || !direct) {
         // one or two K-steps (or a first layer with three input features): bound by HBM bandwidth
         if (!direct && ksteps >= 3 && m >= 500000) return choose_lds_tile(p, m, cus);  // VGG conv1
@@ -190,14 +198,15 @@ MfmaPlan mfma_plan(const ConvProblem& p, int tile, int cus)
     CHIP_REQUIRE(pl.stem == (p.in_t.format == CLDNN_HIP_FMT_B_FS_YX_FSV4 ? 1 : 0), CLDNN_HIP_INVALID_ARG,
                  "b_fs_yx_fsv4 input goes with the first-layer row of the tile table and only with it");
     pl.stream = (tile >= FIRST_STREAM_ROW && tile < FIRST_BDIR_ROW) || pl.stem ? 1 : 0;
-    pl.bdir = ((tile >= FIRST_BDIR_ROW && tile < FIRST_WSL_ROW) || tile >= FIRST_BDIRK_ROW) && !pl.stem ? 1 : 0;
+    pl.gemv = tile == GEMV_ROW ? 1 : 0;
+    pl.bdir = ((tile >= FIRST_BDIR_ROW && tile < FIRST_WSL_ROW) || tile >= FIRST_BDIRK_ROW) && !pl.stem && !pl.gemv ? 1 : 0;
     pl.wsl = tile >= FIRST_WSL_ROW && tile < FIRST_BDIRK_ROW ? 1 : 0;
     CHIP_REQUIRE(!(pl.stream && pl.checked), CLDNN_HIP_INVALID_ARG,
                  "the streaming kernel needs an input whose physical zero border covers the convolution's padding");
     pl.cb = (p.IFM + 15) / 16;
     if (pl.stem) CHIP_REQUIRE(p.IFM <= 4 && p.dx == 1 && p.groups == 1, CLDNN_HIP_INVALID_ARG,
                               "the first-layer kernel takes at most 4 input features and no horizontal dilation");
-    CHIP_REQUIRE(!(pl.bdir || pl.wsl) || (!pl.checked && pl.cb % 4 == 0), CLDNN_HIP_INVALID_ARG,
+    CHIP_REQUIRE(!(pl.bdir || pl.wsl || pl.gemv) || (!pl.checked && pl.cb % 4 == 0), CLDNN_HIP_INVALID_ARG,
                  "the direct-activation kernels need a zero border covering the padding and input features in multiples of 64");
     pl.kchunks = pl.stem ? p.FY * ((p.FX + 3) / 4) : p.FY * p.FX * pl.cb;  // first layer: a chunk is 4 horizontal taps
     pl.ksteps = (pl.kchunks + 3) / 4;
@@ -223,7 +232,7 @@ MfmaPlan mfma_plan(const ConvProblem& p, int tile, int cus)
     pl.mtiles = (int)((pl.m_total + tc.tile_pixels - 1) / tc.tile_pixels);
     // which operand do the eight dies share out?  the larger one (it is then read from memory once, not 8 times)
     const int64_t w_bytes = (int64_t)p.OFM * (p.IFM / p.groups) * p.FY * p.FX, in_bytes = (int64_t)p.B * p.IFM * p.IH * p.IW;
-    pl.by_features = !pl.stream && !pl.wsl && w_bytes > in_bytes && (p.OFM + tc.tile_ofm - 1) / tc.tile_ofm >= 8 ? 1 : 0;
+    pl.by_features = !pl.stream && !pl.wsl && !pl.gemv && w_bytes > in_bytes && (p.OFM + tc.tile_ofm - 1) / tc.tile_ofm >= 8 ? 1 : 0;
     int64_t grid = pl.by_features ? (int64_t)((pl.ofm_tiles + 7) / 8) * 8 * pl.mtiles : (int64_t)((pl.mtiles + 7) / 8) * 8 * pl.ofm_tiles;
     if (pl.stream) grid = ((int64_t)pl.mtiles * pl.ofm_tiles + 3) / 4;  // one wave per (pixel tile, span)
     pl.lds_bytes = pl.stream ? 0 : (pl.bdir ? 3 * 4 * tc.tile_ofm * 16 : 2 * 4 * (tc.tile_ofm + tc.tile_pixels) * 16);
@@ -239,6 +248,12 @@ MfmaPlan mfma_plan(const ConvProblem& p, int tile, int cus)
         parts = ((pl.mtiles + pl.wsl_tpp - 1) / pl.wsl_tpp + 7) / 8 * 8;
         pl.wsl_parts = parts;
         grid = (int64_t)parts * pl.ofm_tiles;
+    }
+    if (pl.gemv) {
+        // one workgroup per 16-feature fragment and 16 pixels; 4, 8 or 16 waves split K, at least four steps each
+        grid = (int64_t)pl.mtiles * pl.ofm_tiles * 4;
+        pl.gemv_waves = pl.ksteps >= 64 ? 16 : (pl.ksteps >= 32 ? 8 : 4);
+        pl.lds_bytes = 16 * 1024;
     }
     CHIP_REQUIRE(grid < (1ll << 31), CLDNN_HIP_UNSUPPORTED_SIZE, "convolution too large for one launch");
     pl.grid = (int)grid;
@@ -382,6 +397,12 @@ bool mfma_fast_epilogue(const ConvProblem& p, const Epilogue& e, const float* ca
     return true;
 }
 
+// a filter of one tap puts the 16 pixels' bytes of a K-step side by side already
+size_t mfma_gather_bytes(const ConvProblem& p, const MfmaPlan& pl)
+{
+    return pl.gemv && p.FY * p.FX > 1 ? gemv_gather_bytes(pl.mtiles, pl.ksteps) : 0;
+}
+
 void launch_conv_mfma(hipStream_t s, const ConvProblem& p, const MfmaPlan& pl, const MfmaBuffers& wb,
                       const int32_t* acc_init, const Epilogue& epi, const FastEpi* fast, const void* in, const void* eltw,
                       void* out, int32_t* raw)
@@ -442,7 +463,9 @@ void launch_conv_mfma(hipStream_t s, const ConvProblem& p, const MfmaPlan& pl, c
             if (fast->fused && fast->act == CLDNN_HIP_ACT_NONE && fast->eltw_relu_folded && epi.eltw_calib) kind = EPI_KIND_FUSED;
         }
     }
-    if (pl.stream) launch_stream(s, a, tc.wave_pixels / 16, pl.grid, kind);
+    a.bpk = (const v4i*)wb.gather;
+    if (pl.gemv) launch_gemv(s, a, pl.grid, pl.gemv_waves, pl.mtiles);  // element-wise epilogue only
+    else if (pl.stream) launch_stream(s, a, tc.wave_pixels / 16, pl.grid, kind);
     else if (pl.bdir && tc.kgroups == 2) launch_bdir_k2(s, a, tc.wave_pixels / 16, pl.grid, pl.lds_bytes, kind);
     else if (pl.bdir && tc.kgroups == 4) launch_bdir_k4(s, a, tc.wave_pixels / 16, pl.grid, pl.lds_bytes, kind);
     else if (pl.bdir && tc.tile_ofm == 64) launch_bdir_f64(s, a, tc.wave_pixels / 16, pl.grid, pl.lds_bytes, kind);

@@ -69,6 +69,7 @@ struct MfmaArgs {
     int32_t px_bytes;
     FastDiv div_cb, div_fx;
     uint32_t xor_mask;  // 0x80808080 for u8 activations, 0 for s8
+    const v4i* bpk;     // small-batch kernel: scratch for the activations in fragment order (nullptr: read them in place)
     FastEpi fe;
     Epilogue epi;
 };

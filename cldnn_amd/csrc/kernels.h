@@ -46,6 +46,8 @@ struct MfmaPlan {
     int wsl_depth;       // its activation look-ahead in K-steps
     int wsl_parts;       // pixel-range partitions per feature tile (multiple of 8)
     int wsl_tpp;         // pixel tiles per partition
+    int gemv;            // 1: few pixels, long K: 16-feature fragments, waves split K (no LDS in the loop)
+    int gemv_waves;      // its waves per workgroup
     int checked;         // 1: taps bounds-checked per load, 0: input carries a sufficient zero border
     int tap_minor;       // K order: 1 = (group of 4 slices, tap), taps innermost; 0 = (tap, slice)
     int cb;              // input feature slices of 16
@@ -67,7 +69,9 @@ void mfma_pack_weights(const ConvProblem& p, const MfmaPlan& plan, const int8_t*
 struct MfmaBuffers {
     const int8_t* packed;
     const int32_t* ktab;
+    void* gather = nullptr;  // small-batch kernel with a filter wider than one tap: mfma_gather_bytes() of scratch
 };
+size_t mfma_gather_bytes(const ConvProblem& p, const MfmaPlan& pl);  // 0 when the plan needs no scratch
 // parameters of the short epilogue (int8 output, float requantisation)
 struct FastEpi {
     int32_t has_wqf;      // multiply by wqf[f] and iqf

@@ -211,13 +211,13 @@ def test_mfma_kernel_all_tiles(eng, shape, in_dt):
                 with pytest.raises(hip.HipError):  # the first-layer row goes with b_fs_yx_fsv4 input
                     hip.conv_forward(eng, x, w, bias, wqf, calib, **kw)
                 continue
-            if tile and names[tile - 1].startswith(("bdir", "wsl")) and (no_border or -(-IFM // 16) % 4 != 0):
+            if tile and names[tile - 1].startswith(("bdir", "wsl", "gemv")) and (no_border or -(-IFM // 16) % 4 != 0):
                 with pytest.raises(hip.HipError):  # needs constant tap offsets and feature slices in fours
                     hip.conv_forward(eng, x, w, bias, wqf, calib, **kw)
                 continue
             go, ga, info = hip.conv_forward(eng, x, w, bias, wqf, calib, **kw)
             name = info.kernel_name.decode()
-            assert info.impl == hip.IMPL_MFMA and "fast" in name, name
+            assert info.impl == hip.IMPL_MFMA and ("fast" in name or "gemv" in name), name  # the small-batch kernel has one epilogue
             seen.add(name)
             np.testing.assert_array_equal(ga, ref_a, err_msg=name)
             assert_same(ref_o, go)
@@ -246,6 +246,36 @@ def test_mfma_epilogue_variants(eng, out_dt, act):
         assert tile == 0 or b"bdir" in info.kernel_name or b"wsl" in info.kernel_name
         np.testing.assert_array_equal(ga, ra)
         assert_same(ro, go)
+
+
+@pytest.mark.parametrize("in_dt", [np.uint8, np.int8], ids=["u8", "s8"])
+@pytest.mark.parametrize("shape", [(5, 64, 7, 7, 70, 7, 7, 0), (20, 256, 1, 1, 200, 1, 1, 0), (3, 64, 4, 4, 96, 3, 3, 0), (2, 128, 3, 3, 64, 3, 3, 1),
+                                   (16, 512, 7, 7, 128, 7, 7, 0)],
+                         ids=["plane7x7_b5", "1x1_b20", "3x3_out2x2", "3x3_padded", "vgg_fc6_slice"])
+def test_small_batch_kernel(eng, shape, in_dt):
+    """few output pixels, long K: 16-feature fragments, the waves of a workgroup split K; a filter wider than one tap
+    gathers the activations into fragment order first.  Every output type and activation, the residual sum, the raw
+    accumulators; pixel counts and feature counts that do not fill the fragments."""
+    B, IFM, H, W, OFM, FY, FX, pad = shape
+    x, w, bias, wqf, calib = problem(31, B, IFM, H, W, OFM, FY, FX, in_dt)
+    gemv = tile_names().index("gemv_p16_f16") + 1
+    OH, OW = H + 2 * pad - FY + 1, W + 2 * pad - FX + 1
+    r = np.random.default_rng(8)
+    for out_dt, act in (("s8", ("relu", 0, 0)), ("u8", ("none", 0, 0)), ("f32", ("relu_slope", 0.1, 0)), ("s8", ("clamp", -20.0, 90.0))):
+        kw = dict(stride=(1, 1), pad=(pad, pad), out_dt=out_dt, act=act[0], act_m=act[1], act_n=act[2], iqf=0.75)
+        (ro, ra), (go, ga, info) = both(eng, x, w, bias, wqf, calib, fmt="fs_b_yx_fsv16", tile=gemv, in_pad=(pad, pad), **kw)
+        assert b"conv_gemv" in info.kernel_name and info.grid == -(-B * OH * OW // 16) * -(-OFM // 64) * 4
+        np.testing.assert_array_equal(ga, ra)
+        assert_same(ro, go)
+    e = r.integers(-128, 128, (B, OFM, OH, OW)).astype(np.int8)
+    ecal = r.uniform(0.3, 1.2, OFM).astype(np.float32)
+    kw = dict(stride=(1, 1), pad=(pad, pad), out_dt="s8", act="none", eltw=e, eltw_act="relu", eltw_calib=ecal)
+    (ro, ra), (go, ga, info) = both(eng, x, w, bias, wqf, calib, fmt="fs_b_yx_fsv16", tile=gemv, in_pad=(pad, pad), **kw)
+    assert b"conv_gemv" in info.kernel_name
+    assert_same(ro, go)
+    # the table picks it by itself from 16 K-steps (K = 1024) on when at most 32 pixels come out
+    _, _, info = hip.conv_forward(eng, x, w, bias, wqf, calib, fmt="fs_b_yx_fsv16", in_pad=(pad, pad), pad=(pad, pad), out_dt="s8", want_acc=True, want_info=True)
+    assert (b"conv_gemv" in info.kernel_name) == (B * OH * OW <= 32 and IFM * FY * FX >= 1024), info.kernel_name
 
 
 def test_mfma_f32_bias_added_after_dequantisation(eng):
@@ -279,7 +309,7 @@ def test_mfma_fused_eltwise(eng, fast, eltw_dt):
               non_conv_scale=1.0 if fast else 0.5)
     for tile in [0] + [t for t in tiles() if not tile_names()[t - 1].startswith("stem")]:
         (ro, ra), (go, ga, info) = both(eng, x, w, bias, wqf, calib, fmt="fs_b_yx_fsv16", tile=tile, **kw)
-        assert (b"fast" in info.kernel_name) == fast
+        assert (b"fast" in info.kernel_name) == (fast and b"gemv" not in info.kernel_name)  # the small-batch kernel has one epilogue
         np.testing.assert_array_equal(ga, ra)
         assert_same(ro, go)
     np.testing.assert_array_equal(ga, ra)
