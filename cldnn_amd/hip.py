@@ -473,10 +473,12 @@ def conv_forward(engine, x, w, bias=None, wqf=None, calib=None, *, stride=(1, 1)
                  groups=1, out_dt=None, iqf=1.0, oqf=1.0, act="none", act_m=0.0, act_n=0.0, eltw=None,
                  non_conv_scale=1.0, eltw_act="none", eltw_m=0.0, eltw_n=0.0, eltw_calib=None, eltw_stride=(1, 1),
                  round_even=False, fmt="bfyx", in_pad=(0, 0), out_pad=(0, 0), impl=IMPL_AUTO, tile=0,
-                 want_acc=False, want_info=False, pad_end=None, fc=False):
+                 want_acc=False, want_info=False, pad_end=None, fc=False, in_place=False):
     """numpy in, numpy out: upload (reordering to `fmt`), run the HIP convolution, download.
 
-    Argument meaning follows oracle.refconv.conv so that parity tests can call both alike.
+    Argument meaning follows oracle.refconv.conv so that parity tests can call both alike.  in_place: the residual
+    operand `eltw` (of the output's type and size) is put into the output buffer and read from there
+    (second_input_in_output).
     """
     x = np.ascontiguousarray(x)
     w = np.ascontiguousarray(w)
@@ -486,7 +488,7 @@ def conv_forward(engine, x, w, bias=None, wqf=None, calib=None, *, stride=(1, 1)
     e_buf = None
     # a first layer reads b_fs_yx_fsv4 and writes the blocked layout the rest of the network runs in
     first_layer = FMT_NAME.get(fmt, fmt) == B_FS_YX_FSV4
-    if eltw is not None:
+    if eltw is not None and not in_place:
         e_buf = upload(engine, np.ascontiguousarray(eltw), "fs_b_yx_fsv16" if first_layer else fmt)
     bias_dt = NO_TYPE if bias is None else DT_OF[np.asarray(bias).dtype]
     d = conv_desc(xin.tensor, w.shape, out_dt, stride=stride, pad=pad, dilation=dilation, groups=groups,
@@ -494,9 +496,13 @@ def conv_forward(engine, x, w, bias=None, wqf=None, calib=None, *, stride=(1, 1)
                   has_calib=calib is not None, iqf=iqf, oqf=oqf, act=act, act_m=act_m, act_n=act_n,
                   eltw_t=None if e_buf is None else e_buf.tensor, non_conv_scale=non_conv_scale, eltw_act=eltw_act,
                   eltw_m=eltw_m, eltw_n=eltw_n, has_eltw_calib=eltw_calib is not None, eltw_stride=eltw_stride,
-                  round_even=round_even, impl=impl, tile=tile, pad_end=pad_end, fc=fc)
+                  round_even=round_even, impl=impl, tile=tile, pad_end=pad_end, fc=fc, in_place=in_place)
     c = Conv(engine, d, w, bias, wqf, calib, eltw_calib)
-    out = Buffer(engine, d.output)
+    if in_place:
+        out = upload(engine, np.ascontiguousarray(eltw), "fs_b_yx_fsv16" if first_layer else fmt, out_pad)
+        assert bytes(out.tensor) == bytes(d.output), "the residual must have the output's type, size and padding"
+    else:
+        out = Buffer(engine, d.output)
     c.enqueue(xin, out, e_buf)
     res = [download(engine, out)]
     if want_acc:

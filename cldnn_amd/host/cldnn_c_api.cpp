@@ -692,7 +692,9 @@ cldnn_network cldnn_allocate_network(cldnn_program program, cldnn_status* status
         for (size_t i = 0; i < program->nodes.size(); ++i) {
             node* n = program->nodes[i].get();
             index[n] = i;
-            if (n->p->type == prim_type::fused_conv_eltwise && n->p->second_input_in_output) aliasing = true;
+            // asked for by the application: anything may alias, the pool stays out of it.  Set by the read/write
+            // pass: the pool follows the buffer through the chain (below)
+            if (n->p->type == prim_type::fused_conv_eltwise && n->p->second_input_in_output && !n->rw_opt) aliasing = true;
         }
         for (auto& u : program->nodes)
             for (node* d : u->deps) last_use[d] = std::max(last_use[d], index[u.get()]);
@@ -716,6 +718,9 @@ cldnn_network cldnn_allocate_network(cldnn_program program, cldnn_status* status
             }
             if (n->p->type == prim_type::fused_conv_eltwise && n->p->second_input_in_output) {
                 net->mem[n] = net->mem[n->deps[1]];
+                // the buffer now holds this tensor: it stays reserved until this tensor's last reader
+                for (auto& f : in_flight)
+                    if (f.second.get() == net->mem[n].get() && last_use.count(n)) f.first = std::max(f.first, last_use[n]);
                 continue;
             }
             // buffers whose tensors nobody reads at or after this primitive become idle

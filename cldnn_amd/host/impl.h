@@ -162,6 +162,7 @@ struct node {
     std::vector<node*> deps;        // data dependencies in primitive order (input, [input2], weights, bias, wqf, calib, [eltw calib])
     std::vector<node*> users;
     bool side_stream = false;       // runs on the engine's second stream, joined before its only user
+    bool rw_opt = false;            // fused_conv_eltwise made to write over its second input by the read/write pass
     cldnn_layout out{};             // output layout incl. physical padding
     int32_t user_format = cldnn_format_any;  // output format before the layout pass (what the topology implies)
     bool is_output = false;

@@ -278,6 +278,43 @@ def test_small_batch_kernel(eng, shape, in_dt):
     assert (b"conv_gemv" in info.kernel_name) == (B * OH * OW <= 32 and IFM * FY * FX >= 1024), info.kernel_name
 
 
+@pytest.mark.parametrize("out_dt,e_dt", [("s8", np.int8), ("u8", np.uint8), ("f32", np.float32)], ids=["s8", "u8", "f32"])
+def test_residual_read_from_the_output_buffer(eng, out_dt, e_dt):
+    """second_input_in_output (reference fused_conv_eltwise_gpu.cpp:92-121): the residual operand already sits in the
+    output buffer and every result replaces the value it was summed with; same numbers as with a separate operand,
+    on every kernel family and on the plain-layout and depthwise kernels"""
+    r = np.random.default_rng(12)
+    def residual(shape):
+        if e_dt == np.float32:
+            return r.integers(-128, 128, shape).astype(np.float32)
+        lo, hi = (-128, 128) if e_dt == np.int8 else (0, 256)
+        return r.integers(lo, hi, shape).astype(e_dt)
+    x, w, bias, wqf, calib = problem(41, 2, 64, 14, 14, 128, 1, 1)
+    e = residual((2, 128, 14, 14))
+    ecal = r.uniform(0.3, 1.2, 128).astype(np.float32)
+    kw = dict(out_dt=out_dt, act="none", eltw=e, eltw_act="relu", eltw_calib=ecal)
+    ref = rc.conv(x, w, bias, wqf=wqf, calib=calib, **kw)
+    seen = set()
+    for tile in [0] + [t for t in tiles() if not tile_names()[t - 1].startswith("stem")]:
+        out, info = hip.conv_forward(eng, x, w, bias, wqf, calib, fmt="fs_b_yx_fsv16", tile=tile, in_place=True, want_info=True, **kw)
+        seen.add(info.kernel_name.decode().split("<")[0])
+        assert_same(ref, out)
+    assert {"conv_mfma", "conv_stream", "conv_bdir", "conv_wsl", "conv_gemv"} <= seen, seen
+    out = hip.conv_forward(eng, x, w, bias, wqf, calib, fmt="bfyx", in_place=True, **kw)  # layout-agnostic kernel
+    assert_same(ref, out)
+    # 3x3 with padding (a second input as large as the output, not as the input), and depthwise
+    x, w, bias, wqf, calib = problem(42, 2, 64, 9, 9, 64, 3, 3)
+    e = residual((2, 64, 9, 9))
+    kw = dict(out_dt=out_dt, pad=(1, 1), act="none", eltw=e, eltw_act="relu", eltw_calib=ecal[:64])
+    assert_same(rc.conv(x, w, bias, wqf=wqf, calib=calib, **kw), hip.conv_forward(eng, x, w, bias, wqf, calib, fmt="fs_b_yx_fsv16", in_pad=(1, 1), in_place=True, **kw))
+    x, w, bias, wqf, calib = problem(43, 2, 32, 9, 9, 32, 3, 3, groups=32)
+    e = residual((2, 32, 9, 9))
+    kw = dict(out_dt=out_dt, pad=(1, 1), groups=32, act="none", eltw=e, eltw_act="relu", eltw_calib=ecal[:32])
+    out, info = hip.conv_forward(eng, x, w, bias, wqf, calib, fmt="fs_b_yx_fsv16", in_pad=(1, 1), in_place=True, want_info=True, **kw)
+    assert b"conv_dw" in info.kernel_name
+    assert_same(rc.conv(x, w, bias, wqf=wqf, calib=calib, **kw), out)
+
+
 def test_mfma_f32_bias_added_after_dequantisation(eng):
     x, w, _, wqf, calib = problem(14, 1, 32, 8, 8, 32, 3, 3, np.int8)
     bias = np.random.default_rng(1).uniform(-50, 50, 32).astype(np.float32)

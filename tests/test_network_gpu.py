@@ -367,6 +367,45 @@ def test_fused_and_unfused_graphs_agree(eng):
     np.testing.assert_array_equal(outs[0], outs[1])
 
 
+def test_closer_writes_over_its_shortcut_without_a_memory_pool():
+    """prepare_conv_eltw_read_write_opt (reference prepare_primitive_fusing.cpp:468-534): the fused closer of a block whose
+    shortcut is an intermediate tensor of the same layout, read by nothing later, takes the shortcut's buffer as its
+    output.  Applied on engines without a memory pool; same numbers either way, over repeated runs."""
+    r = np.random.default_rng(21)
+    B, C, M, H, W = 2, 64, 32, 10, 12
+    x = r.integers(-128, 128, (B, C, H, W)).astype(np.int8)
+    L = [rand_layer(r, C, C, 1, False), rand_layer(r, M, C, 1, False), rand_layer(r, M, M, 3, False), rand_layer(r, C, M, 1, False)]
+    ecal = r.uniform(0.4, 0.9, C).astype(np.float32)
+    results = {}
+    for pool in (False, True):
+        e = cl.engine(enable_memory_pool=pool)
+        prims = [cl.input_layout("input", cl.layout(DT.i8, F.bfyx, cl.tensor(B, C, W, H))), cl.data("ecal", vec_mem(e, ecal))]
+        for i, (w, b, q, c) in enumerate(L):
+            prims += [cl.data(f"w{i}", cl.make_memory(e, w)), cl.data(f"b{i}", vec_mem(e, b)), cl.data(f"q{i}", vec_mem(e, q)), cl.data(f"c{i}", vec_mem(e, c))]
+        prims += [cl.convolution("shortcut", "input", ["w0"], ["b0"], ["q0"], ["c0"], with_activation=True),
+                  cl.convolution("reduce", "shortcut", ["w1"], ["b1"], ["q1"], ["c1"], with_activation=True),
+                  cl.convolution("mid", "reduce", ["w2"], ["b2"], ["q2"], ["c2"], input_offset=cl.tensor(0, 0, -1, -1, 0), with_activation=True),
+                  cl.convolution("expand", "mid", ["w3"], ["b3"], ["q3"], ["c3"], output_data_type=DT.i8),
+                  cl.eltwise("sum", "shortcut", "expand", cl.eltwise_mode.sum, True, 0.0, output_calibration_factors="ecal"),
+                  cl.pooling("pool", "sum", cl.pooling_mode.max, cl.tensor(1, 1, 2, 2), cl.tensor(1, 1, 2, 2))]
+        net = cl.network(e, cl.topology(*prims), cl.build_options(optimize_data=True))
+        info = net.get_primitive_info("expand_fused_sum")
+        assert bool(info.get("second_input_in_output")) == (not pool)
+        for k in range(3):
+            xk = np.roll(x, k, axis=3)
+            net.set_input_data("input", cl.make_memory(e, xk))
+            results[pool, k] = net.execute()["pool"].get_memory().read()
+    for k in range(3):
+        xk = np.roll(x, k, axis=3)
+        s = rc.conv(xk, L[0][0], L[0][1], wqf=L[0][2], calib=L[0][3], out_dt="s8", act="relu")
+        a = rc.conv(s, L[1][0], L[1][1], wqf=L[1][2], calib=L[1][3], out_dt="s8", act="relu")
+        a = rc.conv(a, L[2][0], L[2][1], wqf=L[2][2], calib=L[2][3], pad=(1, 1), out_dt="s8", act="relu")
+        a = rc.conv(a, L[3][0], L[3][1], wqf=L[3][2], calib=L[3][3], out_dt="s8", eltw=s, eltw_act="relu", eltw_calib=ecal)
+        ref = rc.pool(a, "max", (2, 2), stride=(2, 2))
+        np.testing.assert_array_equal(results[False, k], ref)
+        np.testing.assert_array_equal(results[True, k], ref)
+
+
 def test_network_runs_again_with_new_input(eng):
     topo, x, _ = bottleneck(eng, 3)
     net = cl.network(eng, topo, cl.build_options(optimize_data=True))

@@ -128,6 +128,12 @@ def test_memory_pool_shares_buffers_without_changing_results():
         eng = cl.engine(enable_memory_pool=pool)
         base = eng.get_temp_used_device_memory_size()
         net = cl.network(eng, rn.topology(cl, eng, params, B), cl.build_options(optimize_data=True))
+        # without a pool the read / write pass (reference prepare_primitive_fusing.cpp:468-534) lets a fused closer write
+        # over its shortcut when the two have one layout and nothing reads the shortcut later: every block but the
+        # three whose sum was shrunk to the stride of the block behind it
+        in_place = sorted(i.split("_fused_")[1] for i in net.get_all_primitive_ids()
+                          if "_fused_" in i and net.get_primitive_info(i).get("second_input_in_output"))
+        assert in_place == ([] if pool else sorted(b for b in BLOCKS if b not in ("res2c", "res3d", "res4f"))), in_place
         net.set_input_data("input", cl.make_memory(eng, x))
         for _ in range(2):  # a second run reuses the same buffers
             logits[pool] = net.execute()["fc1000"].get_memory().read()
@@ -135,7 +141,8 @@ def test_memory_pool_shares_buffers_without_changing_results():
         del net
     np.testing.assert_array_equal(logits[True], logits[False])
     np.testing.assert_array_equal(logits[True], run_oracle(x, params, fused=BLOCKS)["fc1000"])
-    assert used[True] < 0.9 * used[False], used
+    # 26 MB of either figure are weights; without a pool the 13 closers that write over their shortcuts save nearly as much
+    assert used[True] < used[False] < 40e6, used
 
 
 @pytest.mark.gpu
