@@ -69,12 +69,14 @@ __global__ void __launch_bounds__(1024) conv_gemv_kernel(MfmaArgs a)
         else xb = *reinterpret_cast<const v4i*>(a.in + scalar_table_load(a.ktab, ks * 4) + boff);
     };
     // The loop is branch-free (a branch around a matrix instruction makes the compiler wait for every outstanding
-    // load at the join).  Steps past the end of the wave's range belong to the next wave or to the zero-weight slack:
-    // they are loaded, and multiplied with zeroed activations.
+    // load at the join, and a skipped load would break the counting of outstanding loads the waits rely on).  Steps
+    // past the end of the wave's range load the range's last step again (a hit in the L1) and are multiplied with
+    // zeroed activations.
     // (the fences pin the order of the loads: the waits in the loop count on step d's loads being issued before step d+1's)
+    const int last = s1 > s0 ? s1 - 1 : s0;  // a wave without steps reads one step of the slack or of its neighbour
 #pragma unroll
     for (int d = 0; d < GEMV_D; ++d) {
-        load(s0 + d, ra[d], rb[d]);
+        load(s0 + d < last ? s0 + d : last, ra[d], rb[d]);
         step_fence();
     }
     for (int ks = s0; ks < s1; ks += GEMV_D) {
@@ -83,7 +85,7 @@ __global__ void __launch_bounds__(1024) conv_gemv_kernel(MfmaArgs a)
             const int keep = ks + u < s1 ? -1 : 0;
             const v4i km = {keep, keep, keep, keep};
             acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(ra[u], (rb[u] ^ xm) & km, acc, 0, 0, 0);
-            load(ks + u + GEMV_D, ra[u], rb[u]);
+            load(ks + u + GEMV_D < last ? ks + u + GEMV_D : last, ra[u], rb[u]);
             step_fence();
         }
     }

@@ -250,9 +250,10 @@ MfmaPlan mfma_plan(const ConvProblem& p, int tile, int cus)
         grid = (int64_t)parts * pl.ofm_tiles;
     }
     if (pl.gemv) {
-        // one workgroup per 16-feature fragment and 16 pixels; 4, 8 or 16 waves split K, at least four steps each
+        // one workgroup per 16-feature fragment and 16 pixels; 4, 8 or 16 waves split K, at least eight steps (one
+        // look-ahead window) each
         grid = (int64_t)pl.mtiles * pl.ofm_tiles * 4;
-        pl.gemv_waves = pl.ksteps >= 64 ? 16 : (pl.ksteps >= 32 ? 8 : 4);
+        pl.gemv_waves = pl.ksteps >= 128 ? 16 : (pl.ksteps >= 64 ? 8 : 4);
         pl.lds_bytes = 16 * 1024;
     }
     CHIP_REQUIRE(grid < (1ll << 31), CLDNN_HIP_UNSUPPORTED_SIZE, "convolution too large for one launch");
