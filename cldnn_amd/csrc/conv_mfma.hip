@@ -149,7 +149,7 @@ int mfma_choose(const ConvProblem& p, int cus)
             if (p.OFM >= 512) return ksteps <= 4 ? ROW_WSL_P128 : ROW_BDIR_P128_F128;  // 14x14 expansions / projections
             return stream_fits ? stream_row : ROW_BDIR_P64_F64;
         }
-        if (p.OFM >= 1024) return ROW_P64_F128;                   // 7x7 expansions
+        if (p.OFM >= 1024 && m >= 512) return ROW_P64_F128;       // 7x7 expansions; at a few hundred pixels 64-feature tiles give more workgroups
         return stream_fits ? stream_row : ROW_BDIR_P64_F64;
     }
     // long K
@@ -163,7 +163,7 @@ int mfma_choose(const ConvProblem& p, int cus)
     }
     if (m >= 4096) return ROW_BDIR_P64_F64;                        // 14x14
     if (ksteps >= 32) return m >= 2048 ? ROW_BDIR_K2_P128_F64 : ROW_BDIR_K2_P64_F64;  // few pixels, K >= 2048: split K
-    if (p.OFM >= 1024) return ROW_P128_F128;
+    if (p.OFM >= 1024 && m >= 512) return ROW_P128_F128;
     return ROW_BDIR_P64_F64;
 }
 
