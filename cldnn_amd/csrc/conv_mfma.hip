@@ -228,6 +228,8 @@ MfmaPlan mfma_plan(const ConvProblem& p, int tile, int cus)
     pl.tap_minor = !pl.stream && !pl.wsl && pl.cb % 4 == 0 && p.FY * p.FX > 1 ? 1 : 0;
     pl.ofm_tiles = (p.OFM + tc.tile_ofm - 1) / tc.tile_ofm;
     pl.m_total = (int64_t)p.B * p.OH * p.OW;
+    // every 16 pixels stream all the weights again (and take 1 KB of scratch per K-step when gathered)
+    CHIP_REQUIRE(!pl.gemv || pl.m_total <= 4096, CLDNN_HIP_INVALID_ARG, "the small-batch kernel takes at most 4096 output pixels");
     CHIP_REQUIRE(pl.m_total < (1ll << 31), CLDNN_HIP_UNSUPPORTED_SIZE, "more than 2^31 output pixels");
     pl.mtiles = (int)((pl.m_total + tc.tile_pixels - 1) / tc.tile_pixels);
     // which operand do the eight dies share out?  the larger one (it is then read from memory once, not 8 times)

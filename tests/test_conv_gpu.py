@@ -273,6 +273,10 @@ def test_small_batch_kernel(eng, shape, in_dt):
     (ro, ra), (go, ga, info) = both(eng, x, w, bias, wqf, calib, fmt="fs_b_yx_fsv16", tile=gemv, in_pad=(pad, pad), **kw)
     assert b"conv_gemv" in info.kernel_name
     assert_same(ro, go)
+    if shape == (20, 256, 1, 1, 200, 1, 1, 0):  # every 16 pixels stream the weights again: the row refuses more than 4096 pixels
+        xb, wb, bb, qb, cb = problem(32, 2, 64, 56, 56, 64, 1, 1, in_dt)
+        with pytest.raises(hip.HipError):
+            hip.conv_forward(eng, xb, wb, bb, qb, cb, fmt="fs_b_yx_fsv16", tile=gemv, out_dt="s8")
     # the table picks it by itself from 16 K-steps (K = 1024) on when at most 32 pixels come out
     _, _, info = hip.conv_forward(eng, x, w, bias, wqf, calib, fmt="fs_b_yx_fsv16", in_pad=(pad, pad), pad=(pad, pad), out_dt="s8", want_acc=True, want_info=True)
     assert (b"conv_gemv" in info.kernel_name) == (B * OH * OW <= 32 and IFM * FY * FX >= 1024), info.kernel_name
