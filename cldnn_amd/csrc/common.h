@@ -70,6 +70,7 @@ struct Epilogue {
     int32_t out_dt, eltw_dt, in_dt;
     int32_t round_even;
     int32_t fc;              // quantized fully_connected form (see cldnn_hip_conv_desc.fully_connected)
+    int32_t conv_sat;        // fused form: 1 / 2 = the rounded convolution result is saturated to s8 / u8 before the sum
 };
 
 }  // namespace chip

@@ -144,6 +144,9 @@ void build(cldnn_hip_conv c, const void* weights, const void* bias, const float*
     e.out_dt = p.out_dt, e.eltw_dt = p.eltw_dt, e.in_dt = p.in_dt;
     e.round_even = d.round_to_even;
     e.fc = (d.fully_connected && d.has_wqf && !d.fused) ? 1 : 0;
+    CHIP_REQUIRE(d.conv_saturate >= 0 && d.conv_saturate <= 2 && (!d.conv_saturate || (d.fused && d.has_wqf)), CLDNN_HIP_INVALID_ARG,
+                 "conv_saturate is 0, 1 (s8) or 2 (u8) and goes with the quantized fused form");
+    e.conv_sat = d.conv_saturate;
     if (e.fc) {
         CHIP_REQUIRE(p.OH == 1 && p.OW == 1 && p.FY == p.IH && p.FX == p.IW && p.py == 0 && p.px == 0, CLDNN_HIP_INVALID_ARG,
                      "fully_connected: the filter must cover the whole input plane");

@@ -370,6 +370,8 @@ bool mfma_fast_epilogue(const ConvProblem& p, const Epilogue& e, const float* ca
             return false;
         if (!tame(&e.eltw_m, 1) || !tame(&e.eltw_n, 1)) return false;
         F.eltw_act = e.eltw_act, F.eltw_m = e.eltw_m, F.eltw_n = e.eltw_n;
+        F.conv_sat = e.conv_sat ? 1 : 0;
+        F.conv_lo = e.conv_sat == 1 ? -128.0f : 0.0f, F.conv_hi = e.conv_sat == 1 ? 127.0f : 255.0f;
         F.has_ecal = ecal ? 1 : 0;
         F.eltw_u8 = e.eltw_dt == CLDNN_HIP_U8;
         if (e.eltw_act == CLDNN_HIP_ACT_CLAMP && !(e.eltw_m <= e.eltw_n)) return false;
@@ -463,7 +465,8 @@ void launch_conv_mfma(hipStream_t s, const ConvProblem& p, const MfmaPlan& pl, c
         if (!fast->has_wqf && epi.calib && !fast->fc) {
             if (!fast->fused && fast->relu_folded) kind = EPI_KIND_RELU;
             if (!fast->fused && fast->act == CLDNN_HIP_ACT_NONE) kind = EPI_KIND_LINEAR;
-            if (fast->fused && fast->act == CLDNN_HIP_ACT_NONE && fast->eltw_relu_folded && epi.eltw_calib) kind = EPI_KIND_FUSED;
+            if (fast->fused && fast->act == CLDNN_HIP_ACT_NONE && fast->eltw_relu_folded && epi.eltw_calib && !fast->conv_sat)
+                kind = EPI_KIND_FUSED;
         }
     }
     a.bpk = (const v4i*)wb.gather;

@@ -301,7 +301,8 @@ __device__ __forceinline__ v4i epilogue_fast16(const Args& a, const v4i (&acc)[4
         if (F.fused) {
 #pragma unroll
             for (int c = 0; c < 16; ++c) {
-                const float r = rha(v[c]);
+                float r = rha(v[c]);
+                if (F.conv_sat) r = med3(r, F.conv_lo, F.conv_hi);
                 const unsigned word = (unsigned)ev4[c >> 2];
                 const float e = F.eltw_u8 ? (float)((word >> (8 * (c & 3))) & 255u)
                                           : (float)(int)(int8_t)(word >> (8 * (c & 3)));

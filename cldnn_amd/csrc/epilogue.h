@@ -131,6 +131,7 @@ __device__ __forceinline__ EpiOut epilogue_generic(const Epilogue& e, int acc, i
             return finish(e, cal);
         }
         cal = round_sel(cal, e.round_even);
+        if (e.conv_sat) cal = (float)(e.conv_sat == 1 ? sat_s8(cal) : sat_u8(cal));  // what an int8 tensor in between would hold
         float ev = e.ncs_on ? eltw * e.ncs : eltw;
         float s = cal + ev;
         float ea = act_f(e.eltw_act, e.eltw_m, e.eltw_n, s);

@@ -89,6 +89,8 @@ struct FastEpi {
     int32_t iqf_one;      // iqf == 1: the multiplication is left out (x * 1.0f == x)
     int32_t clamp_folded; // clamp{m, n} with 0 <= m <= n, factors >= 0 and n * factor inside the output range: the result
                           // needs no second clamp and rounds like a non-negative number
+    int32_t conv_sat;     // fused: the rounded convolution result is limited to [conv_lo, conv_hi] before the sum
+    float conv_lo, conv_hi;
     int32_t fc;           // the fully_connected form: float bias after the dequantisation, conversion to char keeps the low byte
 };
 // true (and *out filled) when the short epilogue reproduces the long one bit for bit

@@ -67,6 +67,7 @@ class ConvDesc(C.Structure):
         ("second_input_in_output", C.c_int32), ("round_to_even", C.c_int32),
         ("impl", C.c_int32), ("tile_override", C.c_int32),
         ("pad_end_delta_y", C.c_int32), ("pad_end_delta_x", C.c_int32), ("fully_connected", C.c_int32),
+        ("conv_saturate", C.c_int32),
     ]
 
 
@@ -428,7 +429,7 @@ def conv_desc(x_t, w_shape, out_dt, *, stride=(1, 1), pad=(0, 0), dilation=(1, 1
               out_pad=(0, 0), bias_dt=NO_TYPE, w_dt=S8, has_wqf=False, has_calib=False, iqf=1.0, oqf=1.0,
               act="none", act_m=0.0, act_n=0.0, eltw_t=None, non_conv_scale=1.0, eltw_act="none", eltw_m=0.0,
               eltw_n=0.0, has_eltw_calib=False, eltw_stride=(1, 1), in_place=False, round_even=False,
-              impl=IMPL_AUTO, tile=0, pad_end=None, fc=False):
+              impl=IMPL_AUTO, tile=0, pad_end=None, fc=False, conv_saturate=0):
     """Fill a ConvDesc from an input Tensor and the weight shape [OFM, IFM/groups, FY, FX].
     pad = zero padding on the low side (y, x); pad_end = on the high side (default: the same)."""
     L = lib()
@@ -460,6 +461,7 @@ def conv_desc(x_t, w_shape, out_dt, *, stride=(1, 1), pad=(0, 0), dilation=(1, 1
     d.impl, d.tile_override = impl, tile
     d.pad_end_delta_y, d.pad_end_delta_x = pad_end[0] - pad[0], pad_end[1] - pad[1]
     d.fully_connected = int(fc)
+    d.conv_saturate = int(conv_saturate)
     return d
 
 
@@ -473,7 +475,7 @@ def conv_forward(engine, x, w, bias=None, wqf=None, calib=None, *, stride=(1, 1)
                  groups=1, out_dt=None, iqf=1.0, oqf=1.0, act="none", act_m=0.0, act_n=0.0, eltw=None,
                  non_conv_scale=1.0, eltw_act="none", eltw_m=0.0, eltw_n=0.0, eltw_calib=None, eltw_stride=(1, 1),
                  round_even=False, fmt="bfyx", in_pad=(0, 0), out_pad=(0, 0), impl=IMPL_AUTO, tile=0,
-                 want_acc=False, want_info=False, pad_end=None, fc=False, in_place=False):
+                 want_acc=False, want_info=False, pad_end=None, fc=False, in_place=False, conv_saturate=0):
     """numpy in, numpy out: upload (reordering to `fmt`), run the HIP convolution, download.
 
     Argument meaning follows oracle.refconv.conv so that parity tests can call both alike.  in_place: the residual
@@ -496,7 +498,8 @@ def conv_forward(engine, x, w, bias=None, wqf=None, calib=None, *, stride=(1, 1)
                   has_calib=calib is not None, iqf=iqf, oqf=oqf, act=act, act_m=act_m, act_n=act_n,
                   eltw_t=None if e_buf is None else e_buf.tensor, non_conv_scale=non_conv_scale, eltw_act=eltw_act,
                   eltw_m=eltw_m, eltw_n=eltw_n, has_eltw_calib=eltw_calib is not None, eltw_stride=eltw_stride,
-                  round_even=round_even, impl=impl, tile=tile, pad_end=pad_end, fc=fc, in_place=in_place)
+                  round_even=round_even, impl=impl, tile=tile, pad_end=pad_end, fc=fc, in_place=in_place,
+                  conv_saturate=conv_saturate)
     c = Conv(engine, d, w, bias, wqf, calib, eltw_calib)
     if in_place:
         out = upload(engine, np.ascontiguousarray(eltw), "fs_b_yx_fsv16" if first_layer else fmt, out_pad)

@@ -132,6 +132,7 @@ struct prim {
     int32_t eltw_mode = cldnn_eltwise_sum;
     bool eltw_with_act = false;
     float eltw_slope = 0.f;
+    int32_t conv_saturate = 0;   // fused node made from a sum without activation: the convolution's int8 saturation stays
     std::vector<cldnn_tensor> eltw_stride;
     std::vector<float> eltw_coefficients;
     // convolution / fused conv part

@@ -507,7 +507,11 @@ static void eltwise_remove_stride(cldnn_program_impl* prog)
     }
 }
 
-// convolution (1x1, stride 1) + eltwise sum with relu -> fused_conv_eltwise (reference :181-337)
+// convolution (1x1, stride 1) + eltwise sum with relu -> fused_conv_eltwise (reference :181-337).
+// A sum WITHOUT activation stays a primitive of its own in the reference (a residual sum of MobileNet-v2).  Its
+// arithmetic differs from the fused primitive's in one point: it adds to the convolution's int8 output, that is to the
+// saturated value.  With that saturation kept inside the fused kernel (conv_saturate) the results are the same, so a
+// quantized s8 sum of that kind is fused here as well: one launch and one tensor round trip less per block.
 static void fuse_conv_eltwise(cldnn_program_impl* prog)
 {
     std::vector<node*> convs;
@@ -517,7 +521,15 @@ static void fuse_conv_eltwise(cldnn_program_impl* prog)
         if (c->users.size() != 1 || c->is_output) continue;
         node* e = c->users[0];
         if (e->p->type != prim_type::eltwise || e->is_output || e->p->inputs.size() != 2) continue;
-        if (e->p->eltw_mode != cldnn_eltwise_sum || !e->p->eltw_with_act) continue;
+        if (e->p->eltw_mode != cldnn_eltwise_sum) continue;
+        const bool keep_saturation = !e->p->eltw_with_act;
+        if (keep_saturation) {
+            // the stand-alone quantized sum: round((a + b) * factor[f]), saturated to the signed range
+            // (reference generic_eltwise_ref.cl:318-330); s8 everywhere, no coefficients, quantized convolution
+            bool ok = !e->p->eltw_calib.empty() && e->p->eltw_coefficients.empty() && !c->p->wqf.empty();
+            for (node* t : {c, e, e->deps[0], e->deps[1]}) ok = ok && t->out.data_type == cldnn_i8;
+            if (!ok) continue;
+        }
         const cldnn_layout& cl = c->out;
         const bool ok_type = (is_int8(cl.data_type) && (cl.format == cldnn_format_b_fs_yx_fsv4 || cl.format == cldnn_format_fs_b_yx_fsv16
                                                         || cl.format == cldnn_format_bfyx || cl.format == cldnn_format_byxf))
@@ -541,8 +553,9 @@ static void fuse_conv_eltwise(cldnn_program_impl* prog)
         f->eltw_calib = e->p->eltw_calib;
         f->eltw_oqf = e->p->eltw_oqf;
         f->eltw_mode = e->p->eltw_mode;
-        f->eltw_with_act = true;
+        f->eltw_with_act = e->p->eltw_with_act;
         f->eltw_slope = e->p->eltw_slope;
+        f->conv_saturate = keep_saturation ? 1 : 0;
         f->non_conv_scale = 1.0f;
         f->output_padding = e->p->output_padding;
         f->out_dt.data_type = (cldnn_data_type)e->out.data_type;  // the fused primitive produces what the eltwise produced
@@ -572,6 +585,7 @@ static void fuse_conv_eltwise(cldnn_program_impl* prog)
         for (node* u : std::vector<node*>(e->users)) replace_dep(u, e, nf);
         remove_node(prog, e);
         remove_node(prog, c);
+        calc_layout(nf);  // a later sum asks for the type of this one
     }
 }
 
@@ -825,6 +839,7 @@ static void compile_conv(cldnn_program_impl* prog, node* n)
         d.fused = 1;
         d.non_conv_scale = p.non_conv_scale;
         d.second_input_in_output = p.second_input_in_output ? 1 : 0;
+        d.conv_saturate = p.conv_saturate;
         if (!p.second_input_in_output) d.eltw = to_hip(n->deps[1]->out);
         if (p.eltw_with_act) {
             d.eltw_activation = p.eltw_slope == 0.0f ? CLDNN_HIP_ACT_RELU : CLDNN_HIP_ACT_RELU_SLOPE;
@@ -1015,6 +1030,7 @@ std::string describe_node(const node* n)
         s += ",\"eltw_stride\":" + (p.eltw_stride.empty() ? std::string("null") : four(p.eltw_stride[0].sizes));
         s += ",\"eltw_slope\":" + std::to_string(p.eltw_slope) + ",\"eltw_calib\":\"" + p.eltw_calib + "\"";
         if (p.second_input_in_output) s += ",\"second_input_in_output\":true";
+        if (p.conv_saturate) s += ",\"conv_saturate\":" + std::to_string(p.conv_saturate);
     }
     if (p.type == prim_type::eltwise) {
         s += ",\"mode\":" + std::to_string(p.eltw_mode) + ",\"strides\":[";

@@ -167,7 +167,7 @@ std::string conv_signature(const cldnn_hip_conv_desc& d)
       << ";act=" << d.activation << ";fc=" << d.fully_connected << ";even=" << d.round_to_even;
     if (d.fused)
         o << ";eltw=" << (d.second_input_in_output ? std::string("inplace") : tensor(d.eltw)) << ";es=" << d.eltw_stride_y << "," << d.eltw_stride_x
-          << ";eact=" << d.eltw_activation << ";ecal=" << d.has_eltw_calib << ";scale1=" << (d.non_conv_scale == 1.0f);
+          << ";eact=" << d.eltw_activation << ";ecal=" << d.has_eltw_calib << ";scale1=" << (d.non_conv_scale == 1.0f) << ";csat=" << d.conv_saturate;
     return o.str();
 }
 

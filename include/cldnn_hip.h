@@ -277,6 +277,12 @@ typedef struct {
      * accumulator; conversion to char keeps the low byte; the activation acts on that char.  A fully_connected layer
      * is the convolution whose filter covers the whole input plane; this flag only matters when has_wqf is set. */
     int32_t fully_connected;
+    /* fused form only, needs has_wqf.  1: the convolution's rounded result is saturated to the s8 range before the
+     * second input is added (2: to the u8 range) -- the arithmetic of a convolution that writes int8 followed by a
+     * stand-alone quantized eltwise sum (reference generic_eltwise_ref.cl:318-330 behind convolution_gpu_ref), which
+     * fused_conv_eltwise itself does not have: it adds to the unsaturated value (fused_conv_eltwise_gpu_ref.cl:199-233).
+     * Lets a sum the reference leaves stand-alone run inside the convolution with unchanged results. */
+    int32_t conv_saturate;
 } cldnn_hip_conv_desc;
 
 /* Host pointers: weights [ofm][ifm/groups][fy][fx] dense, bias/wqf/calib/eltw_calib [ofm] or NULL.

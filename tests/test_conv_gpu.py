@@ -319,6 +319,42 @@ def test_residual_read_from_the_output_buffer(eng, out_dt, e_dt):
     assert_same(rc.conv(x, w, bias, wqf=wqf, calib=calib, **kw), out)
 
 
+@pytest.mark.parametrize("in_dt", [np.uint8, np.int8], ids=["u8", "s8"])
+def test_fused_sum_that_keeps_the_convolution_saturation(eng, in_dt):
+    """conv_saturate: the fused kernel limits the convolution's rounded result to the s8 range before it adds the second
+    input, which makes it equal to a convolution writing s8 followed by the reference's stand-alone quantized sum
+    (generic_eltwise_ref.cl:318-330) -- not to fused_conv_eltwise, which adds to the unsaturated value"""
+    x, w, bias, wqf, calib = problem(51, 2, 64, 14, 14, 128, 1, 1, in_dt)
+    calib = calib * 3  # a good share of the convolution results beyond +-127
+    r = np.random.default_rng(9)
+    e = r.integers(-128, 128, (2, 128, 14, 14)).astype(np.int8)
+    ecal = r.uniform(0.3, 1.2, 128).astype(np.float32)
+    conv_s8 = rc.conv(x, w, bias, wqf=wqf, calib=calib, out_dt="s8")
+    ref = rc.eltwise([e, conv_s8], "sum", calib=ecal)
+    unsaturated = rc.conv(x, w, bias, wqf=wqf, calib=calib, out_dt="s8", act="none", eltw=e, eltw_act="none", eltw_calib=ecal)
+    assert 0.02 < (ref != unsaturated).mean() < 0.9  # the two forms do differ on this data
+    kw = dict(out_dt="s8", act="none", eltw=e, eltw_act="none", eltw_calib=ecal, conv_saturate=1)
+    seen = set()
+    for tile in [0] + [t for t in tiles() if not tile_names()[t - 1].startswith("stem")]:
+        out, info = hip.conv_forward(eng, x, w, bias, wqf, calib, fmt="fs_b_yx_fsv16", tile=tile, want_info=True, **kw)
+        seen.add(info.kernel_name.decode().split("<")[0])
+        assert_same(ref, out)
+    assert {"conv_mfma", "conv_stream", "conv_bdir", "conv_wsl", "conv_gemv"} <= seen, seen
+    assert_same(ref, hip.conv_forward(eng, x, w, bias, wqf, calib, fmt="bfyx", **kw))                # layout-agnostic kernel
+    assert_same(ref, hip.conv_forward(eng, x, w, bias, wqf, calib, fmt="fs_b_yx_fsv16", round_even=False, non_conv_scale=1.0, in_place=False, **kw))
+    with pytest.raises(hip.HipError):  # goes with the quantized fused form only
+        hip.conv_forward(eng, x, w, bias, wqf, calib, fmt="fs_b_yx_fsv16", out_dt="s8", conv_saturate=1)
+    # depthwise
+    x, w, bias, wqf, calib = problem(52, 2, 32, 9, 9, 32, 3, 3, in_dt, groups=32)
+    calib = calib * 3
+    e = r.integers(-128, 128, (2, 32, 9, 9)).astype(np.int8)
+    ref = rc.eltwise([e, rc.conv(x, w, bias, wqf=wqf, calib=calib, out_dt="s8", pad=(1, 1), groups=32)], "sum", calib=ecal[:32])
+    out, info = hip.conv_forward(eng, x, w, bias, wqf, calib, fmt="fs_b_yx_fsv16", in_pad=(1, 1), pad=(1, 1), groups=32, out_dt="s8", act="none",
+                                 eltw=e, eltw_act="none", eltw_calib=ecal[:32], conv_saturate=1, want_info=True)
+    assert b"conv_dw" in info.kernel_name
+    assert_same(ref, out)
+
+
 def test_mfma_f32_bias_added_after_dequantisation(eng):
     x, w, _, wqf, calib = problem(14, 1, 32, 8, 8, 32, 3, 3, np.int8)
     bias = np.random.default_rng(1).uniform(-50, 50, 32).astype(np.float32)

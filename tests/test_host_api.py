@@ -295,18 +295,18 @@ def test_unsupported_activation_is_not_folded():
     assert "relu" in opt and opt["conv"]["fused_activation"] == cl.activation_func.none
 
 
-def residual_block(fy=1, stride=1, with_activation=True, eltw_strides=None, in_fmt=F.bfyx):
+def residual_block(fy=1, stride=1, with_activation=True, eltw_strides=None, in_fmt=F.bfyx, sum_calib="c", dt=None):
     """conv(3x3) -> [conv 1x1 | 3x3] + shortcut -> eltwise sum (+relu): the tail of a ResNet block."""
     B, Cn, H, W = 2, 16, 8, 8
     w1 = attach(np.ones((Cn, Cn, 3, 3), np.int8))
     w2 = attach(np.ones((Cn, Cn, fy, fy), np.int8))
-    t = cl.topology(cl.input_layout("in", cl.layout(DT.i8, in_fmt, cl.tensor(B, Cn, W, H))),
+    t = cl.topology(cl.input_layout("in", cl.layout(DT.i8 if dt is None else dt, in_fmt, cl.tensor(B, Cn, W, H))),
                     cl.data("w1", w1), cl.data("w2", w2), cl.data("q", vec(Cn)), cl.data("c", vec(Cn)),
                     cl.convolution("conv1", "in", ["w1"], w_quantization_factor=["q"], output_calibration_factors=["c"],
                                    input_offset=cl.tensor(0, 0, -1, -1, 0), with_activation=True),
                     cl.convolution("conv2", "conv1", ["w2"], w_quantization_factor=["q"], output_calibration_factors=["c"],
                                    input_offset=cl.tensor(0, 0, -(fy // 2), -(fy // 2), 0), stride=cl.tensor(1, 1, stride, stride)),
-                    cl.eltwise("sum", "in", "conv2", cl.eltwise_mode.sum, with_activation, 0.0, output_calibration_factors="c",
+                    cl.eltwise("sum", "in", "conv2", cl.eltwise_mode.sum, with_activation, 0.0, output_calibration_factors=sum_calib,
                                stride=eltw_strides),
                     cl.activation("out", "sum", cl.activation_func.none))
     return t
@@ -326,10 +326,22 @@ def test_conv_eltwise_fusing():
     assert f["format"] == F.fs_b_yx_fsv16
 
 
-@pytest.mark.parametrize("kw", [dict(fy=3), dict(with_activation=False)], ids=["3x3", "no_activation"])
+@pytest.mark.parametrize("kw", [dict(fy=3), dict(with_activation=False, sum_calib=""), dict(with_activation=False, dt=DT.u8)],
+                         ids=["3x3", "no_activation_unquantized", "no_activation_u8"])
 def test_conv_eltwise_not_fused(kw):
     ids = [n["id"] for n in cl.plan(residual_block(**kw), cl.build_options(optimize_data=True))]
     assert "conv2" in ids and "sum" in ids
+
+
+def test_sum_without_activation_is_fused_with_the_saturation_kept():
+    """the reference leaves a sum without activation stand-alone (prepare_primitive_fusing.cpp:181-337 wants the relu); a
+    quantized s8 one is fused here with the one difference of the two forms -- the stand-alone sum adds to the
+    convolution's saturated int8 output -- kept inside the kernel"""
+    opt = by_id(cl.plan(residual_block(with_activation=False), cl.build_options(optimize_data=True)))
+    f = opt["conv2_fused_sum"]
+    assert f["type"] == "fused_conv_eltwise" and f["conv_saturate"] == 1 and f["eltw_calib"] == "c"
+    assert "conv_saturate" not in by_id(cl.plan(residual_block(), cl.build_options(optimize_data=True)))["conv2_fused_sum"]
+    assert "sum" in by_id(cl.plan(residual_block(with_activation=False)))  # as written without optimize_data
 
 
 def downsampling_junction(size=8, user_stride=(2, 2), second_user="conv", mid_filter=3):

@@ -1,5 +1,5 @@
 """A whole quantized MobileNet-v2 (52 convolutions of which 17 depthwise, ReLU6 as clamp activations, 10 residual sums
-that stay stand-alone eltwise primitives, global average pooling, fully_connected) through the clDNN API against the CPU
+without activation, global average pooling, fully_connected) through the clDNN API against the CPU
 oracle run layer by layer, bit for bit."""
 import numpy as np
 import pytest
@@ -78,10 +78,14 @@ def test_mobilenet_v2_int8_network_matches_the_oracle():
         plan = {n["id"]: n for n in cl.plan(topo, opts)}
         folded = [i for i, n in plan.items() if n["type"] == "convolution" and n.get("fused_activation") == cl.activation_func.clamp]
         if optimize:
-            # every clamp is folded into the convolution before it; the residual sums have no activation and stay
-            # stand-alone; every convolution up to the classifier runs in the blocked layout
+            # every clamp is folded into the convolution before it; the residual sums have no activation: the reference
+            # would leave them stand-alone, here they run inside their projection convolution with the int8 saturation of
+            # the convolution's result kept (conv_saturate), except the two that are watched; every convolution up to
+            # the classifier runs in the blocked layout
             assert len(folded) == 35 and not any(n["type"] == "activation" for n in plan.values())
-            assert sum(n["type"] == "eltwise" for n in plan.values()) == 10 and not any("_fused_" in i for i in plan)
+            assert sorted(i for i, n in plan.items() if n["type"] == "eltwise") == ["b10_fsv16", "b3_fsv16"]
+            fused = [n for i, n in plan.items() if "_fused_" in i]
+            assert len(fused) == 8 and all(n["conv_saturate"] == 1 for n in fused)
             assert all(n["format"] == cl.format.fs_b_yx_fsv16 for n in plan.values() if n["type"] == "convolution" and not n.get("fully_connected"))
         else:
             assert folded == [] and sum(n["type"] == "activation" for n in plan.values()) == 35
