@@ -100,3 +100,12 @@ def test_mobilenet_v2_int8_network_matches_the_oracle():
             assert got.shape == ref[name].shape, name
             bad = int((got != ref[name]).sum())
             assert bad == 0, "%s (optimize_data=%s): %d of %d values differ" % (name, optimize, bad, got.size)
+    # an engine without a memory pool also lets the fused sums write over their shortcuts (read / write pass): both
+    # options on one node, same logits
+    eng2 = cl.engine(enable_memory_pool=False)
+    net = cl.network(eng2, mn.topology(cl, eng2, params, B), cl.build_options(optimize_data=True))
+    both = [i for i in net.get_all_primitive_ids() if "_fused_" in i and net.get_primitive_info(i).get("second_input_in_output")
+            and net.get_primitive_info(i).get("conv_saturate") == 1]
+    assert len(both) == 10, both
+    net.set_input_data("input", cl.make_memory(eng2, x))
+    np.testing.assert_array_equal(net.execute()["fc1000"].get_memory().read(), run_oracle(x, params, folded=True)["fc1000"])
