@@ -534,7 +534,7 @@ def main():
             "cores": cb["threads"],
             "kind": "port",
             "sample": "first %d image(s) of every layer of the same stack through oracle/refconv.c "
-                      "(OpenMP over batch x ofm), %.1f s of CPU time" % (cb["images"], cb["seconds"]),
+                      "(OpenMP over batch x ofm), %.1f s on %d threads = %.0f s of CPU work" % (cb["images"], cb["seconds"], cb["threads"], cb["seconds"] * cb["threads"]),
         }
         res["verified"] = {"outputs_compared": cb["checked"], "mismatches": cb["mismatches"],
                            "what": "GPU batch-%d results of the first %d image(s), every layer, vs the CPU oracle "
