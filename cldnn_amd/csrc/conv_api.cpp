@@ -320,7 +320,7 @@ cldnn_hip_status cldnn_hip_conv_release(cldnn_hip_conv c)
     });
 }
 
-static void run(cldnn_hip_conv c, const void* in, void* out, const void* eltw, int32_t* raw)
+static void run(cldnn_hip_conv c, const void* in, void* out, const void* eltw, int32_t* raw, bool static_scratch = false)
 {
     CHIP_REQUIRE(c && in && (out || raw), CLDNN_HIP_INVALID_ARG, "null argument");
     const ConvProblem& p = c->p;
@@ -336,6 +336,14 @@ static void run(cldnn_hip_conv c, const void* in, void* out, const void* eltw, i
         break;
     case CLDNN_HIP_IMPL_MFMA: {
         MfmaBuffers wb{(const int8_t*)c->w_packed, (const int32_t*)c->ktab, c->gather};
+        if (static_scratch) {
+            // the gather scratch comes from the array inside the code object instead of the object's own allocation
+            const size_t need = mfma_gather_bytes(p, c->mplan);
+            CHIP_REQUIRE(need <= mfma_static_scratch_bytes(), CLDNN_HIP_UNSUPPORTED_SIZE,
+                         "this convolution gathers " + std::to_string(need) + " bytes of activations, the static scratch holds "
+                             + std::to_string(mfma_static_scratch_bytes()));
+            if (need) wb.gather = mfma_static_scratch(c->engine->device);
+        }
         if (raw)
             launch_conv_mfma(s, p, c->mplan, wb, (const int32_t*)c->acc_init_raw, c->epi, nullptr, in, nullptr, nullptr, raw);
         else
@@ -355,6 +363,12 @@ static void run(cldnn_hip_conv c, const void* in, void* out, const void* eltw, i
 cldnn_hip_status cldnn_hip_conv_enqueue(cldnn_hip_conv c, const void* input_dev, void* output_dev, const void* eltw_dev)
 {
     return guarded([&] { run(c, input_dev, output_dev, eltw_dev, nullptr); });
+}
+
+cldnn_hip_status cldnn_hip_conv_enqueue_static_scratch(cldnn_hip_conv c, const void* input_dev, void* output_dev,
+                                                       const void* eltw_dev)
+{
+    return guarded([&] { run(c, input_dev, output_dev, eltw_dev, nullptr, true); });
 }
 
 // One candidate of the tuner: microseconds per launch, or a negative value when the row refuses the convolution.

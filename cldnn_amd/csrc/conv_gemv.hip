@@ -11,6 +11,8 @@
 // K-step lie in 64 different cache lines, and every workgroup would pull all of them through its L1 again; a small
 // kernel first gathers the activations into fragment order (1 KB per K-step and pixel fragment, sign flip applied),
 // which the main kernel then reads as it reads the weights.
+#include <mutex>
+
 #include "conv_mfma_kernel.h"
 
 namespace chip {
@@ -19,6 +21,8 @@ enum { GEMV_D = 8 };  // look-ahead in K-steps; the packed stream and the tap ta
 
 // activations in fragment order: bpk[(ptile * (ksteps + GEMV_SLACK) + ks) * 64 + lane]
 enum { GEMV_SLACK = 32 };
+// size of the gather scratch that lives in the code object (for callers that may not allocate)
+enum { GEMV_STATIC_SCRATCH_BYTES = 4 << 20 };
 __global__ void __launch_bounds__(256) gemv_gather_kernel(MfmaArgs a)
 {
     const int lane = threadIdx.x & 63;
@@ -130,5 +134,32 @@ void launch_gemv(hipStream_t s, const MfmaArgs& a, int grid, int waves, int mtil
 }
 
 size_t gemv_gather_bytes(int mtiles, int ksteps) { return ((size_t)mtiles * (ksteps + GEMV_SLACK)) * 1024; }
+
+// ---- gather scratch that nobody allocates: one array per device, part of the loaded code object.
+// Every device the library runs on holds its own copy at its own address until the process ends.  In host code the
+// array's name is only a handle for hipGetSymbolAddress; kernels and copies take the address that call returns.
+static __device__ __align__(256) unsigned char scratch[GEMV_STATIC_SCRATCH_BYTES];
+
+size_t gemv_static_scratch_bytes() { return GEMV_STATIC_SCRATCH_BYTES; }
+
+// Device address of `scratch` on `device`, which the caller has made current.  Looked up once per device.
+void* gemv_static_scratch(int device)
+{
+    enum { MAX_DEVICES = 64 };
+    static std::mutex guard;
+    static void* address[MAX_DEVICES] = {};
+    CHIP_REQUIRE(device >= 0 && device < MAX_DEVICES, CLDNN_HIP_INVALID_ARG, "device index beyond the static scratch table");
+    std::lock_guard<std::mutex> lock(guard);
+    if (!address[device]) {
+        int current = -1;
+        CHIP_CHECK(hipGetDevice(&current));
+        CHIP_REQUIRE(current == device, CLDNN_HIP_ERROR, "the static scratch is looked up with its device current");
+        void* ptr = nullptr;
+        CHIP_CHECK(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
+        CHIP_REQUIRE(ptr, CLDNN_HIP_DEVICE_ERROR, "hipGetSymbolAddress returned no address for the static scratch");
+        address[device] = ptr;
+    }
+    return address[device];
+}
 
 }  // namespace chip

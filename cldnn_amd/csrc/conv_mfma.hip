@@ -18,6 +18,8 @@ void launch_bdir_k2(hipStream_t s, const MfmaArgs& a, int nt, int grid, int lds,
 void launch_bdir_k4(hipStream_t s, const MfmaArgs& a, int nt, int grid, int lds, int epi);
 void launch_gemv(hipStream_t s, const MfmaArgs& a, int grid, int waves, int mtiles);
 size_t gemv_gather_bytes(int mtiles, int ksteps);
+size_t gemv_static_scratch_bytes();
+void* gemv_static_scratch(int device);
 #define DECL_WSL(d) void launch_wsl_d##d(hipStream_t s, const MfmaArgs& a, int nt, int grid, int lds, int epi);
 DECL_WSL(1) DECL_WSL(2) DECL_WSL(3) DECL_WSL(4) DECL_WSL(6) DECL_WSL(8)
 #undef DECL_WSL
@@ -407,6 +409,9 @@ size_t mfma_gather_bytes(const ConvProblem& p, const MfmaPlan& pl)
 {
     return pl.gemv && p.FY * p.FX > 1 ? gemv_gather_bytes(pl.mtiles, pl.ksteps) : 0;
 }
+
+size_t mfma_static_scratch_bytes() { return gemv_static_scratch_bytes(); }
+void* mfma_static_scratch(int device) { return gemv_static_scratch(device); }
 
 void launch_conv_mfma(hipStream_t s, const ConvProblem& p, const MfmaPlan& pl, const MfmaBuffers& wb,
                       const int32_t* acc_init, const Epilogue& epi, const FastEpi* fast, const void* in, const void* eltw,

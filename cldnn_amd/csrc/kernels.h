@@ -72,6 +72,10 @@ struct MfmaBuffers {
     void* gather = nullptr;  // small-batch kernel with a filter wider than one tap: mfma_gather_bytes() of scratch
 };
 size_t mfma_gather_bytes(const ConvProblem& p, const MfmaPlan& pl);  // 0 when the plan needs no scratch
+// The same scratch without an allocation: a fixed-size array inside the loaded code object, one copy per device.
+// mfma_static_scratch returns its device address on `device`, which must be the current device.
+size_t mfma_static_scratch_bytes();
+void* mfma_static_scratch(int device);
 // parameters of the short epilogue (int8 output, float requantisation)
 struct FastEpi {
     int32_t has_wqf;      // multiply by wqf[f] and iqf

@@ -160,6 +160,7 @@ SIGNATURES = {
                                         C.POINTER(C.c_float)]),
     "cldnn_hip_conv_release": (C.c_int32, [C.c_void_p]),
     "cldnn_hip_conv_enqueue": (C.c_int32, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p]),
+    "cldnn_hip_conv_enqueue_static_scratch": (C.c_int32, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p]),
     "cldnn_hip_conv_accumulators": (C.c_int32, [C.c_void_p, C.c_void_p, C.c_void_p]),
     "cldnn_hip_conv_get_info": (C.c_int32, [C.c_void_p, C.POINTER(ConvInfo)]),
     "cldnn_hip_conv_out_extent": (C.c_int32, [C.c_int32] * 5),
@@ -391,6 +392,10 @@ class Conv:
 
     def enqueue(self, src, dst, eltw=None):
         check(lib().cldnn_hip_conv_enqueue(self.h, src.ptr, dst.ptr, eltw.ptr if eltw is not None else None))
+
+    def enqueue_static_scratch(self, src, dst, eltw=None):
+        """the entry point that allocates nothing: scratch from the array inside the code object"""
+        check(lib().cldnn_hip_conv_enqueue_static_scratch(self.h, src.ptr, dst.ptr, eltw.ptr if eltw is not None else None))
 
     def accumulators(self, src):
         d = self.desc

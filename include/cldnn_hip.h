@@ -294,6 +294,16 @@ cldnn_hip_status cldnn_hip_conv_release(cldnn_hip_conv c);
 /* asynchronous on the engine stream; device pointers */
 cldnn_hip_status cldnn_hip_conv_enqueue(cldnn_hip_conv c, const void* input_dev, void* output_dev,
                                         const void* eltw_dev);
+/* cldnn_hip_conv_enqueue for callers that must not allocate device memory (code under HIP graph capture, tight
+ * serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference.  Same arguments and
+ * results as cldnn_hip_conv_enqueue; the one kernel family with a scratch buffer -- the small-batch kernel, which
+ * gathers the activations of a filter wider than one tap into fragment order -- takes that buffer from a fixed
+ * array of 4 MiB inside the library's code object (one copy per device, held until the process ends) instead of
+ * the object's own allocation.  Calls no hipMalloc / hipFree.  A convolution whose gather needs more than 4 MiB is
+ * refused with CLDNN_HIP_UNSUPPORTED_SIZE.  Every call on a device shares that device's array: calls that overlap
+ * on one device (two streams) race; calls on one stream are ordered.  Nothing in the array has to start at zero. */
+cldnn_hip_status cldnn_hip_conv_enqueue_static_scratch(cldnn_hip_conv c, const void* input_dev, void* output_dev,
+                                                       const void* eltw_dev);
 /* raw int32 accumulators (before bias), dense [b][ofm][oy][ox]; test / verification hook */
 cldnn_hip_status cldnn_hip_conv_accumulators(cldnn_hip_conv c, const void* input_dev, int32_t* acc_dev);
 
