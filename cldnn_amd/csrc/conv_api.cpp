@@ -4,6 +4,7 @@
 #include <cstring>
 #include <vector>
 
+#include "conv_chain.h"
 #include "kernels.h"
 #include "runtime.h"
 
@@ -33,6 +34,17 @@ struct cldnn_hip_conv_s {
     void* ecal = nullptr;
     cldnn_hip_conv_info info{};
     std::vector<void*> owned;
+};
+
+struct cldnn_hip_conv_chain_s {
+    cldnn_hip_engine engine = nullptr;
+    int count = 0;
+    cldnn_hip_conv stage[3] = {nullptr, nullptr, nullptr};
+    int keep[3] = {0, 0, 0};
+    ChainStageIn in[3]{};
+    ChainPlan plan{};
+    void* packed = nullptr;
+    cldnn_hip_conv_info info{};
 };
 
 namespace {
@@ -369,6 +381,114 @@ cldnn_hip_status cldnn_hip_conv_enqueue_static_scratch(cldnn_hip_conv c, const v
                                                        const void* eltw_dev)
 {
     return guarded([&] { run(c, input_dev, output_dev, eltw_dev, nullptr, true); });
+}
+
+cldnn_hip_status cldnn_hip_conv_chain_create(cldnn_hip_engine e, int32_t count, const cldnn_hip_conv_desc* descs,
+                                             const void* const* weights, const void* const* bias, const float* const* wqf,
+                                             const float* const* calib, const float* const* eltw_calib,
+                                             const int32_t* keep_output, cldnn_hip_conv_chain* out)
+{
+    return guarded([&] {
+        CHIP_REQUIRE(e && descs && weights && out, CLDNN_HIP_INVALID_ARG, "null argument");
+        CHIP_REQUIRE(count >= 2 && count <= 3, CLDNN_HIP_INVALID_ARG, "a chain has two or three convolutions");
+        *out = nullptr;
+        auto* ch = new cldnn_hip_conv_chain_s();
+        ch->engine = e;
+        ch->count = count;
+        e->refs.fetch_add(1);
+        try {
+            for (int k = 0; k < count; ++k) {
+                // every stage is an ordinary convolution object: validation, arithmetic mode, per-feature vectors and the
+                // accumulator start values come from there
+                cldnn_hip_conv c = nullptr;
+                const cldnn_hip_status st = cldnn_hip_conv_create(e, &descs[k], weights[k], bias ? bias[k] : nullptr, wqf ? wqf[k] : nullptr,
+                                                                  calib ? calib[k] : nullptr, eltw_calib ? eltw_calib[k] : nullptr, &c);
+                if (st != CLDNN_HIP_SUCCESS) throw error(st, std::string("stage ") + std::to_string(k) + ": " + cldnn_hip_last_error());
+                ch->stage[k] = c;
+                CHIP_REQUIRE(c->impl == CLDNN_HIP_IMPL_MFMA, CLDNN_HIP_UNSUPPORTED_FORMAT,
+                             "stage " + std::to_string(k) + " of a chain must be a dense int8 convolution in fs_b_yx_fsv16");
+                CHIP_REQUIRE(!descs[k].second_input_in_output, CLDNN_HIP_UNSUPPORTED_FORMAT, "a chained stage cannot read its residual from its own output");
+                ch->keep[k] = keep_output ? (keep_output[k] != 0) : 1;
+                ch->in[k] = ChainStageIn{&c->p, &c->epi, &c->fe, c->fast, (const int32_t*)c->acc_init};
+            }
+            CHIP_REQUIRE(ch->keep[count - 1], CLDNN_HIP_INVALID_ARG, "the last stage of a chain always writes its output");
+            const int cus = e->props.multiProcessorCount;
+            const std::string why = chain_plan(ch->in, count, cus, &ch->plan);
+            if (!why.empty()) throw error(CLDNN_HIP_UNSUPPORTED_FORMAT, "these convolutions cannot run as one chain: " + why);
+            std::vector<int8_t> packed(chain_packed_bytes(ch->plan));
+            const int8_t* w8[3] = {nullptr, nullptr, nullptr};
+            for (int k = 0; k < count; ++k) w8[k] = (const int8_t*)weights[k];
+            chain_pack_weights(ch->in, ch->plan, cus, w8, packed.data());
+            e->make_current();
+            CHIP_CHECK(hipMalloc(&ch->packed, packed.size()));
+            CHIP_CHECK(hipMemcpyAsync(ch->packed, packed.data(), packed.size(), hipMemcpyHostToDevice, e->stream));
+            CHIP_CHECK(hipStreamSynchronize(e->stream));
+            cldnn_hip_conv_info& inf = ch->info;
+            inf.impl = CLDNN_HIP_IMPL_MFMA, inf.tile_index = -1, inf.tile_pixels = 64 * ch->plan.nt, inf.tile_ofm = 64;
+            inf.grid = ch->plan.grid, inf.block = 256, inf.lds_bytes = ch->plan.lds_bytes;
+            std::snprintf(inf.kernel_name, sizeof(inf.kernel_name), "%s", ch->plan.name);
+            // algorithmic work of the chain: every stage's operations; bytes of what has to cross the memory interface,
+            // i.e. without the intermediate tensors that are neither kept nor re-read
+            for (int k = 0; k < count; ++k) {
+                const cldnn_hip_conv_info& si = ch->stage[k]->info;
+                const ConvProblem& p = ch->stage[k]->p;
+                inf.ops += si.ops;
+                int64_t bytes = si.bytes;
+                if (k > 0) bytes -= (int64_t)p.B * p.IH * p.IW * p.IFM;                  // input comes from registers
+                if (!ch->keep[k]) bytes -= (int64_t)p.B * p.OH * p.OW * p.OFM;           // output stays in registers
+                inf.bytes += bytes;
+            }
+        } catch (...) {
+            cldnn_hip_conv_chain_release(ch);
+            throw;
+        }
+        *out = ch;
+    });
+}
+
+cldnn_hip_status cldnn_hip_conv_chain_release(cldnn_hip_conv_chain ch)
+{
+    return guarded([&] {
+        CHIP_REQUIRE(ch, CLDNN_HIP_INVALID_ARG, "null chain");
+        cldnn_hip_engine e = ch->engine;
+        (void)hipSetDevice(e->device);
+        (void)hipStreamSynchronize(e->stream);
+        if (ch->packed) (void)hipFree(ch->packed);
+        for (int k = 0; k < 3; ++k)
+            if (ch->stage[k]) cldnn_hip_conv_release(ch->stage[k]);
+        delete ch;
+        cldnn_hip_engine_release(e);
+    });
+}
+
+cldnn_hip_status cldnn_hip_conv_chain_enqueue(cldnn_hip_conv_chain ch, const void* input_dev, void* const* outputs_dev,
+                                              const void* const* eltw_dev)
+{
+    return guarded([&] {
+        CHIP_REQUIRE(ch && input_dev && outputs_dev, CLDNN_HIP_INVALID_ARG, "null argument");
+        void* outs[3] = {nullptr, nullptr, nullptr};
+        const void* el[3] = {nullptr, nullptr, nullptr};
+        for (int k = 0; k < ch->count; ++k) {
+            if (ch->keep[k]) {
+                CHIP_REQUIRE(outputs_dev[k], CLDNN_HIP_INVALID_ARG, "a kept stage of the chain has no output buffer");
+                outs[k] = outputs_dev[k];
+            }
+            if (ch->stage[k]->desc.fused) {
+                CHIP_REQUIRE(eltw_dev && eltw_dev[k], CLDNN_HIP_INVALID_ARG, "fused stage of a chain without its second input");
+                el[k] = eltw_dev[k];
+            }
+        }
+        ch->engine->make_current();
+        launch_conv_chain(ch->engine->stream, ch->in, ch->plan, ch->packed, input_dev, outs, el);
+    });
+}
+
+cldnn_hip_status cldnn_hip_conv_chain_get_info(cldnn_hip_conv_chain ch, cldnn_hip_conv_info* info)
+{
+    return guarded([&] {
+        CHIP_REQUIRE(ch && info, CLDNN_HIP_INVALID_ARG, "null argument");
+        *info = ch->info;
+    });
 }
 
 // One candidate of the tuner: microseconds per launch, or a negative value when the row refuses the convolution.

@@ -1,0 +1,168 @@
+// Host side of the convolution chain kernel: eligibility, LDS image of the weights, launch.
+#include <cstring>
+#include <mutex>
+#include <string>
+#include <vector>
+
+#include "conv_chain_kernel.h"
+
+namespace chip {
+
+namespace {
+
+enum { ROW_WSL_P64_FOR_CHAIN = 14 };  // the 64-feature weights-stationary row: its packed stream is the LDS image's unit order
+enum { CHAIN_MAX_LDS = 160 * 1024 };
+
+int epilogue_kind(const ChainStageIn& s)
+{
+    const FastEpi& f = *s.fe;
+    int kind = EPI_KIND_FAST;
+    if (!f.has_wqf && s.epi->calib && !f.fc) {
+        if (!f.fused && f.relu_folded) kind = EPI_KIND_RELU;
+        if (!f.fused && f.act == CLDNN_HIP_ACT_NONE) kind = EPI_KIND_LINEAR;
+        if (f.fused && f.act == CLDNN_HIP_ACT_NONE && f.eltw_relu_folded && s.epi->eltw_calib && !f.conv_sat) kind = EPI_KIND_FUSED;
+    }
+    return kind;
+}
+
+struct Instance {
+    int nt, d, sp0, sp1, sp2, e0, e1, e2;
+    void (*launch)(hipStream_t, const ChainArgs&, int, int);
+};
+#define CHAIN_INSTANCE(NT, D, SP0, SP1, SP2, E0, E1, E2) \
+    {NT, D, SP0, SP1, SP2, E0, E1, E2, &launch_chain_instance<NT, D, SP0, SP1, SP2, E0, E1, E2>}
+// What is compiled: the tails of ResNet bottlenecks with 64 mid features (3x3 -> expansion [+ residual] -> next
+// reduction), with and without the third stage, residual fused or not.
+const Instance g_instances[] = {
+    CHAIN_INSTANCE(2, 3, 1, 4, 1, EPI_KIND_RELU, EPI_KIND_FUSED, EPI_KIND_RELU),
+    CHAIN_INSTANCE(2, 3, 1, 4, 0, EPI_KIND_RELU, EPI_KIND_FUSED, EPI_KIND_RELU),
+    CHAIN_INSTANCE(2, 3, 1, 4, 1, EPI_KIND_RELU, EPI_KIND_RELU, EPI_KIND_RELU),
+    CHAIN_INSTANCE(2, 3, 1, 4, 0, EPI_KIND_RELU, EPI_KIND_RELU, EPI_KIND_RELU),
+};
+
+const Instance* find_instance(const ChainPlan& pl)
+{
+    for (const Instance& i : g_instances)
+        if (i.nt == pl.nt && i.d == pl.depth && i.sp0 == pl.sp[0] && i.sp1 == pl.sp[1] && i.sp2 == pl.sp[2] && i.e0 == pl.epi[0]
+            && i.e1 == pl.epi[1] && (pl.stages < 3 || i.e2 == pl.epi[2]))
+            return &i;
+    return nullptr;
+}
+
+}  // namespace
+
+std::string chain_plan(const ChainStageIn* st, int n, int cus, ChainPlan* out)
+{
+    ChainPlan pl{};
+    if (n < 2 || n > CHAIN_MAX_STAGES) return "a chain has two or three stages";
+    pl.stages = n;
+    const ConvProblem& p0 = *st[0].p;
+    for (int k = 0; k < n; ++k) {
+        const ConvProblem& p = *st[k].p;
+        const std::string at = "stage " + std::to_string(k) + ": ";
+        if (!st[k].fast) return at + "needs the short int8 epilogue";
+        if (st[k].fe->fc) return at + "the fully_connected form is not chained";
+        if (p.groups != 1) return at + "grouped convolution";
+        if (p.in_t.format != CLDNN_HIP_FMT_FS_B_YX_FSV16 || p.out_t.format != CLDNN_HIP_FMT_FS_B_YX_FSV16) return at + "needs fs_b_yx_fsv16";
+        if (((p.IFM + 15) / 16) % 4 != 0) return at + "input features must come in multiples of 64";
+        if (st[k].fe->fused && (p.esy != 1 || p.esx != 1 || p.eltw_t.format != CLDNN_HIP_FMT_FS_B_YX_FSV16)) return at + "strided or unblocked residual";
+        if (tensor_elems(p.out_t) >= (1ull << 31) || tensor_elems(p.in_t) >= (1ull << 31)) return at + "tensor of 2 GiB or more";
+        if (k > 0) {
+            const ConvProblem& q = *st[k - 1].p;
+            if (p.FY != 1 || p.FX != 1 || p.sy != 1 || p.sx != 1 || p.py != 0 || p.px != 0) return at + "only the first stage may be wider than 1x1";
+            if (p.IFM != q.OFM || p.B != q.B || p.IH != q.OH || p.IW != q.OW) return at + "does not read the previous stage's result";
+            if (p.in_dt != q.out_dt) return at + "input type differs from the previous stage's output type";
+        }
+        pl.sp[k] = (p.OFM + 63) / 64;
+        pl.epi[k] = epilogue_kind(st[k]);
+    }
+    if (!conv_border_covers(p0)) return "stage 0: the input needs a zero border as wide as the padding";
+    if (p0.dy != 1 || p0.dx != 1) return "stage 0: dilation";
+    // K-steps of every stage as the weights-stationary row packs them
+    pl.units = 0;
+    int vec = 0;
+    for (int k = 0; k < n; ++k) {
+        MfmaPlan mp{};
+        try {
+            mp = mfma_plan(*st[k].p, ROW_WSL_P64_FOR_CHAIN, cus);
+        } catch (const error& e) {
+            return "stage " + std::to_string(k) + ": " + e.what();
+        }
+        pl.unit0[k] = pl.units;
+        pl.kstride[k] = mp.ksteps;
+        pl.units += pl.sp[k] * mp.ksteps;
+        pl.vec0[k] = vec;
+        vec += 4 * pl.sp[k] * 64;
+        if (k == 0) pl.depth = mp.wsl_depth, pl.ksteps0 = mp.ksteps;
+        else if (mp.ksteps < pl.sp[k - 1]) return "stage " + std::to_string(k) + ": fewer K-steps than the previous stage has spans";
+    }
+    pl.lds_bytes = pl.units * 4096 + vec * 4;
+    if (pl.lds_bytes > CHAIN_MAX_LDS) return "the weights of the chain (" + std::to_string(pl.units * 4) + " KiB) do not fit into LDS";
+    pl.nt = 2;
+    pl.m_total = (int64_t)p0.B * p0.OH * p0.OW;
+    pl.granules = (int)((pl.m_total + 16 * pl.nt - 1) / (16 * pl.nt));
+    if (!find_instance(pl)) return "no compiled instance for this chain shape";
+    const int per_cu = pl.lds_bytes * 2 <= CHAIN_MAX_LDS ? 2 : 1;
+    int grid = cus * per_cu / 8 * 8;
+    const int wanted = ((pl.granules + 3) / 4 + 7) / 8 * 8;  // at least one granule per wave
+    if (grid > wanted) grid = wanted;
+    if (grid < 8) grid = 8;
+    pl.grid = grid;
+    std::snprintf(pl.name, sizeof(pl.name), "conv_chain<%d stages,p%d,d%d,spans %d-%d-%d,epi %d-%d-%d>", n, 16 * pl.nt, pl.depth, pl.sp[0],
+                  pl.sp[1], pl.sp[2], pl.epi[0], pl.epi[1], n > 2 ? pl.epi[2] : -1);
+    *out = pl;
+    return std::string();
+}
+
+size_t chain_packed_bytes(const ChainPlan& pl) { return (size_t)pl.units * 4096 + 4096; }
+
+void chain_pack_weights(const ChainStageIn* st, const ChainPlan& pl, int cus, const int8_t* const* w, int8_t* packed)
+{
+    std::memset(packed, 0, chain_packed_bytes(pl));
+    for (int k = 0; k < pl.stages; ++k) {
+        const MfmaPlan mp = mfma_plan(*st[k].p, ROW_WSL_P64_FOR_CHAIN, cus);
+        std::vector<int8_t> buf(mp.packed_bytes);
+        std::vector<int32_t> ktab(mp.ktab_bytes / sizeof(int32_t));
+        mfma_pack_weights(*st[k].p, mp, w[k], buf.data(), ktab.data());
+        std::memcpy(packed + (size_t)pl.unit0[k] * 4096, buf.data(), (size_t)pl.sp[k] * mp.ksteps * 4096);
+    }
+}
+
+void launch_conv_chain(hipStream_t s, const ChainStageIn* st, const ChainPlan& pl, const void* packed_dev, const void* in,
+                       void* const* outs, const void* const* eltws)
+{
+    const ConvProblem& p0 = *st[0].p;
+    ChainArgs a{};
+    a.in = (const int8_t*)in;
+    a.wpk = (const v4i*)packed_dev;
+    a.units = pl.units;
+    a.granules = pl.granules;
+    a.M = (uint32_t)pl.m_total;
+    a.OHW = p0.OH * p0.OW, a.OW = p0.OW;
+    a.div_ohw = make_fast_div((uint32_t)a.OHW), a.div_ow = make_fast_div((uint32_t)a.OW);
+    a.sy = p0.sy, a.sx = p0.sx, a.py = p0.py, a.px = p0.px;
+    a.in_off = (int32_t)p0.in_p.off, a.in_pb = (int32_t)p0.in_p.pb, a.in_pf = (int32_t)p0.in_p.pf, a.in_py = (int32_t)p0.in_p.py;
+    a.ksteps0 = pl.ksteps0, a.CB = (p0.IFM + 15) / 16, a.FX = p0.FX, a.FY = p0.FY;
+    a.tap_dy = p0.dy * (int32_t)p0.in_p.py, a.tap_dx = p0.dx * 16;
+    for (int k = 0; k < pl.stages; ++k) {
+        const ConvProblem& p = *st[k].p;
+        ChainStage& c = a.st[k];
+        c.acc_init = st[k].acc_init;
+        c.out = outs[k];
+        c.eltw = eltws ? eltws[k] : nullptr;
+        CHIP_REQUIRE(!st[k].fe->fused || c.eltw, CLDNN_HIP_INVALID_ARG, "fused stage of a chain without its second input");
+        c.OFM = p.OFM;
+        c.out_off = (int32_t)p.out_p.off, c.out_pb = (int32_t)p.out_p.pb, c.out_pf = (int32_t)p.out_p.pf, c.out_py = (int32_t)p.out_p.py;
+        c.el_off = (int32_t)p.eltw_p.off, c.el_pb = (int32_t)p.eltw_p.pb, c.el_pf = (int32_t)p.eltw_p.pf, c.el_py = (int32_t)p.eltw_p.py;
+        c.xor_mask = p.in_dt == CLDNN_HIP_U8 ? 0x80808080u : 0u;
+        c.unit0 = pl.unit0[k], c.kstride = pl.kstride[k], c.vec0 = pl.vec0[k];
+        c.fe = *st[k].fe;
+        c.epi = *st[k].epi;
+    }
+    const Instance* inst = find_instance(pl);
+    CHIP_REQUIRE(inst, CLDNN_HIP_ERROR, "chain without a compiled instance");
+    inst->launch(s, a, pl.grid, pl.lds_bytes);
+    CHIP_CHECK(hipGetLastError());
+}
+
+}  // namespace chip

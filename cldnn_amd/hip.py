@@ -161,6 +161,12 @@ SIGNATURES = {
     "cldnn_hip_conv_release": (C.c_int32, [C.c_void_p]),
     "cldnn_hip_conv_enqueue": (C.c_int32, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p]),
     "cldnn_hip_conv_enqueue_static_scratch": (C.c_int32, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p]),
+    "cldnn_hip_conv_chain_create": (C.c_int32, [C.c_void_p, C.c_int32, C.POINTER(ConvDesc), C.POINTER(C.c_void_p), C.POINTER(C.c_void_p),
+                                                C.POINTER(C.c_void_p), C.POINTER(C.c_void_p), C.POINTER(C.c_void_p),
+                                                C.POINTER(C.c_int32), C.POINTER(C.c_void_p)]),
+    "cldnn_hip_conv_chain_release": (C.c_int32, [C.c_void_p]),
+    "cldnn_hip_conv_chain_enqueue": (C.c_int32, [C.c_void_p, C.c_void_p, C.POINTER(C.c_void_p), C.POINTER(C.c_void_p)]),
+    "cldnn_hip_conv_chain_get_info": (C.c_int32, [C.c_void_p, C.POINTER(ConvInfo)]),
     "cldnn_hip_conv_accumulators": (C.c_int32, [C.c_void_p, C.c_void_p, C.c_void_p]),
     "cldnn_hip_conv_get_info": (C.c_int32, [C.c_void_p, C.POINTER(ConvInfo)]),
     "cldnn_hip_conv_out_extent": (C.c_int32, [C.c_int32] * 5),
@@ -409,6 +415,60 @@ class Conv:
     def close(self):
         if self.h:
             check(lib().cldnn_hip_conv_release(self.h))
+            self.h = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+
+class ConvChain:
+    """Two or three convolutions executed as one launch (cldnn_hip_conv_chain_*): stage k + 1 is a 1x1 convolution that
+    reads stage k's result.  stages: list of (desc, weights, bias, wqf, calib, eltw_calib); keep[k] False: stage k's
+    result is never written.  Raises HipError (CLDNN_HIP_UNSUPPORTED_FORMAT) when the stages cannot be chained."""
+
+    def __init__(self, engine, stages, keep=None):
+        self.engine, n = engine, len(stages)
+        self.n = n
+        hold = []
+
+        def column(i, dt=None):
+            arr = (C.c_void_p * n)()
+            for k, st in enumerate(stages):
+                a = st[i] if i < len(st) else None
+                if a is not None:
+                    a = np.ascontiguousarray(a, dtype=dt)
+                    hold.append(a)
+                    arr[k] = a.ctypes.data
+            return arr
+
+        descs = (ConvDesc * n)(*[st[0] for st in stages])
+        keep_arr = (C.c_int32 * n)(*[1 if (keep is None or keep[k]) else 0 for k in range(n)])
+        h = C.c_void_p()
+        check(lib().cldnn_hip_conv_chain_create(engine.h, n, descs, column(1), column(2), column(3, np.float32), column(4, np.float32),
+                                                column(5, np.float32), keep_arr, C.byref(h)))
+        self.h = h
+
+    def info(self):
+        i = ConvInfo()
+        check(lib().cldnn_hip_conv_chain_get_info(self.h, C.byref(i)))
+        return i
+
+    def pointers(self, outs, eltws=None):
+        """device pointer arrays for enqueue_raw (entries may be None)"""
+        o = (C.c_void_p * self.n)(*[None if b is None else b.ptr for b in outs])
+        e = (C.c_void_p * self.n)(*[None if (eltws is None or eltws[k] is None) else eltws[k].ptr for k in range(self.n)])
+        return o, e
+
+    def enqueue(self, src, outs, eltws=None):
+        o, e = self.pointers(outs, eltws)
+        check(lib().cldnn_hip_conv_chain_enqueue(self.h, src.ptr, o, e))
+
+    def close(self):
+        if self.h:
+            check(lib().cldnn_hip_conv_chain_release(self.h))
             self.h = None
 
     def __del__(self):

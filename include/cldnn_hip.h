@@ -38,6 +38,7 @@ typedef struct cldnn_hip_engine_s* cldnn_hip_engine;
 typedef struct cldnn_hip_buffer_s* cldnn_hip_buffer;
 typedef struct cldnn_hip_event_s* cldnn_hip_event;
 typedef struct cldnn_hip_conv_s* cldnn_hip_conv;
+typedef struct cldnn_hip_conv_chain_s* cldnn_hip_conv_chain;
 
 const char* cldnn_hip_last_error(void);
 
@@ -318,6 +319,30 @@ typedef struct {
     char kernel_name[96];
 } cldnn_hip_conv_info;
 cldnn_hip_status cldnn_hip_conv_get_info(cldnn_hip_conv c, cldnn_hip_conv_info* info);
+
+/* ------------------------------------------------------------------ convolution chain
+ * Two or three convolution / fused_conv_eltwise nodes of which every one after the first is a 1x1 / stride-1 /
+ * unpadded convolution that reads its predecessor's result, executed as ONE launch: the requantised int8 tile of a
+ * stage is handed to the next stage in registers.  The reference runs such nodes one launch each
+ * (src/gpu/primitive_gpu_base.h:117-168); the results are the same bits.  Typical use: the tail of a ResNet bottleneck,
+ * 3x3 -> 1x1 expansion with the residual sum -> the next block's 1x1 reduction.
+ * descs / weights / bias / wqf / calib / eltw_calib: `count` entries each, as for cldnn_hip_conv_create (the arrays
+ * bias, wqf, calib, eltw_calib and their entries may be NULL).  descs[k + 1].input must describe the same logical
+ * tensor as descs[k].output.  keep_output[k] == 0: nobody else reads stage k's result and it is never written
+ * (NULL: every result is written).  Fails with CLDNN_HIP_UNSUPPORTED_FORMAT when the convolutions cannot run as one
+ * chain (layout, epilogue form, weights that do not fit into LDS ...): the caller then runs them one by one. */
+cldnn_hip_status cldnn_hip_conv_chain_create(cldnn_hip_engine e, int32_t count, const cldnn_hip_conv_desc* descs,
+                                             const void* const* weights, const void* const* bias, const float* const* wqf,
+                                             const float* const* calib, const float* const* eltw_calib,
+                                             const int32_t* keep_output, cldnn_hip_conv_chain* out);
+cldnn_hip_status cldnn_hip_conv_chain_release(cldnn_hip_conv_chain chain);
+/* asynchronous on the engine stream; outputs_dev / eltw_dev: `count` device pointers (entries of stages that are not
+ * kept / not fused are ignored and may be NULL; eltw_dev itself may be NULL when no stage is fused) */
+cldnn_hip_status cldnn_hip_conv_chain_enqueue(cldnn_hip_conv_chain chain, const void* input_dev, void* const* outputs_dev,
+                                              const void* const* eltw_dev);
+/* ops = sum over the stages; bytes = what crosses the memory interface (intermediate tensors that are neither kept
+ * nor re-read are left out) */
+cldnn_hip_status cldnn_hip_conv_chain_get_info(cldnn_hip_conv_chain chain, cldnn_hip_conv_info* info);
 
 /* computed output extent along one axis (reference src/include/sliding_window_utils.h:90-129) */
 int32_t cldnn_hip_conv_out_extent(int32_t in, int32_t pad, int32_t filt, int32_t dil, int32_t stride);

@@ -1,0 +1,142 @@
+"""cldnn_hip_conv_chain_*: two or three convolutions in one launch against the oracle run layer by layer.
+
+A chain must give the bits the separate convolutions give: the oracle computes stage after stage, each on the int8
+tensor the stage before it produced.  Covered: the tail of a ResNet bottleneck (3x3 -> 1x1 expansion with fused
+residual -> next 1x1 reduction), its two-stage form, the unfused form, results kept and not kept, u8 and s8 inputs,
+pixel counts that do not fill the last granule, padded output buffers, and the refusals."""
+import numpy as np
+import pytest
+
+from cldnn_amd import hip
+from oracle import refconv as rc
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def eng():
+    e = hip.Engine()
+    yield e
+    e.close()
+
+
+def layer(r, ifm, ofm, k, in_dt):
+    w = r.integers(-127, 128, (ofm, ifm, k, k)).astype(np.int8)
+    bias = r.integers(-1000, 1001, ofm).astype(np.int32)
+    wqf = np.ones(ofm, np.float32)
+    rms = 147.4 if in_dt == np.uint8 else 40.0
+    calib = (40.0 / (np.sqrt(ifm * k * k) * rms * 73.3) * r.uniform(0.5, 2.0, ofm)).astype(np.float32)
+    return w, bias, wqf, calib
+
+
+def bottleneck_tail(eng, seed, B, H, W, mid, stages, fused, in_dt=np.uint8, keep=None, out_pad=(0, 0)):
+    """builds descriptors + data of 3x3(mid->mid) -> 1x1(mid->4mid)[+residual] [-> 1x1(4mid->mid)], returns what both
+    the chain and the oracle need"""
+    r = np.random.default_rng(seed)
+    lo, hi = (0, 256) if in_dt == np.uint8 else (-128, 128)
+    x = r.integers(lo, hi, (B, mid, H, W)).astype(in_dt)
+    shapes = [(mid, mid, 3), (mid, 4 * mid, 1), (4 * mid, mid, 1)][:stages]
+    xin = hip.upload(eng, x, "fs_b_yx_fsv16", (1, 1))
+    spec, prev_t = [], xin.tensor
+    ref_in, refs = x, []
+    bufs = []
+    for k, (ifm, ofm, fk) in enumerate(shapes):
+        w, bias, wqf, calib = layer(r, ifm, ofm, fk, in_dt if k == 0 else np.int8)
+        is_fused = fused and k == 1
+        eltw = ecal = ebuf = None
+        kw = dict(stride=(1, 1), pad=(fk // 2,) * 2, bias_dt=hip.I32, has_wqf=True, has_calib=True, out_pad=out_pad if k == 1 else (0, 0))
+        okw = dict(stride=(1, 1), pad=(fk // 2,) * 2, out_dt="s8")
+        if is_fused:
+            eltw = r.integers(-128, 128, (B, ofm, H, W)).astype(np.int8)
+            ecal = r.uniform(0.25, 1.0, ofm).astype(np.float32)
+            ebuf = hip.upload(eng, eltw, "fs_b_yx_fsv16")
+            kw.update(act="none", eltw_t=ebuf.tensor, eltw_act="relu", has_eltw_calib=True)
+            okw.update(act="none", eltw=eltw, eltw_act="relu", eltw_calib=ecal)
+        else:
+            kw.update(act="relu")
+            okw.update(act="relu")
+        d = hip.conv_desc(prev_t, w.shape, "s8", **kw)
+        spec.append((d, w, bias, wqf, calib, ecal))
+        bufs.append((hip.Buffer(eng, d.output), ebuf))
+        ref = rc.conv(ref_in, w, bias, wqf=wqf, calib=calib, **okw)
+        refs.append(ref)
+        ref_in, prev_t = ref, hip.Tensor.make(hip.S8, hip.FS_B_YX_FSV16, B, ofm, H, W)  # the next stage reads a dense tensor
+    return xin, spec, bufs, refs
+
+
+@pytest.mark.parametrize("in_dt", [np.uint8, np.int8], ids=["u8", "s8"])
+@pytest.mark.parametrize("stages,fused", [(3, True), (2, True), (3, False), (2, False)], ids=["3fused", "2fused", "3plain", "2plain"])
+def test_bottleneck_tail_chain_matches_the_oracle(eng, stages, fused, in_dt):
+    B, H, W, mid = 3, 13, 11, 64  # 429 pixels: the last granule of 32 is partly filled, granules span rows and images
+    keep = [False] + [True] * (stages - 1)
+    xin, spec, bufs, refs = bottleneck_tail(eng, 21, B, H, W, mid, stages, fused, in_dt)
+    ch = hip.ConvChain(eng, spec, keep)
+    info = ch.info()
+    assert b"conv_chain" in info.kernel_name
+    assert info.ops == sum(2 * r.size * s[1].shape[1] * s[1].shape[2] * s[1].shape[3] for r, s in zip(refs, spec))
+    outs = [b if k else None for (b, _), k in zip(bufs, keep)]
+    ch.enqueue(xin, outs, [e for _, e in bufs])
+    eng.finish()
+    for k in range(stages):
+        if keep[k]:
+            got = hip.download(eng, bufs[k][0])
+            bad = np.argwhere(got != refs[k])
+            assert bad.size == 0, "stage %d: %d of %d differ, first at %s" % (k, len(bad), got.size, bad[0])
+    # the same chain with every result written, into buffers that were dirty
+    ch2 = hip.ConvChain(eng, spec, None)
+    for b, _ in bufs:
+        b.write_raw(np.full(b.nbytes, 0x55, np.uint8))
+    ch2.enqueue(xin, [b for b, _ in bufs], [e for _, e in bufs])
+    eng.finish()
+    for k in range(stages):
+        assert np.array_equal(hip.download(eng, bufs[k][0]), refs[k]), "stage %d (all kept)" % k
+    ch.close(), ch2.close(), xin.close()
+    for b, e in bufs:
+        b.close()
+        if e is not None:
+            e.close()
+
+
+def test_chain_equals_separate_convolutions_on_a_full_size_slice(eng):
+    """56x56 like the first ResNet stage, two images: the chain against the three convolution objects run one by one"""
+    B, H, W, mid = 2, 56, 56, 64
+    xin, spec, bufs, refs = bottleneck_tail(eng, 5, B, H, W, mid, 3, True)
+    ch = hip.ConvChain(eng, spec, [False, True, True])
+    ch.enqueue(xin, [None, bufs[1][0], bufs[2][0]], [e for _, e in bufs])
+    eng.finish()
+    assert np.array_equal(hip.download(eng, bufs[1][0]), refs[1])
+    assert np.array_equal(hip.download(eng, bufs[2][0]), refs[2])
+    # one by one through cldnn_hip_conv_enqueue
+    src = xin
+    for k, (d, w, bias, wqf, calib, ecal) in enumerate(spec):
+        c = hip.Conv(eng, d, w, bias, wqf, calib, ecal)
+        out = hip.Buffer(eng, d.output)
+        c.enqueue(src, out, bufs[k][1])
+        eng.finish()
+        assert np.array_equal(hip.download(eng, out), refs[k])
+        c.close()
+        src = out
+    ch.close()
+
+
+def test_chain_refusals(eng):
+    xin, spec, bufs, refs = bottleneck_tail(eng, 9, 1, 8, 8, 64, 3, True)
+    # a second stage that is not 1x1
+    d3 = hip.conv_desc(hip.Tensor.make(hip.S8, hip.FS_B_YX_FSV16, 1, 64, 8, 8, 1, 1), (64, 64, 3, 3), "s8", pad=(1, 1), bias_dt=hip.I32,
+                       has_wqf=True, has_calib=True, act="relu")
+    bad = [spec[0], (d3,) + spec[0][1:]]
+    with pytest.raises(hip.HipError) as err:
+        hip.ConvChain(eng, bad)
+    assert err.value.status == -6 and "chain" in str(err.value)
+    # the last stage must be kept; a kept stage needs a buffer
+    with pytest.raises(hip.HipError):
+        hip.ConvChain(eng, spec, [False, True, False])
+    ch = hip.ConvChain(eng, spec, [False, True, True])
+    with pytest.raises(hip.HipError):
+        ch.enqueue(xin, [None, None, bufs[2][0]], [e for _, e in bufs])
+    with pytest.raises(hip.HipError):
+        ch.enqueue(xin, [None, bufs[1][0], bufs[2][0]], None)  # the fused stage has no second input
+    ch.close()
+    # a chain of one
+    with pytest.raises(hip.HipError):
+        hip.ConvChain(eng, spec[:1])
