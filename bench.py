@@ -1,12 +1,14 @@
 #!/usr/bin/env python3
 """Benchmark of the quantized convolution hot path on one MI355X.
 
-A "step" is one pass of a whole int8 convolution stack over one batch of synthetic input:
-every layer is one launch of the HIP convolution through the C-ABI, inputs already resident in
-HBM.  Default workload: the 53 convolutions of ResNet-50 at batch 32 with the residual add fused
-into the 16 block-closing 1x1 convolutions (fused_conv_eltwise).
+A "step" is one pass of a whole int8 convolution stack over one batch of synthetic input through
+the C-ABI, inputs already resident in HBM: one launch per layer, or one launch per convolution
+chain where neighbouring layers feed each other (a 3x3 and the 1x1 convolutions behind it).
+Default workload: the 53 convolutions of ResNet-50 at batch 32 with the residual add fused into the
+16 block-closing 1x1 convolutions (fused_conv_eltwise).  The default run also times the other four
+configurations (VGG-16 b16, MobileNet-v2 b32, ResNet-50 b1, the single convolution) more briefly.
 
-Prints ONE JSON line (metric, value, roofline, cpu_baseline, ...).
+Prints ONE JSON line (metric, value, roofline with the dominant kernel, cpu_baseline, other_workloads ...).
 """
 import argparse
 import ctypes as C
@@ -34,9 +36,31 @@ class Layer:
     pass
 
 
-def build_stack(eng, layers, batch, fuse_residual, seed=1337, tile=0, in_dt=np.uint8):
-    """Create device tensors and convolution objects for every layer (seeded synthetic data)."""
+def build_stack(eng, layers, batch, fuse_residual, seed=1337, tile=0, in_dt=np.uint8, chains=True):
+    """Create device tensors and convolution objects for every layer (seeded synthetic data).
+
+    chains: neighbouring layers that feed each other in the network (follows_prev) run as ONE launch of the
+    convolution chain kernel where the library accepts them (a spatial convolution followed by one or two 1x1
+    convolutions); a chained layer reads what the layer before it produced instead of a fresh random tensor, and the
+    result of a chain's first stage, which only the second stage reads, is never written."""
     out = []
+    follows = set()  # indices of layers that run as stage 1 / 2 of a chain
+    if chains and not tile:
+        i = 0
+        while i < len(layers):
+            n = 1
+            if layers[i]["k"] > 1 and layers[i]["groups"] == 1 and layers[i]["ifm"] % 64 == 0:
+                while n < 3 and i + n < len(layers):
+                    l, q = layers[i + n], layers[i + n - 1]
+                    ok = l["follows_prev"] and l["k"] == 1 and l["stride"] == 1 and l["groups"] == 1 and l["ifm"] == q["ofm"] \
+                        and l["in_hw"] == q["out_hw"] and (not q["closes_block"] or fuse_residual)
+                    if not ok:
+                        break
+                    n += 1
+            if n > 1:
+                layers[i] = dict(layers[i], chain_len=n)
+                follows.update(range(i + 1, i + n))
+            i += n
     for i, l in enumerate(layers):
         r = np.random.default_rng(seed + i)
         L = Layer()
@@ -44,7 +68,9 @@ def build_stack(eng, layers, batch, fuse_residual, seed=1337, tile=0, in_dt=np.u
         ifm, ofm, k, g = l["ifm"], l["ofm"], l["k"], l["groups"]
         hw, ohw = l["in_hw"], l["out_hw"]
         lo, hi = (0, 256) if in_dt == np.uint8 else (-128, 128)
-        L.x = r.integers(lo, hi, (batch, ifm, hw, hw), dtype=np.int16).astype(in_dt)
+        L.follows = i in follows
+        L.chain = None
+        L.x = None if L.follows else r.integers(lo, hi, (batch, ifm, hw, hw), dtype=np.int16).astype(in_dt)
         L.w = r.integers(-127, 128, (ofm, ifm // g, k, k), dtype=np.int16).astype(np.int8)
         L.bias = r.integers(-1000, 1001, ofm).astype(np.int32)
         L.wqf = np.ones(ofm, np.float32)
@@ -63,7 +89,12 @@ def build_stack(eng, layers, batch, fuse_residual, seed=1337, tile=0, in_dt=np.u
             kw.update(act=act)
         # zero border as wide as the padding; a first layer (3 input features) takes b_fs_yx_fsv4
         first = ifm <= 4 and g == 1
-        L.xin = hip.upload(eng, L.x, "b_fs_yx_fsv4" if first else "fs_b_yx_fsv16", (l["pad"], l["pad"]))
+        if L.follows:  # reads the int8 tensor of the stage before it, which stays in registers
+            L.xin = None
+            in_tensor = hip.Tensor.make(hip.S8, hip.FS_B_YX_FSV16, batch, ifm, hw, hw)
+        else:
+            L.xin = hip.upload(eng, L.x, "b_fs_yx_fsv4" if first else "fs_b_yx_fsv16", (l["pad"], l["pad"]))
+            in_tensor = L.xin.tensor
         L.ein = None
         if L.fused:
             L.eltw = r.integers(-128, 128, (batch, ofm, ohw, ohw), dtype=np.int16).astype(np.int8)
@@ -73,24 +104,67 @@ def build_stack(eng, layers, batch, fuse_residual, seed=1337, tile=0, in_dt=np.u
         L.kw = kw
         if first:
             kw["out_fmt"] = hip.FS_B_YX_FSV16
-        L.desc = hip.conv_desc(L.xin.tensor, L.w.shape, "s8", tile=0 if first else tile, **kw)
+        L.desc = hip.conv_desc(in_tensor, L.w.shape, "s8", tile=0 if first else tile, **kw)
         try:
             L.conv = hip.Conv(eng, L.desc, L.w, L.bias, L.wqf, L.calib, L.ecal)
         except hip.HipError:
             if not tile:
                 raise
-            L.desc = hip.conv_desc(L.xin.tensor, L.w.shape, "s8", tile=0, **kw)  # forced row not applicable here
+            L.desc = hip.conv_desc(in_tensor, L.w.shape, "s8", tile=0, **kw)  # forced row not applicable here
             L.conv = hip.Conv(eng, L.desc, L.w, L.bias, L.wqf, L.calib, L.ecal)
         L.out = hip.Buffer(eng, L.desc.output)
         L.info = L.conv.info()
+        L.kept = True
         out.append(L)
+    # the chains: three stages where the library takes them, else two, else the layers run one by one
+    for i, L in enumerate(out):
+        n = L.spec.get("chain_len", 1)
+        while n > 1:
+            members = out[i:i + n]
+            keep = [False] + [True] * (n - 1)  # only the next stage reads the first stage's result
+            try:
+                L.chain = hip.ConvChain(eng, [(M.desc, M.w, M.bias, M.wqf, M.calib, M.ecal) for M in members], keep)
+            except hip.HipError as e:
+                if e.status != -6:
+                    raise
+                n -= 1
+                continue
+            L.members = members
+            L.chain_args = L.chain.pointers([M.out if k else None for M, k in zip(members, keep)], [M.ein for M in members])
+            L.info = L.chain.info()
+            L.kept = False
+            for M in members[1:]:
+                M.info = None  # counted in the chain head
+            break
+        if L.chain is None and n == 1 and L.spec.get("chain_len", 1) > 1:
+            log("bench.py: %s and its followers do not chain on this device, running them one by one" % L.spec["name"])
+        if L.chain is None or len(L.members) < L.spec.get("chain_len", 1):
+            # followers that did not make it into a chain need a real input tensor: the layer before them writes it
+            first_loose = i + (len(L.members) if L.chain is not None else 1)
+            for j in range(first_loose, i + L.spec.get("chain_len", 1)):
+                M = out[j]
+                M.follows, M.xin_from = False, out[j - 1]
     return out
 
 
-def run_step(stack):
-    enq = hip.lib().cldnn_hip_conv_enqueue
+def launches(stack):
+    """what one step enqueues: (library function, arguments) per launch"""
+    lib = hip.lib()
+    seq = []
     for L in stack:
-        st = enq(L.conv.h, L.xin.ptr, L.out.ptr, L.ein.ptr if L.ein is not None else None)
+        if L.follows:
+            continue
+        if L.chain is not None:
+            seq.append((lib.cldnn_hip_conv_chain_enqueue, (L.chain.h, L.xin.ptr, L.chain_args[0], L.chain_args[1])))
+        else:
+            src = L.xin.ptr if L.xin is not None else L.xin_from.out.ptr
+            seq.append((lib.cldnn_hip_conv_enqueue, (L.conv.h, src, L.out.ptr, L.ein.ptr if L.ein is not None else None)))
+    return seq
+
+
+def run_step(seq):
+    for fn, args in seq:
+        st = fn(*args)
         if st:
             hip.check(st)
 
@@ -120,20 +194,24 @@ class GpuTimer:
 
 def cpu_pass(eng, stack, images, verify):
     """Run the CPU oracle on the first `images` image(s) of every layer; optionally compare with the
-    GPU results of the same images (a convolution is independent per image)."""
+    GPU results of the same images (a convolution is independent per image).  A layer that runs as a later stage of
+    a chain (or behind a layer whose chain was refused) reads what the oracle computed for the layer before it."""
     from oracle import refconv as rc
     threads = rc.lib().rc_threads_available()
     t_total, checked, mism = 0.0, 0, 0
+    prev = None
     for L in stack:
         l = L.spec
         kw = dict(stride=(l["stride"],) * 2, pad=(l["pad"],) * 2, groups=l["groups"], out_dt="s8",
                   act=L.kw.get("act", "none"), act_m=L.kw.get("act_m", 0.0), act_n=L.kw.get("act_n", 0.0))
         if L.fused:
             kw.update(eltw=L.eltw[:images], eltw_act="relu", eltw_calib=L.ecal)
+        x = L.x[:images] if L.x is not None else prev
         t0 = time.perf_counter()
-        ref = rc.conv(L.x[:images], L.w, L.bias, wqf=L.wqf, calib=L.calib, nthreads=threads, **kw)
+        ref = rc.conv(x, L.w, L.bias, wqf=L.wqf, calib=L.calib, nthreads=threads, **kw)
         t_total += time.perf_counter() - t0
-        if verify:
+        prev = ref
+        if verify and L.kept:
             got = hip.download(eng, L.out)[:images]
             checked += ref.size
             mism += int(np.count_nonzero(ref != got))
@@ -287,15 +365,289 @@ def network_workload(args):
 
 
 def measured_traffic(workload):
-    """HBM bytes per launch from the committed counter summary of this workload (None when there is none)."""
+    """HBM bytes per launch from the committed counter summary of this workload.  None when there is none, or when
+    the summary is older than the kernels: it carries the commit it was taken at, and any later commit that touches
+    cldnn_amd/csrc/ makes it stale."""
     path = os.path.join(ROOT, "profiles", "conv_stack_%s_hbm_traffic.txt" % workload)
     if not os.path.exists(path):
         return None
+    value = commit = None
     with open(path) as f:
         for line in f:
             if line.startswith("traffic_bytes_per_launch:"):
-                return int(line.split(":")[1])
-    return None
+                value = int(line.split(":")[1])
+            if line.startswith("taken_at_commit:"):
+                commit = line.split(":")[1].strip()
+    if value is None or not commit:
+        return None
+    try:
+        import subprocess
+        later = subprocess.run(["git", "-C", ROOT, "log", "--oneline", "%s..HEAD" % commit, "--", "cldnn_amd/csrc"],
+                               stdout=subprocess.PIPE, stderr=subprocess.DEVNULL, text=True, timeout=20)
+        if later.returncode != 0 or later.stdout.strip():
+            return None
+    except Exception:
+        return None  # no git history at hand (a bare copy of the tree): the stamp cannot be checked
+    return value
+
+
+def stack_of(wl):
+    if wl.startswith("resnet50"):
+        return workloads.resnet50(), (1 if wl.endswith("b1") else 32), wl.endswith("fused")
+    if wl == "vgg16_b16":
+        return workloads.vgg16(), 16, False
+    if wl == "mobilenet_v2_b32":
+        return workloads.mobilenet_v2(), 32, False
+    return [workloads._layer("c1", 64, 64, 3, 1, 1, 56)], 1, False
+
+
+def release_stack(stack):
+    for L in stack:
+        if L.chain is not None:
+            L.chain.close()
+        L.conv.close(), L.out.close()
+        if L.xin is not None:
+            L.xin.close()
+        if L.ein is not None:
+            L.ein.close()
+
+
+def time_launches(eng, stack, seq, steps):
+    """GPU time of every launch inside whole steps (so every kernel starts with cold caches, as in the real run):
+    one event pair per launch on the engine's stream.  -> seconds per launch, in launch order"""
+    acc = [0.0] * len(seq)
+    for _ in range(steps):
+        timers = []
+        for fn, a in seq:
+            tmr = GpuTimer(eng)
+            with tmr:
+                st = fn(*a)
+                if st:
+                    hip.check(st)
+            timers.append(tmr)
+        eng.finish()
+        for i, tmr in enumerate(timers):
+            acc[i] += tmr.seconds()
+    return [v / steps for v in acc]
+
+
+def kernel_rooflines(heads, times):
+    """Per kernel instance: launches per step, average duration, algorithmic ops and bytes per launch, and the
+    fraction of the roofline that bounds it (int8 MFMA peak or HBM peak, whichever the layer's work is closer to)."""
+    groups = {}
+    for L, dt in zip(heads, times):
+        g = groups.setdefault(L.info.kernel_name.decode(), dict(n=0, t=0.0, ops=0, bytes=0))
+        g["n"] += 1
+        g["t"] += dt
+        g["ops"] += L.info.ops
+        g["bytes"] += L.info.bytes
+    rows = []
+    for name, g in groups.items():
+        t_m, t_h = g["ops"] / PEAK_INT8_OPS, g["bytes"] / PEAK_HBM
+        bound = "mfma" if t_m > t_h else "hbm"
+        rows.append({"name": name, "launches_per_step": g["n"], "avg_us": g["t"] / g["n"] * 1e6, "share_of_step": 0.0,
+                     "ops_per_launch": g["ops"] / g["n"], "bytes_per_launch": g["bytes"] / g["n"], "bound": bound,
+                     "achieved": g["ops"] / g["t"] / 1e12 if bound == "mfma" else g["bytes"] / g["t"] / 1e9,
+                     "unit": "TOP/s" if bound == "mfma" else "GB/s", "frac": max(t_m, t_h) / g["t"], "_t": g["t"]})
+    total = sum(r["_t"] for r in rows)
+    for r in rows:
+        r["share_of_step"] = r.pop("_t") / total
+    rows.sort(key=lambda r: -r["share_of_step"])
+    return rows
+
+
+def measure_stack(args, wl, steps, warmup, in_flight_n, cpu_seconds, extras):
+    """Build one workload's stack, time `steps` whole steps, per-kernel times, optionally requests in flight and the
+    CPU oracle leg (bounded sample + bit-exact check).  -> result dict, parity ok"""
+    layers, batch, fuse = stack_of(wl)
+    if args.only and extras:
+        keep = set(args.only.split(","))
+        layers = [l for l in layers if l["name"] in keep]
+        if not layers:
+            log("bench.py: no layer of %s is named in --only" % wl)
+            sys.exit(2)
+    eng = hip.Engine(0, profiling=True)
+    t0 = time.perf_counter()
+    stack = build_stack(eng, layers, batch, fuse, tile=args.tile, chains=not args.no_chains)
+    seq = launches(stack)
+    heads = [L for L in stack if not L.follows]
+    eng.finish()
+    log("%s: built %d layers (%d launches per step) in %.1f s" % (wl, len(stack), len(seq), time.perf_counter() - t0))
+
+    ops = sum(L.info.ops for L in heads)
+    nbytes = sum(L.info.bytes for L in heads)
+    for _ in range(warmup):
+        run_step(seq)
+    eng.finish()
+    t_wall0 = time.perf_counter()
+    with GpuTimer(eng) as tm:
+        for _ in range(steps):
+            run_step(seq)
+    eng.finish()
+    t_wall = time.perf_counter() - t_wall0
+    t_gpu = tm.seconds()
+    n_launch = len(seq) * steps
+
+    per_launch = time_launches(eng, stack, seq, max(3, min(10, steps // 4)))
+    kernels = kernel_rooflines(heads, per_launch)
+
+    in_flight = None
+    if in_flight_n > 1 and not args.only:
+        # What an application gets that keeps several requests going (the reference's users run one network per request
+        # and thread): every request has an engine = stream of its own; kernels of different requests overlap on the
+        # device and fill what one request's kernels leave idle.
+        import threading
+        engines = [eng] + [hip.Engine(0, profiling=False) for _ in range(in_flight_n - 1)]
+        stacks = [stack] + [build_stack(e, layers, batch, fuse, seed=1337 + 1000 * (k + 1), tile=args.tile, chains=not args.no_chains)
+                            for k, e in enumerate(engines[1:])]
+        seqs = [seq] + [launches(st) for st in stacks[1:]]
+
+        def request_loop(k, count):
+            for _ in range(count):
+                run_step(seqs[k])
+            engines[k].finish()
+        for k in range(len(engines)):
+            request_loop(k, 5)
+        threads = [threading.Thread(target=request_loop, args=(k, steps)) for k in range(len(engines))]
+        t0 = time.perf_counter()
+        for t in threads:
+            t.start()
+        for t in threads:
+            t.join()
+        dt = time.perf_counter() - t0
+        in_flight = {"requests": len(engines), "steps_per_request": steps, "images_per_s": len(engines) * batch * steps / dt,
+                     "ms_per_request_step": dt / steps * 1e3, "tops": len(engines) * ops * steps / dt / 1e12,
+                     "frac_of_int8_peak": len(engines) * ops * steps / dt / PEAK_INT8_OPS,
+                     "what": "independent requests of this workload, one engine (HIP stream at default priority) and one host thread each"}
+        for st in stacks[1:]:
+            release_stack(st)
+        del stacks, seqs
+        for e in engines[1:]:
+            e.close()
+    host_io = None
+    if args.host_io and extras:
+        # what a caller holding host tensors pays: bfyx input host -> device, device reorder into the blocked layout
+        # with its border, the stack, blocked output device -> host
+        first, last_l = stack[0], stack[-1]
+        plain = hip.Buffer(eng, hip.Tensor.make(first.xin.tensor.dtype, hip.BFYX, *first.x.shape))
+        for _ in range(2):
+            plain.write_raw(first.x); hip.reorder(eng, plain, first.xin); run_step(seq); last_l.out.read_raw()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            plain.write_raw(first.x)
+            hip.reorder(eng, plain, first.xin)
+            run_step(seq)
+            last_l.out.read_raw()
+        dt = time.perf_counter() - t0
+        host_io = {"images_per_s": batch * steps / dt, "ms_per_step": dt / steps * 1e3,
+                   "host_to_device_bytes": int(first.x.nbytes), "device_to_host_bytes": int(last_l.out.nbytes)}
+        plain.close()
+
+    def table(stk, times):
+        log("%-18s %-52s %6s %9s %8s %8s %7s" % ("layer", "kernel", "grid", "us", "TOP/s", "GB/s", "bound"))
+        for L, dt in zip(stk, times):
+            tops, gbs = L.info.ops / dt / 1e12, L.info.bytes / dt / 1e9
+            t_m, t_h = L.info.ops / PEAK_INT8_OPS, L.info.bytes / PEAK_HBM
+            name = L.spec["name"] + ("+%d" % (len(L.members) - 1) if L.chain is not None else "")
+            log("%-18s %-52s %6d %9.1f %8.1f %8.0f %7s %5.1f%%" % (
+                name, L.info.kernel_name.decode(), L.info.grid, dt * 1e6, tops, gbs,
+                "mfma" if t_m > t_h else "hbm", 100 * max(t_m, t_h) / dt))
+        log("sum of per-launch times: %.1f us" % (sum(times) * 1e6))
+
+    if (args.per_layer or args.tune) and extras:
+        table(heads, per_launch)
+        if args.tune:
+            # every row of the tile table forced on every layer where it applies (no chains); report the best row per layer
+            names = [hip.lib().cldnn_hip_tile_config_name(i).decode() for i in range(hip.lib().cldnn_hip_tile_config_count())]
+            base = build_stack(eng, layers, batch, fuse, chains=False)
+            bseq = launches(base)
+            run_step(bseq)
+            base_t = time_launches(eng, base, bseq, max(3, steps // 3))
+            best = [(t, "table:" + L.info.kernel_name.decode()) for t, L in zip(base_t, base)]
+            for row in range(1, len(names) + 1):
+                alt = build_stack(eng, layers, batch, fuse, tile=row, chains=False)
+                aseq = launches(alt)
+                for _ in range(2):
+                    run_step(aseq)
+                times = time_launches(eng, alt, aseq, max(3, steps // 3))
+                for i, (t, L) in enumerate(zip(times, alt)):
+                    if L.info.tile_index == row - 1 and t < best[i][0]:
+                        best[i] = (t, names[row - 1])
+                release_stack(alt)
+            log("%-18s %6s %6s %5s %3s %9s %9s  %s" % ("layer", "M", "OFM", "K", "k", "table us", "best us", "best row"))
+            for L, t0, (t1, nm) in zip(base, base_t, best):
+                l = L.spec
+                log("%-18s %6d %6d %5d %3d %9.1f %9.1f  %s" % (l["name"], batch * l["out_hw"] ** 2, l["ofm"],
+                                                             l["ifm"] * l["k"] ** 2, l["k"], t0 * 1e6, t1 * 1e6, nm))
+            log("sum with the table: %.1f us; sum of per-layer bests: %.1f us" % (sum(base_t) * 1e6, sum(t for t, _ in best) * 1e6))
+            release_stack(base)
+
+    dom = kernels[0]
+    # the roofline the workload is priced against: the dense stacks against the int8 matrix peak (the baseline's
+    # metric), the depthwise / 1x1 network and the batch-1 stack (weights dominate) against HBM
+    hbm_bound = wl in ("mobilenet_v2_b32", "resnet50_b1")
+    res = {
+        "value": batch * steps / t_wall,
+        "unit": "images/s",
+        "steps": steps,
+        "warmup": warmup,
+        "ms_per_step": t_wall / steps * 1e3,
+        "config": {"workload": wl, "batch": batch, "layers": len(stack), "launches_per_step": len(seq),
+                   "chained_layers": sum(len(L.members) for L in stack if L.chain is not None),
+                   "layout": "fs_b_yx_fsv16",
+                   "variant": "stride on the first 1x1 (Caffe form)" if wl.startswith("resnet50") else wl,
+                   "fused_residual_layers": sum(1 for L in stack if L.fused)},
+        "achieved_tops": ops * steps / t_gpu / 1e12,
+        "roofline": {
+            "bound": "hbm" if hbm_bound else "mfma",
+            "achieved": nbytes * steps / t_gpu / 1e9 if hbm_bound else ops * steps / t_gpu / 1e12,
+            "peak": PEAK_HBM / 1e9 if hbm_bound else PEAK_INT8_OPS / 1e12,
+            "unit": "GB/s" if hbm_bound else "TOP/s",
+            "frac": nbytes * steps / t_gpu / PEAK_HBM if hbm_bound else ops * steps / t_gpu / PEAK_INT8_OPS,
+            "traffic": measured_traffic(wl),
+            "kernel": "all convolution kernels of the step",
+            "launches": n_launch,
+            "avg_launch_us": t_gpu / n_launch * 1e6,
+            "ops_per_launch": ops / len(seq),
+            "bytes_per_launch": nbytes / len(seq),
+            "dominant_kernel": dom,
+            "kernels": kernels[1:6],
+        },
+        "roofline_hbm": {
+            "bound": "hbm",
+            "achieved": nbytes * steps / t_gpu / 1e9,
+            "peak": PEAK_HBM / 1e9,
+            "unit": "GB/s",
+            "frac": nbytes * steps / t_gpu / PEAK_HBM,
+            "bytes_per_launch": nbytes / len(seq),
+        },
+        "gpu_seconds_events": t_gpu,
+        "wall_seconds": t_wall,
+    }
+    if host_io:
+        res["pcie_inclusive"] = host_io
+    if in_flight:
+        res["requests_in_flight"] = in_flight
+    ok = True
+    if cpu_seconds > 0:
+        cb = cpu_baseline_and_check(eng, stack, batch, cpu_seconds)
+        res["cpu_baseline"] = {
+            "value": cb["images"] / cb["seconds"],
+            "unit": "images/s",
+            "cores": cb["threads"],
+            "kind": "port",
+            "sample": "first %d image(s) of every layer of the same stack through oracle/refconv.c "
+                      "(OpenMP over batch x ofm), %.1f s on %d threads = %.0f s of CPU work" % (cb["images"], cb["seconds"], cb["threads"], cb["seconds"] * cb["threads"]),
+        }
+        res["verified"] = {"outputs_compared": cb["checked"], "mismatches": cb["mismatches"],
+                           "what": "GPU batch-%d results of the first %d image(s), every tensor the step writes, vs the CPU "
+                                   "oracle run layer by layer (bit-exact)" % (batch, cb["images"])}
+        if cb["mismatches"]:
+            log("PARITY FAILURE in %s: %d mismatching outputs" % (wl, cb["mismatches"]))
+            ok = False
+    release_stack(stack)
+    eng.close()
+    return res, ok
 
 
 def main():
@@ -306,8 +658,9 @@ def main():
     ap.add_argument("--workload", default="resnet50_b32_fused",
                     choices=["resnet50_b32_fused", "resnet50_b32", "resnet50_b1", "vgg16_b16", "mobilenet_v2_b32", "c1",
                              "copy_256m", "resnet50_b32_network", "mobilenet_v2_b32_network", "vgg16_b16_network"])
-    ap.add_argument("--tile", type=int, default=0, help="force one row (index+1) of the tile table on every layer")
-    ap.add_argument("--per-layer", action="store_true", help="time every layer on its own and print a table to stderr")
+    ap.add_argument("--tile", type=int, default=0, help="force one row (index+1) of the tile table on every layer (no chains)")
+    ap.add_argument("--no-chains", action="store_true", help="every layer is a launch of its own (no convolution chains)")
+    ap.add_argument("--per-layer", action="store_true", help="print the per-launch table to stderr")
     ap.add_argument("--tune", action="store_true", help="try every row of the tile table on every layer, print the best")
     ap.add_argument("--only", default="", help="comma-separated layer names: run just these layers of the workload "
                                                "(same buffers every step, so their tensors stay cache-resident)")
@@ -320,6 +673,7 @@ def main():
                          "flight at once, one engine (HIP stream) and one host thread each; reported under "
                          "requests_in_flight, never as the headline value (0 or 1 = skip)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline / full-size check")
+    ap.add_argument("--no-others", action="store_true", help="default workload only: do not time the other four configurations")
     ap.add_argument("--host-io", action="store_true",
                     help="also report the rate with the first layer's input crossing PCIe into the device and the last "
                          "layer's output crossing back, every step (never the headline value)")
@@ -335,216 +689,33 @@ def main():
         return copy_calibration(args)
     if wl.endswith("_network"):
         return network_workload(args)
-    if wl.startswith("resnet50"):
-        layers, batch, fuse = workloads.resnet50(), (1 if wl.endswith("b1") else 32), wl.endswith("fused")
-    elif wl == "vgg16_b16":
-        layers, batch, fuse = workloads.vgg16(), 16, False
-    elif wl == "mobilenet_v2_b32":
-        layers, batch, fuse = workloads.mobilenet_v2(), 32, False
-    else:
-        layers, batch, fuse = [workloads._layer("c1", 64, 64, 3, 1, 1, 56)], 1, False
 
-    if args.only:
-        keep = set(args.only.split(","))
-        layers = [l for l in layers if l["name"] in keep]
-        if not layers:
-            log("bench.py: no layer of %s is named in --only" % wl)
-            sys.exit(2)
-
-    eng = hip.Engine(0, profiling=True)
-    info = eng.info()
-    log("device: %s (%s), %d CUs @ %d MHz" % (info.name.decode(), info.arch.decode(), info.cores_count, info.core_frequency))
-    t0 = time.perf_counter()
-    stack = build_stack(eng, layers, batch, fuse, tile=args.tile)
-    eng.finish()
-    log("built %d layers in %.1f s" % (len(stack), time.perf_counter() - t0))
-
-    ops = sum(L.info.ops for L in stack)
-    nbytes = sum(L.info.bytes for L in stack)
-
-    for _ in range(args.warmup):
-        run_step(stack)
-    eng.finish()
-    t_wall0 = time.perf_counter()
-    with GpuTimer(eng) as tm:
-        for _ in range(args.steps):
-            run_step(stack)
-    eng.finish()
-    t_wall = time.perf_counter() - t_wall0
-    t_gpu = tm.seconds()
-    launches = len(stack) * args.steps
-    ms_per_step = t_wall / args.steps * 1e3
-    value = batch * args.steps / t_wall
-
-    in_flight = None
-    if args.in_flight > 1 and not args.only:
-        # What an application gets that keeps several requests going (the reference's users run one network per request
-        # and thread): every request has an engine = stream of its own; kernels of different requests overlap on the
-        # device and fill what one request's kernels leave idle.
-        import threading
-        engines = [eng] + [hip.Engine(0, profiling=False) for _ in range(args.in_flight - 1)]
-        stacks = [stack] + [build_stack(e, layers, batch, fuse, seed=1337 + 1000 * (k + 1), tile=args.tile) for k, e in enumerate(engines[1:])]
-
-        def request_loop(k, count):
-            for _ in range(count):
-                run_step(stacks[k])
-            engines[k].finish()
-        for k in range(len(engines)):
-            request_loop(k, 5)
-        threads = [threading.Thread(target=request_loop, args=(k, args.steps)) for k in range(len(engines))]
-        t0 = time.perf_counter()
-        for t in threads:
-            t.start()
-        for t in threads:
-            t.join()
-        dt = time.perf_counter() - t0
-        in_flight = {"requests": len(engines), "steps_per_request": args.steps, "images_per_s": len(engines) * batch * args.steps / dt,
-                     "ms_per_request_step": dt / args.steps * 1e3, "tops": len(engines) * ops * args.steps / dt / 1e12,
-                     "frac_of_int8_peak": len(engines) * ops * args.steps / dt / PEAK_INT8_OPS,
-                     "what": "independent requests of this workload, one engine (HIP stream at default priority) and one host thread each"}
-        for L in [L for st in stacks[1:] for L in st]:
-            L.conv.close(), L.out.close(), L.xin.close()
-            if L.ein is not None:
-                L.ein.close()
-        del stacks
-        for e in engines[1:]:
-            e.close()
-    host_io = None
-    if args.host_io:
-        # what a caller holding host tensors pays: bfyx input host -> device, device reorder into the blocked layout
-        # with its border, the stack, blocked output device -> host
-        first, last_l = stack[0], stack[-1]
-        plain = hip.Buffer(eng, hip.Tensor.make(first.xin.tensor.dtype, hip.BFYX, *first.x.shape))
-        for _ in range(2):
-            plain.write_raw(first.x); hip.reorder(eng, plain, first.xin); run_step(stack); last_l.out.read_raw()
-        t0 = time.perf_counter()
-        for _ in range(args.steps):
-            plain.write_raw(first.x)
-            hip.reorder(eng, plain, first.xin)
-            run_step(stack)
-            last_l.out.read_raw()
-        dt = time.perf_counter() - t0
-        host_io = {"images_per_s": batch * args.steps / dt, "ms_per_step": dt / args.steps * 1e3,
-                   "host_to_device_bytes": int(first.x.nbytes), "device_to_host_bytes": int(last_l.out.nbytes)}
-        plain.close()
-
-    per_layer = None
-    if args.per_layer or args.tune:
-        def time_layers(stk, steps):
-            """per-layer GPU time inside whole steps (so every layer starts with cold caches, as in the real run)"""
-            acc = [0.0] * len(stk)
-            for _ in range(steps):
-                timers = []
-                for L in stk:
-                    tmr = GpuTimer(eng)
-                    with tmr:
-                        L.conv.enqueue(L.xin, L.out, L.ein)
-                    timers.append(tmr)
-                eng.finish()
-                for i, tmr in enumerate(timers):
-                    acc[i] += tmr.seconds()
-            return [v / steps for v in acc]
-
-        def table(stk, times):
-            log("%-18s %-40s %6s %9s %8s %8s %7s" % ("layer", "kernel", "grid", "us", "TOP/s", "GB/s", "bound"))
-            for L, dt in zip(stk, times):
-                tops, gbs = L.info.ops / dt / 1e12, L.info.bytes / dt / 1e9
-                t_m, t_h = L.info.ops / PEAK_INT8_OPS, L.info.bytes / PEAK_HBM
-                log("%-18s %-40s %6d %9.1f %8.1f %8.0f %7s %5.1f%%" % (
-                    L.spec["name"], L.info.kernel_name.decode(), L.info.grid, dt * 1e6, tops, gbs,
-                    "mfma" if t_m > t_h else "hbm", 100 * max(t_m, t_h) / dt))
-            log("sum of per-layer times: %.1f us" % (sum(times) * 1e6))
-
-        per_layer = time_layers(stack, max(3, args.steps // 3))
-        table(stack, per_layer)
-        if args.tune:
-            # every row of the tile table forced on every layer where it applies; report the best row per layer
-            names = [hip.lib().cldnn_hip_tile_config_name(i).decode() for i in range(hip.lib().cldnn_hip_tile_config_count())]
-            best = [(t, "table:" + L.info.kernel_name.decode()) for t, L in zip(per_layer, stack)]
-            for row in range(1, len(names) + 1):
-                alt = build_stack(eng, layers, batch, fuse, tile=row)
-                for _ in range(2):
-                    run_step(alt)
-                times = time_layers(alt, max(3, args.steps // 3))
-                for i, (t, L) in enumerate(zip(times, alt)):
-                    if L.info.tile_index == row - 1 and t < best[i][0]:
-                        best[i] = (t, names[row - 1])
-                for L in alt:
-                    L.conv.close(); L.out.close(); L.xin.close()
-                    if L.ein is not None:
-                        L.ein.close()
-            log("%-18s %6s %6s %5s %3s %9s %9s  %s" % ("layer", "M", "OFM", "K", "k", "table us", "best us", "best row"))
-            for L, t0, (t1, nm) in zip(stack, per_layer, best):
-                l = L.spec
-                log("%-18s %6d %6d %5d %3d %9.1f %9.1f  %s" % (l["name"], batch * l["out_hw"] ** 2, l["ofm"],
-                                                             l["ifm"] * l["k"] ** 2, l["k"], t0 * 1e6, t1 * 1e6, nm))
-            log("sum with the table: %.1f us; sum of per-layer bests: %.1f us" % (sum(per_layer) * 1e6, sum(t for t, _ in best) * 1e6))
-
-    res = {
+    res, ok = measure_stack(args, wl, args.steps, args.warmup, args.in_flight, 0.0 if args.no_cpu else args.cpu_seconds, True)
+    line = {
         "metric": "ResNet-50 int8 conv stack images/sec @b32; achieved TOPS vs INT8 MFMA peak"
         if wl.startswith("resnet50_b32") else "int8 conv stack images/sec",
-        "value": value,
-        "unit": "images/s",
-        "n_gpus": 1,
-        "steps": args.steps,
-        "warmup": args.warmup,
-        "ms_per_step": ms_per_step,
-        "higher_is_better": True,
-        "scaling": "weak",
-        "vs_baseline": None,
-        "dtype": "i8xi8->i32 (f32 requantisation)",
-        "data": "synthetic",
-        "config": {"workload": wl, "batch": batch, "layers": len(stack), "layout": "fs_b_yx_fsv16",
-                   "variant": "stride on the first 1x1 (Caffe form)" if wl.startswith("resnet50") else wl,
-                   "fused_residual_layers": sum(1 for L in stack if L.fused)},
-        "achieved_tops": ops * args.steps / t_gpu / 1e12,
-        "roofline": {
-            "bound": "mfma",
-            "achieved": ops * args.steps / t_gpu / 1e12,
-            "peak": PEAK_INT8_OPS / 1e12,
-            "unit": "TOP/s",
-            "frac": ops * args.steps / t_gpu / PEAK_INT8_OPS,
-            "traffic": measured_traffic(wl),
-            "kernel": "convolution kernels of the step (all instances of the tile table)",
-            "launches": launches,
-            "avg_launch_us": t_gpu / launches * 1e6,
-            "ops_per_launch": ops / len(stack),
-        },
-        "roofline_hbm": {
-            "bound": "hbm",
-            "achieved": nbytes * args.steps / t_gpu / 1e9,
-            "peak": PEAK_HBM / 1e9,
-            "unit": "GB/s",
-            "frac": nbytes * args.steps / t_gpu / PEAK_HBM,
-            "bytes_per_launch": nbytes / len(stack),
-        },
-        "gpu_seconds_events": t_gpu,
-        "wall_seconds": t_wall,
+        "value": res.pop("value"), "unit": res.pop("unit"), "n_gpus": 1, "steps": res.pop("steps"), "warmup": res.pop("warmup"),
+        "ms_per_step": res.pop("ms_per_step"), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "i8xi8->i32 (f32 requantisation)", "data": "synthetic",
     }
-    if host_io:
-        res["pcie_inclusive"] = host_io
-    if in_flight:
-        res["requests_in_flight"] = in_flight
-
-    if not args.no_cpu:
-        cb = cpu_baseline_and_check(eng, stack, batch, args.cpu_seconds)
-        res["cpu_baseline"] = {
-            "value": cb["images"] / cb["seconds"],
-            "unit": "images/s",
-            "cores": cb["threads"],
-            "kind": "port",
-            "sample": "first %d image(s) of every layer of the same stack through oracle/refconv.c "
-                      "(OpenMP over batch x ofm), %.1f s on %d threads = %.0f s of CPU work" % (cb["images"], cb["seconds"], cb["threads"], cb["seconds"] * cb["threads"]),
-        }
-        res["verified"] = {"outputs_compared": cb["checked"], "mismatches": cb["mismatches"],
-                           "what": "GPU batch-%d results of the first %d image(s), every layer, vs the CPU oracle "
-                                   "(bit-exact)" % (batch, cb["images"])}
-        if cb["mismatches"]:
-            log("PARITY FAILURE: %d mismatching outputs" % cb["mismatches"])
-    print(json.dumps(res), flush=True)
-    for L in stack:
-        L.conv.close()
-    if not args.no_cpu and res["verified"]["mismatches"]:
+    line.update(res)
+    if wl == "resnet50_b32_fused" and not args.no_others and not args.only and not args.tune:
+        # the other four configurations of the baseline, shorter runs, same measurement (a CPU sample of a few seconds each)
+        others = {}
+        for other in ("vgg16_b16", "mobilenet_v2_b32", "resnet50_b1", "c1"):
+            r, ok2 = measure_stack(args, other, max(20, args.steps // 4), max(5, args.warmup // 4), 0,
+                                   0.0 if args.no_cpu else min(args.cpu_seconds, 4.0), False)
+            ok = ok and ok2
+            keep = {k: r[k] for k in ("ms_per_step", "achieved_tops", "config")}
+            keep["images_per_s"] = r["value"]
+            keep["roofline"] = {k: r["roofline"][k] for k in ("bound", "achieved", "peak", "unit", "frac", "dominant_kernel")}
+            for k in ("cpu_baseline", "verified"):
+                if k in r:
+                    keep[k] = r[k]
+            others[other] = keep
+        line["other_workloads"] = others
+    print(json.dumps(line), flush=True)
+    if not ok:
         sys.exit(1)
 
 

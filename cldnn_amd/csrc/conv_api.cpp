@@ -418,8 +418,18 @@ cldnn_hip_status cldnn_hip_conv_chain_create(cldnn_hip_engine e, int32_t count, 
             std::vector<int8_t> packed(chain_packed_bytes(ch->plan));
             const int8_t* w8[3] = {nullptr, nullptr, nullptr};
             for (int k = 0; k < count; ++k) w8[k] = (const int8_t*)weights[k];
-            chain_pack_weights(ch->in, ch->plan, cus, w8, packed.data());
+            // the accumulator start values exist on the device only (the stage objects folded offset correction and bias)
             e->make_current();
+            std::vector<std::vector<int32_t>> init(count);
+            ChainVectors vec[3]{};
+            for (int k = 0; k < count; ++k) {
+                init[k].resize(descs[k].ofm);
+                CHIP_CHECK(hipMemcpy(init[k].data(), ch->stage[k]->acc_init, (size_t)descs[k].ofm * 4, hipMemcpyDeviceToHost));
+                const bool calib_on = ch->stage[k]->epi.calib != nullptr;
+                vec[k] = ChainVectors{init[k].data(), calib_on && calib ? calib[k] : nullptr, eltw_calib ? eltw_calib[k] : nullptr,
+                                      wqf ? wqf[k] : nullptr};
+            }
+            chain_pack_weights(ch->in, ch->plan, cus, w8, vec, packed.data());
             CHIP_CHECK(hipMalloc(&ch->packed, packed.size()));
             CHIP_CHECK(hipMemcpyAsync(ch->packed, packed.data(), packed.size(), hipMemcpyHostToDevice, e->stream));
             CHIP_CHECK(hipStreamSynchronize(e->stream));

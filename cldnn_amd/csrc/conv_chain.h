@@ -36,8 +36,17 @@ struct ChainPlan {
 // empty string: the chain can run and *out is filled; otherwise the reason why not
 std::string chain_plan(const ChainStageIn* st, int n, int cus, ChainPlan* out);
 size_t chain_packed_bytes(const ChainPlan& pl);
-// w[k]: dense host weights of stage k, [ofm][ifm][fy][fx]
-void chain_pack_weights(const ChainStageIn* st, const ChainPlan& pl, int cus, const int8_t* const* w, int8_t* packed);
+// host copies of one stage's per-feature vectors, OFM entries each (nullptr: absent)
+struct ChainVectors {
+    const int32_t* acc_init;
+    const float* calib;
+    const float* eltw_calib;
+    const float* wqf;
+};
+// w[k]: dense host weights of stage k, [ofm][ifm][fy][fx].  The image is what a workgroup copies into LDS: the weight
+// units of all stages, then their per-feature vectors.
+void chain_pack_weights(const ChainStageIn* st, const ChainPlan& pl, int cus, const int8_t* const* w, const ChainVectors* vec,
+                        int8_t* packed);
 // outs[k] == nullptr: stage k's result is not written; eltws[k]: residual operand of a fused stage
 void launch_conv_chain(hipStream_t s, const ChainStageIn* st, const ChainPlan& pl, const void* packed_dev, const void* in,
                        void* const* outs, const void* const* eltws);

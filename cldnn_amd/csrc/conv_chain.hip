@@ -64,7 +64,7 @@ std::string chain_plan(const ChainStageIn* st, int n, int cus, ChainPlan* out)
         if (st[k].fe->fc) return at + "the fully_connected form is not chained";
         if (p.groups != 1) return at + "grouped convolution";
         if (p.in_t.format != CLDNN_HIP_FMT_FS_B_YX_FSV16 || p.out_t.format != CLDNN_HIP_FMT_FS_B_YX_FSV16) return at + "needs fs_b_yx_fsv16";
-        if (((p.IFM + 15) / 16) % 4 != 0) return at + "input features must come in multiples of 64";
+        if (p.IFM % 64 != 0 || p.OFM % 64 != 0) return at + "feature counts must be multiples of 64";
         if (st[k].fe->fused && (p.esy != 1 || p.esx != 1 || p.eltw_t.format != CLDNN_HIP_FMT_FS_B_YX_FSV16)) return at + "strided or unblocked residual";
         if (tensor_elems(p.out_t) >= (1ull << 31) || tensor_elems(p.in_t) >= (1ull << 31)) return at + "tensor of 2 GiB or more";
         if (k > 0) {
@@ -114,11 +114,29 @@ std::string chain_plan(const ChainStageIn* st, int n, int cus, ChainPlan* out)
     return std::string();
 }
 
-size_t chain_packed_bytes(const ChainPlan& pl) { return (size_t)pl.units * 4096 + 4096; }
+size_t chain_packed_bytes(const ChainPlan& pl) { return (size_t)pl.lds_bytes + 4096; }
 
-void chain_pack_weights(const ChainStageIn* st, const ChainPlan& pl, int cus, const int8_t* const* w, int8_t* packed)
+void chain_pack_weights(const ChainStageIn* st, const ChainPlan& pl, int cus, const int8_t* const* w, const ChainVectors* vec,
+                        int8_t* packed)
 {
     std::memset(packed, 0, chain_packed_bytes(pl));
+    // per-feature vectors behind the weight units: per stage init, calib, eltw_calib, wqf, spans * 64 entries each
+    int32_t* v = reinterpret_cast<int32_t*>(packed + (size_t)pl.units * 4096);
+    const float one = 1.0f;
+    int32_t one_bits;
+    std::memcpy(&one_bits, &one, 4);
+    for (int k = 0; k < pl.stages; ++k) {
+        const int n = pl.sp[k] * 64, ofm = st[k].p->OFM;
+        const void* src[4] = {vec[k].acc_init, vec[k].calib, vec[k].eltw_calib, vec[k].wqf};
+        for (int kind = 0; kind < 4; ++kind) {
+            int32_t* dst = v + pl.vec0[k] + kind * n;
+            // without calibration factors the epilogue multiplies by the output quantization factor (or by one)
+            int32_t fill = kind == 0 ? 0 : one_bits;
+            if (kind == 1 && !src[kind] && st[k].epi->oqf_on) std::memcpy(&fill, &st[k].epi->oqf, 4);
+            for (int f = 0; f < n; ++f) dst[f] = fill;
+            if (src[kind]) std::memcpy(dst, src[kind], (size_t)ofm * 4);
+        }
+    }
     for (int k = 0; k < pl.stages; ++k) {
         const MfmaPlan mp = mfma_plan(*st[k].p, ROW_WSL_P64_FOR_CHAIN, cus);
         std::vector<int8_t> buf(mp.packed_bytes);
@@ -136,6 +154,7 @@ void launch_conv_chain(hipStream_t s, const ChainStageIn* st, const ChainPlan& p
     a.in = (const int8_t*)in;
     a.wpk = (const v4i*)packed_dev;
     a.units = pl.units;
+    a.vec_quads = (pl.lds_bytes - pl.units * 4096) / 16;
     a.granules = pl.granules;
     a.M = (uint32_t)pl.m_total;
     a.OHW = p0.OH * p0.OW, a.OW = p0.OW;
@@ -147,7 +166,6 @@ void launch_conv_chain(hipStream_t s, const ChainStageIn* st, const ChainPlan& p
     for (int k = 0; k < pl.stages; ++k) {
         const ConvProblem& p = *st[k].p;
         ChainStage& c = a.st[k];
-        c.acc_init = st[k].acc_init;
         c.out = outs[k];
         c.eltw = eltws ? eltws[k] : nullptr;
         CHIP_REQUIRE(!st[k].fe->fused || c.eltw, CLDNN_HIP_INVALID_ARG, "fused stage of a chain without its second input");

@@ -11,7 +11,7 @@
 //
 // Work split: persistent workgroups of four INDEPENDENT waves.  All weights of all stages (a few tens of KB) and
 // the per-feature vectors are copied into LDS once per workgroup; after that a wave walks over its own range of
-// 16*NT-pixel granules without any barrier.  Stage 0 reads its activations straight from global memory, D K-steps
+// 16*NT-pixel granules without any barrier.  Feature counts are multiples of 64.  Stage 0 reads its activations straight from global memory, D K-steps
 // ahead of their use, and the look-ahead runs across granule boundaries (as in the weights-stationary kernel).
 // Every stage has its own epilogue kind, per-feature vectors, output tensor and (optional) residual tensor.
 #pragma once
@@ -25,7 +25,6 @@ namespace chip {
 enum { CHAIN_MAX_STAGES = 3 };
 
 struct ChainStage {
-    const int32_t* acc_init;   // [spans * 64] accumulator start values (offset correction + int32 bias)
     void* out;                 // nullptr: the result of this stage is not materialised
     const void* eltw;          // residual operand of a fused stage
     int32_t OFM;
@@ -41,8 +40,9 @@ struct ChainStage {
 
 struct ChainArgs {
     const int8_t* in;
-    const v4i* wpk;            // LDS image of the weights: unit after unit, [unit][kq][64 rows] x 16 bytes
+    const v4i* wpk;            // LDS image: weight units [unit][kq][64 rows] x 16 bytes, then the per-feature vectors
     int32_t units;
+    int32_t vec_quads;         // 16-byte pieces of per-feature vectors behind the units
     int32_t granules;          // ceil(M / (16 * NT))
     uint32_t M;
     int32_t OHW, OW;
@@ -130,37 +130,29 @@ __global__ void __launch_bounds__(256) conv_chain_kernel(ChainArgs a)
     v4i* ldsW = reinterpret_cast<v4i*>(smem);                              // [units][4][64]
     int32_t* ldsV = reinterpret_cast<int32_t*>(smem + (size_t)a.units * 4096);  // per-feature vectors
     {
-        const int total = a.units * 256;
-        for (int i = t; i < total; i += 8 * 256) {  // eight requests in flight per thread
-            v4i r[8];
+        // one bulk copy: the image holds the weight units and, behind them, the per-feature vectors of all stages
+        // (absent vectors filled with their neutral values by the host); all requests of a thread are in flight at once
+        const int total = a.units * 256 + a.vec_quads;
+        constexpr int BATCH = 20;
+        for (int i = t; i < total; i += BATCH * 256) {
+            v4i r[BATCH];
 #pragma unroll
-            for (int u = 0; u < 8; ++u) r[u] = a.wpk[min(i + u * 256, total - 1)];
+            for (int u = 0; u < BATCH; ++u) r[u] = a.wpk[min(i + u * 256, total - 1)];
 #pragma unroll
-            for (int u = 0; u < 8; ++u)
+            for (int u = 0; u < BATCH; ++u)
                 if (i + u * 256 < total) ldsW[i + u * 256] = r[u];
-        }
-        auto copy_vec = [&](const ChainStage& st, int spans, int kind, const void* src, int32_t neutral) {
-            for (int i = t; i < spans * 64; i += 256)
-                ldsV[st.vec0 + kind * spans * 64 + i] = src ? reinterpret_cast<const int32_t*>(src)[i] : neutral;
-        };
-        const int32_t one = __float_as_int(1.0f);
-        copy_vec(s0, SP0, 0, s0.acc_init, 0), copy_vec(s0, SP0, 1, s0.epi.calib, one);
-        copy_vec(s0, SP0, 2, s0.epi.eltw_calib, one), copy_vec(s0, SP0, 3, s0.epi.wqf, one);
-        copy_vec(s1, SP1, 0, s1.acc_init, 0), copy_vec(s1, SP1, 1, s1.epi.calib, one);
-        copy_vec(s1, SP1, 2, s1.epi.eltw_calib, one), copy_vec(s1, SP1, 3, s1.epi.wqf, one);
-        if constexpr (SP2 > 0) {
-            copy_vec(s2, SP2, 0, s2.acc_init, 0), copy_vec(s2, SP2, 1, s2.epi.calib, one);
-            copy_vec(s2, SP2, 2, s2.epi.eltw_calib, one), copy_vec(s2, SP2, 3, s2.epi.wqf, one);
         }
     }
 
     // Every die gets one contiguous run of workgroups, every wave one contiguous range of granules: rows that
-    // share filter taps stay inside one die's L2.
+    // share filter taps stay inside one die's L2.  (A shared counter that hands out granules one by one was tried:
+    // device-scope atomics on a handful of addresses take about 0.2 us each, one after the other, which cost four
+    // times what the better balance saved.)
     const int per_xcd = gridDim.x >> 3;  // the grid is a multiple of 8
     const uint32_t vb = (blockIdx.x & 7u) * (uint32_t)per_xcd + (blockIdx.x >> 3);
     const uint32_t gw = vb * 4u + (uint32_t)wave, waves = gridDim.x * 4u;
     const int g_begin = (int)(((uint64_t)gw * (uint32_t)a.granules) / waves);
-    const int g_end = (int)(((uint64_t)(gw + 1) * (uint32_t)a.granules) / waves);
+    const int g1 = (int)(((uint64_t)(gw + 1) * (uint32_t)a.granules) / waves);
 
     const v4i xm0 = {(int)s0.xor_mask, (int)s0.xor_mask, (int)s0.xor_mask, (int)s0.xor_mask};
     const v4i xm1 = {(int)s1.xor_mask, (int)s1.xor_mask, (int)s1.xor_mask, (int)s1.xor_mask};
@@ -175,7 +167,7 @@ __global__ void __launch_bounds__(256) conv_chain_kernel(ChainArgs a)
 #pragma unroll
         for (int nt = 0; nt < NT; ++nt) {
             const uint32_t m = (uint32_t)g * WP + nt * 16 + l16;
-            const bool ok = g < g_end && m < a.M;
+            const bool ok = g < g1 && m < a.M;
             const PixelPos pp = chain_pixel_pos(a, ok ? m : 0);
             r.boff[nt] = (uint32_t)(a.in_off + (int)pp.b * a.in_pb + ((int)pp.oy * a.sy - a.py) * a.in_py
                                     + ((int)pp.ox * a.sx - a.px) * 16 + kq * a.in_pf);
@@ -199,12 +191,11 @@ __global__ void __launch_bounds__(256) conv_chain_kernel(ChainArgs a)
     auto unit = [&](const ChainStage& st, int span, int ks) { return ldsW + (size_t)(st.unit0 + span * st.kstride + ks) * 256; };
     auto residual = [&](const ChainStage& st, int ebase, int span) {
         v4i v = {0, 0, 0, 0};
-        if (st.fe.fused && span * 64 + kq * 16 < st.OFM)
-            v = *reinterpret_cast<const v4i*>((const int8_t*)st.eltw + ebase + span * 4 * st.el_pf);
+        if (st.fe.fused) v = *reinterpret_cast<const v4i*>((const int8_t*)st.eltw + ebase + span * 4 * st.el_pf);
         return v;
     };
 
-    if (g_begin >= g_end) {
+    if (g_begin >= g1) {
         __syncthreads();
         return;
     }
@@ -220,7 +211,7 @@ __global__ void __launch_bounds__(256) conv_chain_kernel(ChainArgs a)
     }
     __syncthreads();  // weights and vectors are in LDS; no barrier after this point
 
-    for (int g = g_begin; g < g_end; ++g) {
+    for (int g = g_begin; g < g1; ++g) {
         setup(g + 1, nxt);
         // residual of stage 1 for the first spans: requested now, used after the whole of stage 0
         v4i ev1[EVD][NT];
@@ -285,9 +276,8 @@ __global__ void __launch_bounds__(256) conv_chain_kernel(ChainArgs a)
             for (int nt = 0; nt < NT; ++nt) {
                 v4i ev = {0, 0, 0, 0};
                 if constexpr (chain_reads_residual<EPI0>()) ev = residual(s0, cur.e0[nt], sp);
-                v4i packed = epilogue_fast16<NT, EPI0>(s0, acc_sp, nt, sc.wq, sc.cal, sc.ecal, ev, s0.OFM - f0);
-                if (f0 >= s0.OFM) packed = v4i{0, 0, 0, 0};
-                else if (cur.o0[nt] >= 0) *reinterpret_cast<v4i*>((int8_t*)s0.out + cur.o0[nt] + sp * 4 * s0.out_pf) = packed;
+                const v4i packed = epilogue_fast16<NT, EPI0>(s0, acc_sp, nt, sc.wq, sc.cal, sc.ecal, ev, 16);
+                if (cur.o0[nt] >= 0) *reinterpret_cast<v4i*>((int8_t*)s0.out + cur.o0[nt] + sp * 4 * s0.out_pf) = packed;
                 bf0[sp][nt] = packed ^ xm1;
             }
         }
@@ -332,9 +322,8 @@ __global__ void __launch_bounds__(256) conv_chain_kernel(ChainArgs a)
             for (int nt = 0; nt < NT; ++nt) {
                 v4i ev = {0, 0, 0, 0};
                 if constexpr (chain_reads_residual<EPI1>()) ev = ev1[s % EVD][nt];
-                v4i packed = epilogue_fast16<NT, EPI1>(s1, acc1, nt, sc.wq, sc.cal, sc.ecal, ev, s1.OFM - f0);
-                if (f0 >= s1.OFM) packed = v4i{0, 0, 0, 0};
-                else if (cur.o1[nt] >= 0) *reinterpret_cast<v4i*>((int8_t*)s1.out + cur.o1[nt] + s * 4 * s1.out_pf) = packed;
+                const v4i packed = epilogue_fast16<NT, EPI1>(s1, acc1, nt, sc.wq, sc.cal, sc.ecal, ev, 16);
+                if (cur.o1[nt] >= 0) *reinterpret_cast<v4i*>((int8_t*)s1.out + cur.o1[nt] + s * 4 * s1.out_pf) = packed;
                 bf1[nt] = packed ^ xm2;
             }
             if constexpr (chain_reads_residual<EPI1>()) {
@@ -366,7 +355,6 @@ __global__ void __launch_bounds__(256) conv_chain_kernel(ChainArgs a)
 #pragma unroll
             for (int sp = 0; sp < SP2; ++sp) {
                 const int f0 = sp * 64 + kq * 16;
-                if (f0 >= s2.OFM) continue;
                 LaneScales sc;
                 chain_scales<EPI2>(s2, ldsV, SP2, f0, sc);
                 const v4i(&acc_sp)[4][NT] = *reinterpret_cast<const v4i(*)[4][NT]>(&acc2[sp * 4]);
@@ -375,7 +363,7 @@ __global__ void __launch_bounds__(256) conv_chain_kernel(ChainArgs a)
                     if (cur.o2[nt] < 0) continue;
                     v4i ev = {0, 0, 0, 0};
                     if constexpr (chain_reads_residual<EPI2>()) ev = residual(s2, cur.e2[nt], sp);
-                    const v4i packed = epilogue_fast16<NT, EPI2>(s2, acc_sp, nt, sc.wq, sc.cal, sc.ecal, ev, s2.OFM - f0);
+                    const v4i packed = epilogue_fast16<NT, EPI2>(s2, acc_sp, nt, sc.wq, sc.cal, sc.ecal, ev, 16);
                     *reinterpret_cast<v4i*>((int8_t*)s2.out + cur.o2[nt] + sp * 4 * s2.out_pf) = packed;
                 }
             }
