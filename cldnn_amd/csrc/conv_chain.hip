@@ -1,4 +1,5 @@
 // Host side of the convolution chain kernel: eligibility, LDS image of the weights, launch.
+#include <algorithm>
 #include <cstring>
 #include <mutex>
 #include <string>
@@ -78,40 +79,51 @@ std::string chain_plan(const ChainStageIn* st, int n, int cus, ChainPlan* out)
     }
     if (!conv_border_covers(p0)) return "stage 0: the input needs a zero border as wide as the padding";
     if (p0.dy != 1 || p0.dx != 1) return "stage 0: dilation";
-    // K-steps of every stage as the weights-stationary row packs them
-    pl.units = 0;
-    int vec = 0;
-    for (int k = 0; k < n; ++k) {
-        MfmaPlan mp{};
-        try {
-            mp = mfma_plan(*st[k].p, ROW_WSL_P64_FOR_CHAIN, cus);
-        } catch (const error& e) {
-            return "stage " + std::to_string(k) + ": " + e.what();
-        }
-        pl.unit0[k] = pl.units;
-        pl.kstride[k] = mp.ksteps;
-        pl.units += pl.sp[k] * mp.ksteps;
-        pl.vec0[k] = vec;
-        vec += 4 * pl.sp[k] * 64;
-        if (k == 0) pl.depth = mp.wsl_depth, pl.ksteps0 = mp.ksteps;
-        else if (mp.ksteps < pl.sp[k - 1]) return "stage " + std::to_string(k) + ": fewer K-steps than the previous stage has spans";
-    }
-    pl.lds_bytes = pl.units * 4096 + vec * 4;
-    if (pl.lds_bytes > CHAIN_MAX_LDS) return "the weights of the chain (" + std::to_string(pl.units * 4) + " KiB) do not fit into LDS";
     pl.nt = 2;
     pl.m_total = (int64_t)p0.B * p0.OH * p0.OW;
     pl.granules = (int)((pl.m_total + 16 * pl.nt - 1) / (16 * pl.nt));
-    if (!find_instance(pl)) return "no compiled instance for this chain shape";
-    const int per_cu = pl.lds_bytes * 2 <= CHAIN_MAX_LDS ? 2 : 1;
-    int grid = cus * per_cu / 8 * 8;
-    const int wanted = ((pl.granules + 3) / 4 + 7) / 8 * 8;  // at least one granule per wave
-    if (grid > wanted) grid = wanted;
-    if (grid < 8) grid = 8;
-    pl.grid = grid;
-    std::snprintf(pl.name, sizeof(pl.name), "conv_chain<%d stages,p%d,d%d,spans %d-%d-%d,epi %d-%d-%d>", n, 16 * pl.nt, pl.depth, pl.sp[0],
-                  pl.sp[1], pl.sp[2], pl.epi[0], pl.epi[1], n > 2 ? pl.epi[2] : -1);
-    *out = pl;
-    return std::string();
+    // K-steps of every stage as the weights-stationary row packs them
+    MfmaPlan mp[3]{};
+    for (int k = 0; k < n; ++k) {
+        ConvProblem q = *st[k].p;
+        try {
+            mp[k] = mfma_plan(q, ROW_WSL_P64_FOR_CHAIN, cus);
+        } catch (const error&) {
+            // K beyond what that row keeps in LDS: only the K-step count is wanted here
+            mp[k] = MfmaPlan{};
+            mp[k].ksteps = (q.FY * q.FX * ((q.IFM + 15) / 16) + 3) / 4;
+            mp[k].wsl_depth = 0;
+        }
+        if (k > 0 && mp[k].ksteps < pl.sp[k - 1]) return "stage " + std::to_string(k) + ": fewer K-steps than the previous stage has spans";
+    }
+    // everything in LDS, independent waves
+    {
+        pl.units = 0;
+        int vec = 0;
+        for (int k = 0; k < n; ++k) {
+            pl.unit0[k] = pl.units, pl.kstride[k] = mp[k].ksteps;
+            pl.units += pl.sp[k] * mp[k].ksteps;
+            pl.vec0[k] = vec;
+            vec += 4 * pl.sp[k] * 64;
+        }
+        pl.depth = mp[0].wsl_depth, pl.ksteps0 = mp[0].ksteps;
+        pl.lds_bytes = pl.units * 4096 + vec * 4;
+        if (mp[0].wsl_depth > 0 && pl.lds_bytes <= CHAIN_MAX_LDS && find_instance(pl)) {
+            const int per_cu = pl.lds_bytes * 2 <= CHAIN_MAX_LDS ? 2 : 1;
+            int grid = cus * per_cu / 8 * 8;
+            const int wanted = ((pl.granules + 3) / 4 + 7) / 8 * 8;  // at least one granule per wave
+            if (grid > wanted) grid = wanted;
+            if (grid < 8) grid = 8;
+            pl.grid = grid;
+            std::snprintf(pl.name, sizeof(pl.name), "conv_chain<%d stages,p%d,d%d,spans %d-%d-%d,epi %d-%d-%d>", n, 16 * pl.nt, pl.depth,
+                          pl.sp[0], pl.sp[1], pl.sp[2], pl.epi[0], pl.epi[1], n > 2 ? pl.epi[2] : -1);
+            *out = pl;
+            return std::string();
+        }
+    }
+    if (mp[0].wsl_depth <= 0 || pl.lds_bytes > CHAIN_MAX_LDS)
+        return "the weights of the chain (" + std::to_string(pl.units * 4) + " KiB) do not fit into LDS";
+    return "no compiled instance for this chain shape";
 }
 
 size_t chain_packed_bytes(const ChainPlan& pl) { return (size_t)pl.lds_bytes + 4096; }

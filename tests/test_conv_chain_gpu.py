@@ -67,7 +67,8 @@ def bottleneck_tail(eng, seed, B, H, W, mid, stages, fused, in_dt=np.uint8, keep
 @pytest.mark.parametrize("in_dt", [np.uint8, np.int8], ids=["u8", "s8"])
 @pytest.mark.parametrize("stages,fused", [(3, True), (2, True), (3, False), (2, False)], ids=["3fused", "2fused", "3plain", "2plain"])
 def test_bottleneck_tail_chain_matches_the_oracle(eng, stages, fused, in_dt):
-    B, H, W, mid = 3, 13, 11, 64  # 429 pixels: the last granule of 32 is partly filled, granules span rows and images
+    mid = 64
+    B, H, W = 3, 13, 11  # 429 pixels: the last granule of 32 is partly filled, granules span rows and images
     keep = [False] + [True] * (stages - 1)
     xin, spec, bufs, refs = bottleneck_tail(eng, 21, B, H, W, mid, stages, fused, in_dt)
     ch = hip.ConvChain(eng, spec, keep)
@@ -140,3 +141,8 @@ def test_chain_refusals(eng):
     # a chain of one
     with pytest.raises(hip.HipError):
         hip.ConvChain(eng, spec[:1])
+    # 128 mid features: the weights of the three stages (275 KB) do not fit into LDS
+    xin, spec, bufs, refs = bottleneck_tail(eng, 9, 1, 8, 8, 128, 3, True)
+    with pytest.raises(hip.HipError) as err:
+        hip.ConvChain(eng, spec, [False, True, True])
+    assert err.value.status == -6 and "LDS" in str(err.value)
