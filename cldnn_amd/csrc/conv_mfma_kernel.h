@@ -27,6 +27,8 @@
 // Weight rows are stored permuted inside each 64-feature span so that a lane's 16 accumulators
 // of one pixel are 16 CONSECUTIVE features: the int8 result is written with one 128-bit store.
 #pragma once
+#include <mutex>
+
 #include "epilogue.h"
 #include "kernels.h"
 
@@ -1135,14 +1137,14 @@ template <int BN, int NT, int KG>
 void launch_bdir_instance(hipStream_t s, const MfmaArgs& a, int grid, int lds, int epi)
 {
     const dim3 g(grid), b(256 * KG);
+    // more than 64 KiB of dynamic LDS has to be allowed per kernel, once (any host thread may be the first to launch)
 #define BDIR_LAUNCH(KIND)                                                                                       \
     {                                                                                                           \
-        static bool allowed = false;                                                                            \
-        if (!allowed && lds > 48 * 1024) {                                                                      \
+        static std::once_flag allowed;                                                                          \
+        std::call_once(allowed, [] {                                                                            \
             CHIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(&conv_bdir_kernel<BN, NT, KG, KIND>),  \
                                            hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));            \
-            allowed = true;                                                                                     \
-        }                                                                                                       \
+        });                                                                                                     \
         hipLaunchKernelGGL((conv_bdir_kernel<BN, NT, KG, KIND>), g, b, lds, s, a);                              \
     }
     switch (epi) {
@@ -1159,15 +1161,14 @@ template <int NT, int D>
 void launch_wsl_instance(hipStream_t s, const MfmaArgs& a, int grid, int lds, int epi)
 {
     const dim3 g(grid), b(256);
-    // more than 64 KiB of dynamic LDS has to be allowed per kernel, once
+    // more than 64 KiB of dynamic LDS has to be allowed per kernel, once (any host thread may be the first to launch)
 #define WSL_LAUNCH(KIND)                                                                                       \
     {                                                                                                          \
-        static bool allowed = false;                                                                           \
-        if (!allowed) {                                                                                        \
+        static std::once_flag allowed;                                                                         \
+        std::call_once(allowed, [] {                                                                           \
             CHIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(&conv_wsl_kernel<NT, D, KIND>),       \
                                            hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));           \
-            allowed = true;                                                                                    \
-        }                                                                                                      \
+        });                                                                                                    \
         hipLaunchKernelGGL((conv_wsl_kernel<NT, D, KIND>), g, b, lds, s, a);                                   \
     }
     switch (epi) {

@@ -52,7 +52,15 @@ __global__ void __launch_bounds__(256) pooling_kernel(PoolArgs a, const void* __
         b = (int)(r / a.F);
     }
     const int oy0 = y * a.sy - a.py, ox0 = x * a.sx - a.px;
-    if (oy0 + a.ky < 0 || oy0 >= a.IH || ox0 + a.kx < 0 || ox0 >= a.IW) return;
+    if (oy0 + a.ky < 0 || oy0 >= a.IH || ox0 + a.kx < 0 || ox0 >= a.IW) {
+        // A window that lies wholly outside the input: the reference's kernel leaves such an output untouched, i.e. at
+        // the zero its buffers are created with (pooling_gpu_int8_ref.cl:62-68).  A buffer handed over by the memory
+        // pool is not zero, so the zero is written.
+        EpiOut z;
+        z.f = 0.0f, z.i = 0;
+        store_out(out, a.dt, a.out.at(b, f, y, x), z);
+        return;
+    }
     const bool is_max = a.mode == CLDNN_HIP_POOL_MAX;
     int valid = 0;
     EpiOut o;
@@ -117,7 +125,13 @@ __global__ void __launch_bounds__(256) pooling_fsv16_kernel(PoolFastArgs p, cons
     const uint32_t fs = p.div_b.div(r2);
     const int b = (int)(r2 - fs * (uint32_t)a.B);
     const int oy0 = y * a.sy - a.py, ox0 = x * a.sx - a.px;
-    if (oy0 + a.ky < 0 || oy0 >= a.IH || ox0 + a.kx < 0 || ox0 >= a.IW) return;
+    if (oy0 + a.ky < 0 || oy0 >= a.IH || ox0 + a.kx < 0 || ox0 >= a.IW) {
+        // a window wholly outside the input: zero, as a freshly created buffer of the reference holds (see pooling_kernel);
+        // the lanes of a SPLIT group share the window and leave together
+        if (part == 0)
+            *reinterpret_cast<uint4*>(out + (p.out_off + b * p.out_pb + (int)fs * p.out_pf + y * p.out_py + x * 16)) = make_uint4(0, 0, 0, 0);
+        return;
+    }
     int acc[16];
 #pragma unroll
     for (int c = 0; c < 16; ++c) acc[c] = MAX ? -128 : 0;

@@ -375,6 +375,50 @@ cldnn_hip_status cldnn_hip_event_record(cldnn_hip_engine e, cldnn_hip_event* out
     });
 }
 
+cldnn_hip_status cldnn_hip_event_create_deferred(cldnn_hip_engine e, cldnn_hip_event* out)
+{
+    return guarded([&] {
+        CHIP_REQUIRE(e && out, CLDNN_HIP_INVALID_ARG, "null argument");
+        cldnn_hip_event ev = new_event(e, false);
+        ev->deferred = true;
+        ev->deferred_pending = true;
+        *out = ev;
+    });
+}
+
+cldnn_hip_status cldnn_hip_event_record_deferred(cldnn_hip_event ev)
+{
+    return guarded([&] {
+        CHIP_REQUIRE(ev && ev->deferred, CLDNN_HIP_INVALID_ARG, "not a deferred event");
+        hipError_t r = hipSuccess;
+        {
+            std::lock_guard<std::mutex> g(ev->deferred_mutex);
+            CHIP_REQUIRE(ev->deferred_pending, CLDNN_HIP_ERROR, "deferred event recorded twice");
+            ev->engine->make_current();
+            ev->stop = ev->engine->take_event();
+            r = hipEventRecord(ev->stop, ev->engine->stream);
+            ev->deferred_pending = false;  // also after a failed record: nobody may wait for ever
+        }
+        ev->deferred_cv.notify_all();
+        CHIP_CHECK(r);
+    });
+}
+
+// a deferred event: block until the work it stands for has been submitted
+static void await_submission(cldnn_hip_event ev)
+{
+    if (!ev->deferred) return;
+    std::unique_lock<std::mutex> g(ev->deferred_mutex);
+    ev->deferred_cv.wait(g, [&] { return !ev->deferred_pending; });
+}
+
+static bool submission_pending(cldnn_hip_event ev)
+{
+    if (!ev->deferred) return false;
+    std::lock_guard<std::mutex> g(ev->deferred_mutex);
+    return ev->deferred_pending;
+}
+
 cldnn_hip_status cldnn_hip_event_retain(cldnn_hip_event ev)
 {
     return guarded([&] {
@@ -418,8 +462,9 @@ cldnn_hip_status cldnn_hip_event_wait(cldnn_hip_event ev)
         CHIP_REQUIRE(ev, CLDNN_HIP_INVALID_ARG, "null event");
         if (ev->user) {
             while (!ev->user_set.load()) std::this_thread::sleep_for(std::chrono::microseconds(50));
-        } else if (ev->stop) {
-            CHIP_CHECK(hipEventSynchronize(ev->stop));
+        } else {
+            await_submission(ev);
+            if (ev->stop) CHIP_CHECK(hipEventSynchronize(ev->stop));
         }
         fire_handlers(ev);
     });
@@ -429,7 +474,7 @@ int32_t cldnn_hip_event_is_set(cldnn_hip_event ev)
 {
     if (!ev) return 0;
     if (ev->user) return ev->user_set.load() ? 1 : 0;
-    if (!ev->stop) return 0;
+    if (submission_pending(ev) || !ev->stop) return 0;
     hipError_t r = hipEventQuery(ev->stop);
     if (r == hipSuccess) return 1;
     (void)hipGetLastError();
@@ -466,6 +511,7 @@ cldnn_hip_status cldnn_hip_event_add_handler(cldnn_hip_event ev, cldnn_hip_event
             cldnn_hip_event_retain(ev);
             std::thread([ev] {
                 (void)hipSetDevice(ev->engine->device);
+                await_submission(ev);
                 if (ev->stop) (void)hipEventSynchronize(ev->stop);
                 fire_handlers(ev);
                 cldnn_hip_event_release(ev);
@@ -480,6 +526,7 @@ cldnn_hip_status cldnn_hip_event_elapsed_ns(cldnn_hip_event ev, uint64_t* ns)
         CHIP_REQUIRE(ev && ns, CLDNN_HIP_INVALID_ARG, "null argument");
         *ns = 0;
         if (!ev->start || !ev->stop) return;
+        await_submission(ev);
         CHIP_CHECK(hipEventSynchronize(ev->stop));
         float ms = 0.f;
         CHIP_CHECK(hipEventElapsedTime(&ms, ev->start, ev->stop));
@@ -497,8 +544,9 @@ cldnn_hip_status cldnn_hip_engine_wait_events(cldnn_hip_engine e, const cldnn_hi
             if (ev->user) {
                 // a stream cannot wait for a host flag: hold back submission until it is set
                 while (!ev->user_set.load()) std::this_thread::sleep_for(std::chrono::microseconds(50));
-            } else if (ev->stop && ev->engine != e) {
-                CHIP_CHECK(hipStreamWaitEvent(e->stream, ev->stop, 0));
+            } else {
+                await_submission(ev);
+                if (ev->stop && ev->engine != e) CHIP_CHECK(hipStreamWaitEvent(e->stream, ev->stop, 0));
             }
             // same engine: the single in-order stream already orders the work
         }

@@ -1,6 +1,7 @@
 // Engine, buffer and event objects behind the C handles of cldnn_hip.h.
 #pragma once
 #include <atomic>
+#include <condition_variable>
 #include <mutex>
 #include <utility>
 #include <vector>
@@ -39,6 +40,12 @@ struct cldnn_hip_event_s {
     std::atomic<bool> user_set{false};
     hipEvent_t start = nullptr;  // only with profiling
     hipEvent_t stop = nullptr;
+    // a deferred event stands for work that has not been submitted yet: it is recorded later, and whoever waits for
+    // it first waits for that
+    bool deferred = false;
+    std::mutex deferred_mutex;
+    std::condition_variable deferred_cv;
+    bool deferred_pending = false;
     std::mutex handler_mutex;
     bool handlers_fired = false;
     std::vector<std::pair<cldnn_hip_event_handler, void*>> handlers;

@@ -135,6 +135,8 @@ SIGNATURES = {
     "cldnn_hip_event_record": (C.c_int32, [C.c_void_p, C.POINTER(C.c_void_p)]),
     "cldnn_hip_event_record_begin": (C.c_int32, [C.c_void_p, C.POINTER(C.c_void_p)]),
     "cldnn_hip_event_record_end": (C.c_int32, [C.c_void_p]),
+    "cldnn_hip_event_create_deferred": (C.c_int32, [C.c_void_p, C.POINTER(C.c_void_p)]),
+    "cldnn_hip_event_record_deferred": (C.c_int32, [C.c_void_p]),
     "cldnn_hip_event_retain": (C.c_int32, [C.c_void_p]),
     "cldnn_hip_event_release": (C.c_int32, [C.c_void_p]),
     "cldnn_hip_event_wait": (C.c_int32, [C.c_void_p]),

@@ -109,20 +109,35 @@ static ref<cldnn_memory_impl> on_engine(cldnn_engine_impl* e, cldnn_memory_impl*
     return c;
 }
 
-static void execute(cldnn_network_impl* net, cldnn_event* deps, size_t ndeps)
+// A run that was postponed must have been submitted before the network is touched again.  Blocks until the user
+// events it waits for are set (what the reference's set_input_data / execute do by waiting for the previous run).
+static void await_pending_run(cldnn_network_impl* net)
+{
+    std::shared_ptr<deferred_run> run = net->pending;
+    if (!run) return;
+    std::string error;
+    {
+        std::unique_lock<std::mutex> g(run->m);
+        run->cv.wait(g, [&] { return run->submitted; });
+        error = run->error;
+    }
+    net->pending.reset();
+    HOST_REQUIRE(error.empty(), CLDNN_ERROR, "the postponed run of the network failed: " + error);
+}
+
+// Enqueue one run.  deferred_marker: the run was announced earlier (its outputs already carry that event) and is
+// submitted now that its user events are set.
+static void submit(cldnn_network_impl* net, cldnn_event* deps, size_t ndeps, cldnn_event_impl* deferred_marker)
 {
     cldnn_program_impl* prog = net->program.get();
     cldnn_engine_impl* eng = prog->engine.get();
     if (ndeps) {
         std::vector<cldnn_hip_event> hs;
-        for (size_t i = 0; i < ndeps; ++i) {
-            HOST_REQUIRE(deps && deps[i], CLDNN_INVALID_ARG, "null event in the dependency list");
-            hs.push_back(deps[i]->h);
-        }
+        for (size_t i = 0; i < ndeps; ++i) hs.push_back(deps[i]->h);
         hip_check(cldnn_hip_engine_wait_events(eng->h, hs.data(), hs.size()));
     }
     net->executed.clear();
-    net->events.clear();
+    if (!deferred_marker) net->events.clear();
     for (cldnn_hip_event ev : net->stream_events) cldnn_hip_event_release(ev);  // the previous run's; it has been waited for
     net->stream_events.clear();
     std::map<node*, cldnn_hip_event> joins;  // completion of the primitives on the second stream
@@ -225,25 +240,105 @@ static void execute(cldnn_network_impl* net, cldnn_event* deps, size_t ndeps)
             ref<cldnn_event_impl> ev(new cldnn_event_impl(), false);
             ev->engine = ref<cldnn_engine_impl>(eng, true);
             ev->h = pev;
-            net->events[n] = ev;
+            // an output of a postponed run keeps the event its users were given when the run was announced
+            if (!(deferred_marker && n->is_output)) net->events[n] = ev;
         }
         net->executed.push_back(p.id);
     }
-    // one marker for every output that has no event of its own (reference ocl_toolkit.cpp:170-178,197-230)
-    ref<cldnn_event_impl> marker;
-    for (auto& u : prog->nodes) {
-        node* n = u.get();
-        if (!n->is_output || net->events.count(n)) continue;
-        if (!marker) {
-            marker = ref<cldnn_event_impl>(new cldnn_event_impl(), false);
-            marker->engine = ref<cldnn_engine_impl>(eng, true);
-            hip_check(cldnn_hip_event_record(eng->h, &marker->h));
+    if (deferred_marker) {
+        hip_check(cldnn_hip_event_record_deferred(deferred_marker->h));
+    } else {
+        // one marker for every output that has no event of its own (reference ocl_toolkit.cpp:170-178,197-230)
+        ref<cldnn_event_impl> marker;
+        for (auto& u : prog->nodes) {
+            node* n = u.get();
+            if (!n->is_output || net->events.count(n)) continue;
+            if (!marker) {
+                marker = ref<cldnn_event_impl>(new cldnn_event_impl(), false);
+                marker->engine = ref<cldnn_engine_impl>(eng, true);
+                hip_check(cldnn_hip_event_record(eng->h, &marker->h));
+            }
+            net->events[n] = marker;
         }
-        net->events[n] = marker;
     }
     if (eng->side) hip_check(cldnn_hip_engine_flush(eng->side));
     hip_check(cldnn_hip_engine_flush(eng->h));
     net->has_run = true;
+}
+
+// called by cldnn_hip_event_set (or at once, if the event got set in the meantime) for every user event a postponed
+// run waits for; the last one submits the run
+static void gate_opened(void* param)
+{
+    std::shared_ptr<deferred_run> run = *static_cast<std::shared_ptr<deferred_run>*>(param);
+    delete static_cast<std::shared_ptr<deferred_run>*>(param);
+    bool last = false;
+    {
+        std::lock_guard<std::mutex> g(run->m);
+        last = --run->gates_left == 0;
+    }
+    if (!last) return;
+    std::string error;
+    try {
+        submit(run->net, run->deps.data(), run->deps.size(), run->marker.get());
+    } catch (const std::exception& e) {
+        error = e.what();
+        (void)cldnn_hip_event_record_deferred(run->marker->h);  // nobody may wait for ever
+    }
+    for (cldnn_event d : run->deps) d->release();
+    run->deps.clear();
+    cldnn_network_impl* net = run->net;
+    {
+        std::lock_guard<std::mutex> g(run->m);
+        run->error = error;
+        run->submitted = true;
+    }
+    run->cv.notify_all();
+    net->release();
+}
+
+// reference network_impl::execute (src/network.cpp:280-353) enqueues behind the dependency events and returns; an
+// OpenCL user event among them may be set later, also by the calling thread.  A HIP stream cannot wait for a host
+// flag, so a run behind user events that are not set yet is postponed: this call announces it (every output gets one
+// deferred event), returns, and the run is submitted by the thread that sets the last of those events.
+static void execute(cldnn_network_impl* net, cldnn_event* deps, size_t ndeps)
+{
+    for (size_t i = 0; i < ndeps; ++i) HOST_REQUIRE(deps && deps[i], CLDNN_INVALID_ARG, "null event in the dependency list");
+    await_pending_run(net);
+    std::vector<cldnn_event> gates;
+    for (size_t i = 0; i < ndeps; ++i)
+        if (cldnn_hip_event_is_user(deps[i]->h) && !cldnn_hip_event_is_set(deps[i]->h)) gates.push_back(deps[i]);
+    if (gates.empty()) {
+        submit(net, deps, ndeps, nullptr);
+        return;
+    }
+    cldnn_program_impl* prog = net->program.get();
+    cldnn_engine_impl* eng = prog->engine.get();
+    for (auto& u : prog->nodes)  // what submit() would refuse is refused now, while the caller can still react
+        if (u->p->type == prim_type::input_layout)
+            HOST_REQUIRE(net->input_set[u->p->id], CLDNN_ERROR, "network input " + u->p->id + " has not been set");
+    auto run = std::make_shared<deferred_run>();
+    run->gates_left = (int)gates.size();
+    run->net = net;
+    net->retain();
+    for (size_t i = 0; i < ndeps; ++i) {
+        deps[i]->retain();
+        run->deps.push_back(deps[i]);
+    }
+    run->marker = ref<cldnn_event_impl>(new cldnn_event_impl(), false);
+    run->marker->engine = ref<cldnn_engine_impl>(eng, true);
+    hip_check(cldnn_hip_event_create_deferred(eng->h, &run->marker->h));
+    net->events.clear();
+    net->executed.clear();
+    for (auto& u : prog->nodes) {
+        node* n = u.get();
+        if (n->is_output) net->events[n] = run->marker;
+        if (!n->constant && n->p->type != prim_type::input_layout) net->executed.push_back(n->p->id);
+    }
+    net->has_run = true;
+    net->pending = run;
+    for (cldnn_event g : gates)
+        hip_check(cldnn_hip_event_add_handler(g->h, gate_opened, new std::shared_ptr<deferred_run>(run)));
 }
 
 }  // namespace host
@@ -777,6 +872,7 @@ void cldnn_set_network_input(cldnn_network network, cldnn_primitive_id id, cldnn
         HOST_REQUIRE(it != prog->by_id.end() && it->second->p->type == prim_type::input_layout, CLDNN_INVALID_ARG,
                      std::string("primitive ") + id + " is not an input");
         // the previous run must be over before its input is replaced (reference network.cpp:112-113)
+        await_pending_run(network);
         hip_check(cldnn_hip_engine_finish(prog->engine->h));
         HOST_REQUIRE(same_layout(mem->layout, it->second->out), CLDNN_INVALID_ARG, "set_network_input: memory layout differs from the input's layout");
         network->mem[it->second] = on_engine(prog->engine.get(), mem);

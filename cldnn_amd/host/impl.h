@@ -3,8 +3,10 @@
 // program,network}_impl.h, refcounted_obj.h) for the one path this library serves.
 #pragma once
 #include <atomic>
+#include <condition_variable>
 #include <map>
 #include <memory>
+#include <mutex>
 #include <stdexcept>
 #include <string>
 #include <vector>
@@ -191,8 +193,22 @@ struct cldnn_program_impl : host::refcounted {
     ~cldnn_program_impl() override;
 };
 
+// A run whose submission waits for user events that were not set when cldnn_execute_network was called.  The last of
+// those events to be set submits the run from cldnn_set_event; until then the outputs carry one deferred event.
+struct deferred_run {
+    std::mutex m;
+    std::condition_variable cv;
+    int gates_left = 0;
+    bool submitted = false;
+    std::string error;                     // a failure of the late submission, reported by the next call on the network
+    std::vector<cldnn_event> deps;         // retained dependency list
+    host::ref<cldnn_event_impl> marker;    // the deferred event the outputs carry
+    cldnn_network_impl* net = nullptr;     // retained
+};
+
 struct cldnn_network_impl : host::refcounted {
     host::ref<cldnn_program_impl> program;
+    std::shared_ptr<deferred_run> pending;  // a run that has not been submitted yet
     std::map<host::node*, host::ref<cldnn_memory_impl>> mem;
     std::map<host::node*, host::ref<cldnn_event_impl>> events;
     std::map<std::string, bool> input_set;

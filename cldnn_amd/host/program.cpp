@@ -507,6 +507,8 @@ static void eltwise_remove_stride(cldnn_program_impl* prog)
     }
 }
 
+static bool wants_blocked(node* n);
+
 // convolution (1x1, stride 1) + eltwise sum with relu -> fused_conv_eltwise (reference :181-337).
 // A sum WITHOUT activation stays a primitive of its own in the reference (a residual sum of MobileNet-v2).  Its
 // arithmetic differs from the fused primitive's in one point: it adds to the convolution's int8 output, that is to the
@@ -530,9 +532,14 @@ static void fuse_conv_eltwise(cldnn_program_impl* prog)
             for (node* t : {c, e, e->deps[0], e->deps[1]}) ok = ok && t->out.data_type == cldnn_i8;
             if (!ok) continue;
         }
+        // Which convolutions the reference fuses (prepare_primitive_fusing.cpp:197-205): int8 in fs_bs_yx_bsv4_fsv32,
+        // int8 / uint8 in b_fs_yx_fsv4, f32 in bfyx.  The blocked layout of this library stands where the reference has
+        // fs_bs_yx_bsv4_fsv32, so the first case reads: an int8 convolution that the layout rule is going to run in
+        // fs_b_yx_fsv16.  Any other int8 convolution in a plain layout (grouped ones, unquantized ones) stays unfused,
+        // as in the reference: fused, the sum would see the unsaturated accumulator instead of the int8 tensor.
         const cldnn_layout& cl = c->out;
         const bool ok_type = (is_int8(cl.data_type) && (cl.format == cldnn_format_b_fs_yx_fsv4 || cl.format == cldnn_format_fs_b_yx_fsv16
-                                                        || cl.format == cldnn_format_bfyx || cl.format == cldnn_format_byxf))
+                                                        || wants_blocked(c)))
                              || (cl.format == cldnn_format_bfyx && cl.data_type == cldnn_f32);
         if (!ok_type) continue;
         node* w = dep_named(c, c->p->weights.at(0));

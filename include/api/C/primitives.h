@@ -100,7 +100,7 @@ cldnn_tensor stride;
 cldnn_tensor dilation;
 uint32_t with_activation;
 float activation_negative_slope;
-uint32_t split;              /* must be 1 (use groups) */
+uint32_t split;              /* number of weight / bias / factor primitives; executed as groups = split in one launch */
 uint32_t with_output_size;
 cldnn_tensor output_size;
 cldnn_primitive_id_arr weights;
@@ -110,7 +110,7 @@ cldnn_primitive_id_arr output_calibration_factors;
 float input_quantization_factor;
 float output_quantization_factor;
 uint32_t groups;
-cldnn_tensor padding_above;  /* symmetric use only */
+cldnn_tensor padding_above;  /* zero padding in front of / behind the data, each side on its own (may differ) */
 cldnn_tensor padding_below;
 CLDNN_END_PRIMITIVE_DESC(convolution)
 CLDNN_DECLARE_PRIMITIVE_TYPE_ID(convolution);

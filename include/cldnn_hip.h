@@ -102,6 +102,12 @@ cldnn_hip_status cldnn_hip_event_record(cldnn_hip_engine e, cldnn_hip_event* out
  * its execution time (reference src/gpu/ocl_toolkit.cpp:170-178 returns such an event per kernel) */
 cldnn_hip_status cldnn_hip_event_record_begin(cldnn_hip_engine e, cldnn_hip_event* out);
 cldnn_hip_status cldnn_hip_event_record_end(cldnn_hip_event ev);
+/* An event for work that will be submitted LATER (reference: an OpenCL command enqueued behind a user event exists, and
+ * can be waited for, before that user event is set -- src/gpu/ocl_toolkit.cpp:153-195 with deps).  create_deferred makes
+ * the event; record_deferred, called once when the work has been enqueued on the event's engine, records it.  Until then
+ * is_set is 0 and wait / add_handler / elapsed_ns block (or call back) only after the recording AND the work are done. */
+cldnn_hip_status cldnn_hip_event_create_deferred(cldnn_hip_engine e, cldnn_hip_event* out);
+cldnn_hip_status cldnn_hip_event_record_deferred(cldnn_hip_event ev);
 cldnn_hip_status cldnn_hip_event_retain(cldnn_hip_event ev);
 cldnn_hip_status cldnn_hip_event_release(cldnn_hip_event ev);
 cldnn_hip_status cldnn_hip_event_wait(cldnn_hip_event ev);
@@ -111,7 +117,11 @@ cldnn_hip_status cldnn_hip_event_set(cldnn_hip_event ev);
 cldnn_hip_status cldnn_hip_event_add_handler(cldnn_hip_event ev, cldnn_hip_event_handler h, void* param);
 /* "executing" interval in ns (reference src/gpu/ocl_base_event.cpp:68-96); 0 when profiling is off */
 cldnn_hip_status cldnn_hip_event_elapsed_ns(cldnn_hip_event ev, uint64_t* ns);
-/* make the engine stream wait for events before later work (gpu_toolkit::sync_events, reference src/gpu/ocl_toolkit.cpp:313-346) */
+/* make the engine stream wait for events before later work (gpu_toolkit::sync_events, reference src/gpu/ocl_toolkit.cpp:313-346).
+ * A stream cannot wait for a host flag: for a user event that is not set yet the CALLING THREAD is held until it is.  A
+ * caller that must not block looks at cldnn_hip_event_is_user / cldnn_hip_event_is_set first and postpones its
+ * submission (libclDNN does: cldnn_execute_network behind an unset user event returns at once and submits from
+ * cldnn_hip_event_set). */
 cldnn_hip_status cldnn_hip_engine_wait_events(cldnn_hip_engine e, const cldnn_hip_event* evs, size_t n);
 
 /* ------------------------------------------------------------------ tensors */

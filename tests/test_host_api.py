@@ -295,17 +295,19 @@ def test_unsupported_activation_is_not_folded():
     assert "relu" in opt and opt["conv"]["fused_activation"] == cl.activation_func.none
 
 
-def residual_block(fy=1, stride=1, with_activation=True, eltw_strides=None, in_fmt=F.bfyx, sum_calib="c", dt=None):
+def residual_block(fy=1, stride=1, with_activation=True, eltw_strides=None, in_fmt=F.bfyx, sum_calib="c", dt=None, groups=1,
+                   quantized=True):
     """conv(3x3) -> [conv 1x1 | 3x3] + shortcut -> eltwise sum (+relu): the tail of a ResNet block."""
     B, Cn, H, W = 2, 16, 8, 8
     w1 = attach(np.ones((Cn, Cn, 3, 3), np.int8))
-    w2 = attach(np.ones((Cn, Cn, fy, fy), np.int8))
+    w2 = attach(np.ones((Cn, Cn // groups, fy, fy), np.int8))
+    q2 = dict(w_quantization_factor=["q"], output_calibration_factors=["c"]) if quantized else {}
     t = cl.topology(cl.input_layout("in", cl.layout(DT.i8 if dt is None else dt, in_fmt, cl.tensor(B, Cn, W, H))),
                     cl.data("w1", w1), cl.data("w2", w2), cl.data("q", vec(Cn)), cl.data("c", vec(Cn)),
                     cl.convolution("conv1", "in", ["w1"], w_quantization_factor=["q"], output_calibration_factors=["c"],
                                    input_offset=cl.tensor(0, 0, -1, -1, 0), with_activation=True),
-                    cl.convolution("conv2", "conv1", ["w2"], w_quantization_factor=["q"], output_calibration_factors=["c"],
-                                   input_offset=cl.tensor(0, 0, -(fy // 2), -(fy // 2), 0), stride=cl.tensor(1, 1, stride, stride)),
+                    cl.convolution("conv2", "conv1", ["w2"], input_offset=cl.tensor(0, 0, -(fy // 2), -(fy // 2), 0),
+                                   stride=cl.tensor(1, 1, stride, stride), groups=groups, **q2),
                     cl.eltwise("sum", "in", "conv2", cl.eltwise_mode.sum, with_activation, 0.0, output_calibration_factors=sum_calib,
                                stride=eltw_strides),
                     cl.activation("out", "sum", cl.activation_func.none))
@@ -331,6 +333,17 @@ def test_conv_eltwise_fusing():
 def test_conv_eltwise_not_fused(kw):
     ids = [n["id"] for n in cl.plan(residual_block(**kw), cl.build_options(optimize_data=True))]
     assert "conv2" in ids and "sum" in ids
+
+
+@pytest.mark.parametrize("kw", [dict(groups=2), dict(quantized=False)], ids=["grouped", "unquantized"])
+def test_int8_convolutions_that_stay_in_a_plain_layout_are_not_fused(kw):
+    """the reference fuses int8 convolutions only in its blocked int8 formats (prepare_primitive_fusing.cpp:197-205); here
+    that means the ones the layout rule runs in fs_b_yx_fsv16.  A grouped or unquantized int8 1x1 convolution stays in
+    bfyx on the reference kernel, and its relu sum stays a primitive of its own (the sum then adds to the saturated
+    int8 tensor, not to the accumulator)."""
+    opt = by_id(cl.plan(residual_block(**kw), cl.build_options(optimize_data=True)))
+    assert "conv2" in opt and "sum" in opt and "conv2_fused_sum" not in opt
+    assert opt["conv2"]["type"] == "convolution" and opt["sum"]["type"] == "eltwise"
 
 
 def test_sum_without_activation_is_fused_with_the_saturation_kept():

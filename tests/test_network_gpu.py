@@ -367,6 +367,34 @@ def test_fused_and_unfused_graphs_agree(eng):
     np.testing.assert_array_equal(outs[0], outs[1])
 
 
+@pytest.mark.parametrize("optimize", OPT, ids=["plain", "optimize_data"])
+def test_grouped_convolution_keeps_its_sum_unfused_on_saturating_data(eng, optimize):
+    """a grouped int8 1x1 convolution stays on the plain-layout kernel and, as in the reference
+    (prepare_primitive_fusing.cpp:197-205), its relu sum stays a primitive of its own: the sum adds to the SATURATED int8
+    tensor.  The factors are chosen so that a good share of the convolution's results leave the int8 range, where the
+    fused arithmetic (sum on the unsaturated value) would give other numbers."""
+    r = np.random.default_rng(23)
+    B, Cn, H, W, G = 2, 32, 6, 7, 2
+    x = r.integers(-128, 128, (B, Cn, H, W)).astype(np.int8)
+    w = r.integers(-127, 128, (Cn, Cn // G, 1, 1)).astype(np.int8)
+    cal = r.uniform(4e-3, 1.2e-2, Cn).astype(np.float32)  # accumulators of a few 10^4: results around +-200
+    ecal = r.uniform(0.4, 0.9, Cn).astype(np.float32)
+    t = cl.topology(cl.input_layout("input", cl.layout(DT.i8, F.bfyx, cl.tensor(B, Cn, W, H))), cl.data("w", cl.make_memory(eng, w)),
+                    cl.data("q", vec_mem(eng, np.ones(Cn, np.float32))), cl.data("c", vec_mem(eng, cal)), cl.data("e", vec_mem(eng, ecal)),
+                    cl.convolution("conv", "input", ["w"], None, ["q"], ["c"], groups=G),
+                    cl.eltwise("sum", "input", "conv", cl.eltwise_mode.sum, True, 0.0, output_calibration_factors="e"),
+                    cl.reorder("out", "sum", F.bfyx))
+    net, outs = run(eng, t, {"input": cl.make_memory(eng, x)}, optimize)
+    conv = rc.conv(x, w, None, wqf=np.ones(Cn, np.float32), calib=cal, groups=G, out_dt="s8")
+    assert np.count_nonzero(np.abs(conv) == 127) + np.count_nonzero(conv == -128) > conv.size // 10  # it does saturate
+    expected = rc.eltwise_sum(x, conv, calib=ecal, relu=True)
+    fused_form = rc.conv(x, w, None, wqf=np.ones(Cn, np.float32), calib=cal, groups=G, out_dt="s8", eltw=x, eltw_act="relu", eltw_calib=ecal)
+    assert np.count_nonzero(fused_form != expected) > 0  # the two arithmetics do differ on this data
+    np.testing.assert_array_equal(outs["out"].get_memory().read(), expected)
+    executed = net.get_executed_primitive_ids()
+    assert "conv" in executed and "sum" in executed
+
+
 def test_closer_writes_over_its_shortcut_without_a_memory_pool():
     """prepare_conv_eltw_read_write_opt (reference prepare_primitive_fusing.cpp:468-534): the fused closer of a block whose
     shortcut is an intermediate tensor of the same layout, read by nothing later, takes the shortcut's buffer as its
@@ -568,6 +596,51 @@ def test_events_and_profiling():
     cb = cl.EVENT_HANDLER(lambda p: fired.append(1))
     cl._call("cldnn_add_event_handler", ev.h, cb, None)
     assert fired == [1]  # the event is complete: the handler runs at once
+
+
+@pytest.mark.parametrize("profiling", [False, True], ids=["plain", "profiling"])
+def test_execute_behind_a_user_event_that_is_set_afterwards(profiling):
+    """reference network::execute enqueues behind its dependency events and returns; an OpenCL user event among them
+    may be set later by the same thread.  Here the run is postponed: execute returns at once, the output's event is
+    not complete, and the run is submitted when the last gate is set."""
+    eng = cl.engine(enable_profiling=profiling)
+    topo, x, oracle = bottleneck(eng, 4)
+    net = cl.network(eng, topo, cl.build_options(optimize_data=True))
+    net.set_input_data("input", cl.make_memory(eng, x))
+    gate_a, gate_b = cl.event.create_user_event(eng), cl.event.create_user_event(eng)
+    fired = []
+    outs = net.execute([gate_a, gate_b])        # returns although neither gate is set
+    ev = outs["out"].get_event()
+    cb = cl.EVENT_HANDLER(lambda p: fired.append(1))
+    cl._call("cldnn_add_event_handler", ev.h, cb, None)
+    assert fired == []                           # nothing has run
+    assert "expand_fused_sum" in net.get_executed_primitive_ids()
+    gate_a.set()
+    assert fired == []                           # one gate is still closed
+    gate_b.set()                                 # submits the run from this thread
+    ev.wait()
+    np.testing.assert_array_equal(outs["out"].get_memory().read(), oracle())
+    import time
+    for _ in range(200):                         # the handler of a stream event is called from a helper thread
+        if fired:
+            break
+        time.sleep(0.01)
+    assert fired == [1]
+    # the network runs again the ordinary way, and behind a gate that is already open
+    x2 = np.roll(x, 1, axis=0)
+    net.set_input_data("input", cl.make_memory(eng, x2))
+    outs = net.execute([gate_a])
+    outs["out"].get_event().wait()
+    assert not np.array_equal(x, x2)
+    # a postponed run must be submitted before the input can be replaced: set_input_data waits for the gate, so the
+    # gate is opened from another thread
+    import threading
+    gate_c = cl.event.create_user_event(eng)
+    net.set_input_data("input", cl.make_memory(eng, x))
+    outs = net.execute([gate_c])
+    threading.Timer(0.05, gate_c.set).start()
+    net.set_input_data("input", cl.make_memory(eng, x2))   # blocks until the timer opens the gate and the run is over
+    np.testing.assert_array_equal(outs["out"].get_memory().read(), oracle())
 
 
 def test_unsupported_requests_fail_loudly(eng):
