@@ -1,0 +1,99 @@
+"""Every distinct layer of the five benchmark configurations at its REAL batch size against the oracle.
+
+The row of the tile-config table depends on the pixel count, so the kernels production uses at batch 32 / 16 / 1 are
+not the ones the small-shape tests reach.  Here each distinct layer signature is built exactly as bench.py builds it
+(same seeded data, same descriptors, same chain grouping), run once at full size, and the first image(s) of its
+output are compared with the oracle bit for bit (a convolution is independent per image).  The kernels the committed
+profiles name as dominant are asserted by name."""
+import numpy as np
+import pytest
+
+import bench
+from cldnn_amd import hip, workloads
+
+pytestmark = pytest.mark.gpu
+
+CONFIGS = {  # workload -> (layers, batch, residual fused, images compared)
+    "resnet50_b32_fused": (workloads.resnet50(), 32, True, 2),
+    "resnet50_b1": (workloads.resnet50(), 1, False, 1),
+    "vgg16_b16": (workloads.vgg16(), 16, False, 1),
+    "mobilenet_v2_b32": (workloads.mobilenet_v2(), 32, False, 2),
+    "c1": ([workloads._layer("c1", 64, 64, 3, 1, 1, 56)], 1, False, 1),
+}
+
+# kernels the per-layer tables under profiles/ show for these layers (kernel family and row of the tile table)
+EXPECTED = {
+    ("resnet50_b32_fused", "conv1"): "conv_stream<stem_p32",
+    ("resnet50_b32_fused", "res2a_branch2b"): "conv_chain<3 stages",
+    ("resnet50_b32_fused", "res2c_branch2b"): "conv_chain<2 stages",
+    ("resnet50_b32_fused", "res3a_branch2b"): "conv_bdir<bdir_p128_f64",
+    ("resnet50_b32_fused", "res4a_branch2b"): "conv_bdir<bdir_p64_f64",
+    ("resnet50_b32_fused", "res4a_branch2c"): "conv_wsl<wsl_p128",
+    ("resnet50_b32_fused", "res5a_branch2b"): "conv_bdir<bdir_k2_p64_f64",
+    ("vgg16_b16", "conv6"): "conv_mfma<p256_f128",
+    ("vgg16_b16", "conv9"): "conv_bdir<bdir_p128_f128",
+    ("mobilenet_v2_b32", "b2_dw"): "conv_dw3x3_kernel",
+    ("mobilenet_v2_b32", "b2_expand"): "conv_stream<stream_p32",
+    ("c1", "c1"): "conv_bdir<bdir_p64_f64",
+}
+
+
+def groups_of(layers, fuse):
+    """the launches bench.py forms: a spatial layer with the 1x1 followers that may chain behind it, else single layers"""
+    out, i = [], 0
+    while i < len(layers):
+        n = 1
+        if layers[i]["k"] > 1 and layers[i]["groups"] == 1 and layers[i]["ifm"] % 64 == 0:
+            while n < 3 and i + n < len(layers):
+                l, q = layers[i + n], layers[i + n - 1]
+                if not (l["follows_prev"] and l["k"] == 1 and l["stride"] == 1 and l["groups"] == 1 and l["ifm"] == q["ofm"]
+                        and l["in_hw"] == q["out_hw"] and (not q["closes_block"] or fuse)):
+                    break
+                n += 1
+        out.append(layers[i:i + n])
+        i += n
+    return out
+
+
+def signature(group, fuse):
+    return tuple((l["ifm"], l["ofm"], l["k"], l["stride"], l["pad"], l["in_hw"], l["groups"], l["act"], bool(l["closes_block"] and fuse))
+                 for l in group)
+
+
+def cases():
+    out = []
+    for wl, (layers, batch, fuse, images) in CONFIGS.items():
+        seen = set()
+        for g in groups_of(layers, fuse):
+            s = signature(g, fuse)
+            if s in seen and (wl, g[0]["name"]) not in EXPECTED:
+                continue
+            seen.add(s)
+            out.append(pytest.param(wl, [dict(l) for l in g], id="%s-%s" % (wl, g[0]["name"] + ("+%d" % (len(g) - 1) if len(g) > 1 else ""))))
+    return out
+
+
+@pytest.fixture(scope="module")
+def eng():
+    e = hip.Engine()
+    yield e
+    e.close()
+
+
+@pytest.mark.parametrize("wl,group", cases())
+def test_layer_at_its_real_batch_matches_the_oracle(eng, wl, group):
+    _, batch, fuse, images = CONFIGS[wl]
+    stack = bench.build_stack(eng, group, batch, fuse)
+    head = stack[0]
+    name = head.info.kernel_name.decode()
+    assert not name.startswith("conv_ref"), name  # every layer of the configurations runs on a fast kernel
+    want = EXPECTED.get((wl, group[0]["name"]))
+    if want:
+        assert name.startswith(want), "%s runs on %s, the profile shows %s" % (group[0]["name"], name, want)
+    bench.run_step(bench.launches(stack))
+    eng.finish()
+    _, _, checked, mismatches = bench.cpu_pass(eng, stack, min(images, batch), verify=True)
+    kept = [L for L in stack if L.kept]
+    assert checked == sum(min(images, batch) * L.spec["ofm"] * L.spec["out_hw"] ** 2 for L in kept)
+    assert mismatches == 0, "%d of %d outputs differ from the oracle (%s)" % (mismatches, checked, name)
+    bench.release_stack(stack)
