@@ -174,16 +174,23 @@ void build(cldnn_hip_conv c, const void* weights, const void* bias, const float*
     const bool stem = d.input.format == CLDNN_HIP_FMT_B_FS_YX_FSV4 && d.output.format == CLDNN_HIP_FMT_FS_B_YX_FSV16
                       && (!d.fused || p.eltw_t.format == CLDNN_HIP_FMT_FS_B_YX_FSV16) && d.ifm <= 4 && d.groups == 1
                       && d.dilation_x == 1 && conv_border_covers(p) && (p.FY * ((p.FX + 3) / 4) + 3) / 4 <= 8;
+    // Grouped (not depthwise) convolutions run on the same matrix-core kernels as one dense convolution whose weight
+    // matrix is block-diagonal: feature f only has weights for the input features of its own group, the rest are zero.
+    // That is the arithmetic of the reference's per-group launches (fused_conv_eltwise_gpu_ref.cl:108-112,134-136) in one
+    // launch; the zero blocks cost matrix-core time that these layers do not miss (they are bound by launch and memory),
+    // and dense weights of more than 64 MiB stay on the one-thread-per-output kernel.
+    const bool grouped = d.groups > 1 && !depthwise;
+    const bool grouped_dense = grouped && blocked && (size_t)d.ofm * d.ifm * d.fy * d.fx <= ((size_t)64 << 20);
     int impl = d.impl;
     if (impl == CLDNN_HIP_IMPL_AUTO) {
-        if ((blocked || stem) && int_path && d.groups == 1) impl = CLDNN_HIP_IMPL_MFMA;
+        if ((blocked || stem) && int_path && (d.groups == 1 || grouped_dense)) impl = CLDNN_HIP_IMPL_MFMA;
         else if (blocked && int_path && depthwise) impl = CLDNN_HIP_IMPL_DEPTHWISE;
         else impl = CLDNN_HIP_IMPL_REF;
     }
     if (impl == CLDNN_HIP_IMPL_MFMA)
-        CHIP_REQUIRE((blocked || stem) && int_path && d.groups == 1, CLDNN_HIP_UNSUPPORTED_FORMAT,
+        CHIP_REQUIRE((blocked || stem) && int_path && (d.groups == 1 || grouped_dense), CLDNN_HIP_UNSUPPORTED_FORMAT,
                      "the MFMA kernel needs int8 data in fs_b_yx_fsv16 (first layers: bordered b_fs_yx_fsv4 input), "
-                     "quantisation and groups == 1");
+                     "quantisation, and groups == 1 or a block-diagonal weight matrix of at most 64 MiB");
     if (impl == CLDNN_HIP_IMPL_DEPTHWISE)
         CHIP_REQUIRE(blocked && int_path && depthwise, CLDNN_HIP_UNSUPPORTED_FORMAT,
                      "the depthwise kernel needs int8 data in fs_b_yx_fsv16, quantisation and groups == features");
@@ -252,6 +259,18 @@ void build(cldnn_hip_conv c, const void* weights, const void* bias, const float*
         e.bias_dt = CLDNN_HIP_NO_TYPE;
     }
 
+    std::vector<int8_t> dense;
+    if (impl == CLDNN_HIP_IMPL_MFMA && grouped) {
+        // [ofm][ifm / groups][fy][fx] -> block-diagonal [ofm][ifm][fy][fx]
+        const size_t taps = (size_t)p.FY * p.FX, ofm_g = (size_t)p.OFM / p.groups;
+        dense.assign((size_t)p.OFM * p.IFM * taps, 0);
+        for (int f = 0; f < p.OFM; ++f) {
+            const size_t g = (size_t)f / ofm_g;
+            std::memcpy(&dense[((size_t)f * p.IFM + g * ifm_g) * taps], w8 + (size_t)f * ifm_g * taps, (size_t)ifm_g * taps);
+        }
+        w8 = dense.data();
+        p.groups = 1;  // from here on the problem is the dense one (the algorithmic work above counts the real weights)
+    }
     if (impl == CLDNN_HIP_IMPL_MFMA) {
         int tile = d.tile_override > 0 ? d.tile_override - 1 : mfma_choose(p, c->engine->props.multiProcessorCount);
         CHIP_REQUIRE(tile >= 0 && tile < tile_config_count(), CLDNN_HIP_INVALID_ARG, "tile_override out of range");
@@ -408,6 +427,7 @@ cldnn_hip_status cldnn_hip_conv_chain_create(cldnn_hip_engine e, int32_t count, 
                 CHIP_REQUIRE(c->impl == CLDNN_HIP_IMPL_MFMA, CLDNN_HIP_UNSUPPORTED_FORMAT,
                              "stage " + std::to_string(k) + " of a chain must be a dense int8 convolution in fs_b_yx_fsv16");
                 CHIP_REQUIRE(!descs[k].second_input_in_output, CLDNN_HIP_UNSUPPORTED_FORMAT, "a chained stage cannot read its residual from its own output");
+                CHIP_REQUIRE(descs[k].groups == 1, CLDNN_HIP_UNSUPPORTED_FORMAT, "a chained stage cannot be a grouped convolution");
                 ch->keep[k] = keep_output ? (keep_output[k] != 0) : 1;
                 ch->in[k] = ChainStageIn{&c->p, &c->epi, &c->fe, c->fast, (const int32_t*)c->acc_init};
             }

@@ -614,7 +614,11 @@ static bool wants_blocked(node* n)
     if (!int_mode) return false;
     const int groups = p.groups ? (int)p.groups : 1;
     const bool depthwise = groups > 1 && groups == in.size.sizes[1] && groups == w->out.size.sizes[0];
-    return groups == 1 || depthwise;
+    if (groups == 1 || depthwise) return true;
+    // other group counts run on the matrix-core kernels with a block-diagonal weight matrix, up to 64 MiB of it
+    if (p.weights.size() != 1) return false;
+    const size_t dense = (size_t)w->out.size.sizes[0] * (size_t)in.size.sizes[1] * (size_t)w->out.size.sizes[2] * (size_t)w->out.size.sizes[3];
+    return dense <= ((size_t)64 << 20);
 }
 
 // The layout rule that stands where the reference has byxf_af32 / fs_bs_yx_bsv4_fsv32 (which its own

@@ -628,8 +628,52 @@ def test_error_paths(eng):
     with pytest.raises(hip.HipError) as ei:
         hip.Conv(eng, d, w)
     assert ei.value.status == -2
-    d = hip.conv_desc(xin.tensor, w.shape, "s8", pad=(1, 1), has_wqf=True, groups=2, impl=hip.IMPL_MFMA)
-    d.ifm = 16
+    plain = hip.upload(eng, x, "bfyx")  # the matrix-core kernels read the blocked layout only
+    d = hip.conv_desc(plain.tensor, w.shape, "s8", pad=(1, 1), has_wqf=True, impl=hip.IMPL_MFMA)
     with pytest.raises(hip.HipError) as ei:
-        hip.Conv(eng, d, np.zeros((16, 8, 3, 3), np.int8), None, np.ones(16, np.float32))
+        hip.Conv(eng, d, w, None, np.ones(16, np.float32))
     assert ei.value.status == -6
+    d = hip.conv_desc(xin.tensor, (16, 1, 3, 3), "s8", pad=(1, 1), has_wqf=True, groups=16, impl=hip.IMPL_MFMA)  # depthwise has its own kernel
+    with pytest.raises(hip.HipError) as ei:
+        hip.Conv(eng, d, np.zeros((16, 1, 3, 3), np.int8), None, np.ones(16, np.float32))
+    assert ei.value.status == -6
+
+
+@pytest.mark.parametrize("in_dt", [np.uint8, np.int8], ids=["u8", "s8"])
+@pytest.mark.parametrize("shape", [(2, 64, 10, 9, 64, 3, 2), (3, 128, 7, 7, 128, 3, 32), (2, 48, 6, 6, 96, 1, 3), (1, 256, 14, 14, 256, 3, 4)],
+                         ids=["g2_3x3", "g32_3x3_resnext", "g3_1x1_ifm16", "g4_3x3"])
+def test_grouped_convolution_on_the_matrix_core_kernels(eng, shape, in_dt):
+    """2 <= groups < features: one launch of the dense kernels on a block-diagonal weight matrix.  Accumulators and
+    requantised outputs equal the oracle's grouped convolution, and the oracle's grouped result equals its dense result
+    on the block-diagonal expansion (the identity the kernel relies on)."""
+    B, IFM, H, W, OFM, FK, G = shape
+    r = np.random.default_rng(41)
+    lo, hi = (0, 256) if in_dt == np.uint8 else (-128, 128)
+    x = r.integers(lo, hi, (B, IFM, H, W)).astype(in_dt)
+    w = r.integers(-127, 128, (OFM, IFM // G, FK, FK)).astype(np.int8)
+    bias = r.integers(-1000, 1001, OFM).astype(np.int32)
+    wqf = np.ones(OFM, np.float32)
+    calib = (40.0 / (np.sqrt(IFM // G * FK * FK) * 147.4 * 73.3) * r.uniform(0.5, 2.0, OFM)).astype(np.float32)
+    pad = FK // 2
+    kw = dict(stride=(1, 1), pad=(pad, pad), groups=G, out_dt="s8", act="relu")
+    (ro, ra), (go, ga, info) = both(eng, x, w, bias, wqf, calib, fmt="fs_b_yx_fsv16", in_pad=(pad, pad), **kw)
+    name = info.kernel_name.decode()
+    assert info.impl == hip.IMPL_MFMA and not name.startswith("conv_ref"), name
+    assert info.ops == 2 * ro.size * (IFM // G) * FK * FK  # algorithmic work counts the real weights
+    np.testing.assert_array_equal(ga, ra)
+    assert_same(ro, go)
+    dense = np.zeros((OFM, IFM, FK, FK), np.int8)
+    for f in range(OFM):
+        g = f // (OFM // G)
+        dense[f, g * (IFM // G):(g + 1) * (IFM // G)] = w[f]
+    assert np.array_equal(rc.conv(x, dense, bias, wqf=wqf, calib=calib, stride=(1, 1), pad=(pad, pad), out_dt="s8", act="relu"), ro)
+    # the fused residual form
+    e = r.integers(-128, 128, (B, OFM, H, W)).astype(np.int8)
+    ecal = r.uniform(0.3, 1.2, OFM).astype(np.float32)
+    kw = dict(stride=(1, 1), pad=(pad, pad), groups=G, out_dt="s8", act="none", eltw=e, eltw_act="relu", eltw_calib=ecal)
+    (ro, ra), (go, ga, info) = both(eng, x, w, bias, wqf, calib, fmt="fs_b_yx_fsv16", in_pad=(pad, pad), **kw)
+    assert info.impl == hip.IMPL_MFMA
+    assert_same(ro, go)
+    # plain layouts keep the one-thread-per-output kernel
+    _, (go, ga, info) = both(eng, x, w, bias, wqf, calib, fmt="bfyx", stride=(1, 1), pad=(pad, pad), groups=G, out_dt="s8", act="relu")
+    assert info.impl == hip.IMPL_REF

@@ -335,15 +335,21 @@ def test_conv_eltwise_not_fused(kw):
     assert "conv2" in ids and "sum" in ids
 
 
-@pytest.mark.parametrize("kw", [dict(groups=2), dict(quantized=False)], ids=["grouped", "unquantized"])
-def test_int8_convolutions_that_stay_in_a_plain_layout_are_not_fused(kw):
+def test_int8_convolutions_that_stay_on_the_plain_kernel_are_not_fused():
     """the reference fuses int8 convolutions only in its blocked int8 formats (prepare_primitive_fusing.cpp:197-205); here
-    that means the ones the layout rule runs in fs_b_yx_fsv16.  A grouped or unquantized int8 1x1 convolution stays in
-    bfyx on the reference kernel, and its relu sum stays a primitive of its own (the sum then adds to the saturated
-    int8 tensor, not to the accumulator)."""
-    opt = by_id(cl.plan(residual_block(**kw), cl.build_options(optimize_data=True)))
+    that means the ones the layout rule runs in fs_b_yx_fsv16 on the matrix-core kernels.  An unquantized int8 1x1
+    convolution stays on the one-thread-per-output kernel, and its relu sum stays a primitive of its own (the sum then
+    adds to the int8 tensor the convolution wrote, not to an accumulator)."""
+    opt = by_id(cl.plan(residual_block(quantized=False), cl.build_options(optimize_data=True)))
     assert "conv2" in opt and "sum" in opt and "conv2_fused_sum" not in opt
     assert opt["conv2"]["type"] == "convolution" and opt["sum"]["type"] == "eltwise"
+
+
+def test_grouped_quantized_convolution_is_blocked_and_fused():
+    """a grouped (not depthwise) quantized convolution runs on the matrix-core kernels too (block-diagonal weights), so
+    the layout rule blocks it and the fusing pass treats it like any other blocked convolution"""
+    opt = by_id(cl.plan(residual_block(groups=2), cl.build_options(optimize_data=True)))
+    assert "conv2_fused_sum" in opt and opt["conv2_fused_sum"]["format"] == F.fs_b_yx_fsv16
 
 
 def test_sum_without_activation_is_fused_with_the_saturation_kept():
@@ -471,13 +477,18 @@ def test_layout_rule_keeps_user_blocked_tensors():
     assert by_id(opt)["conv"]["format"] == F.fs_b_yx_fsv16
 
 
-@pytest.mark.parametrize("kw", [dict(quant=False), dict(in_dt=DT.f32), dict(IFM=16, OFM=8, groups=2)])
+@pytest.mark.parametrize("kw", [dict(quant=False), dict(in_dt=DT.f32), dict(IFM=16, OFM=8, groups=2, quant=False)])
 def test_layout_rule_leaves_other_convolutions_alone(kw):
     if kw.get("in_dt") == DT.f32:
         kw = dict(kw, quant=False)
     opt = cl.plan(conv_topology(**kw), cl.build_options(optimize_data=True))
     assert not any("fsv16" in n["id"] for n in opt)
     assert by_id(opt)["conv"]["format"] == F.bfyx
+
+
+def test_layout_rule_takes_grouped_quantized_convolutions():
+    opt = by_id(cl.plan(conv_topology(IFM=16, OFM=8, groups=2), cl.build_options(optimize_data=True)))
+    assert opt["conv_fsv16"]["type"] == "convolution" and opt["conv_fsv16"]["format"] == F.fs_b_yx_fsv16
 
 
 def test_layout_rule_takes_depthwise():

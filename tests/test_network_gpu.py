@@ -368,31 +368,51 @@ def test_fused_and_unfused_graphs_agree(eng):
 
 
 @pytest.mark.parametrize("optimize", OPT, ids=["plain", "optimize_data"])
-def test_grouped_convolution_keeps_its_sum_unfused_on_saturating_data(eng, optimize):
-    """a grouped int8 1x1 convolution stays on the plain-layout kernel and, as in the reference
-    (prepare_primitive_fusing.cpp:197-205), its relu sum stays a primitive of its own: the sum adds to the SATURATED int8
-    tensor.  The factors are chosen so that a good share of the convolution's results leave the int8 range, where the
-    fused arithmetic (sum on the unsaturated value) would give other numbers."""
+def test_unquantized_int8_convolution_keeps_its_sum_unfused(eng, optimize):
+    """an int8 1x1 convolution without quantization factors stays on the plain-layout kernel (its accumulator is the
+    8-bit type, wrap-around included, fused_conv_eltwise_gpu_ref.cl:43-48) and, as in the reference
+    (prepare_primitive_fusing.cpp:197-205), its relu sum stays a primitive of its own: the sum adds to the int8 tensor
+    the convolution wrote.  The fused primitive would accumulate in int and give other numbers on this data."""
     r = np.random.default_rng(23)
-    B, Cn, H, W, G = 2, 32, 6, 7, 2
+    B, Cn, H, W = 2, 32, 6, 7
     x = r.integers(-128, 128, (B, Cn, H, W)).astype(np.int8)
-    w = r.integers(-127, 128, (Cn, Cn // G, 1, 1)).astype(np.int8)
-    cal = r.uniform(4e-3, 1.2e-2, Cn).astype(np.float32)  # accumulators of a few 10^4: results around +-200
+    w = r.integers(-3, 4, (Cn, Cn, 1, 1)).astype(np.int8)
     ecal = r.uniform(0.4, 0.9, Cn).astype(np.float32)
     t = cl.topology(cl.input_layout("input", cl.layout(DT.i8, F.bfyx, cl.tensor(B, Cn, W, H))), cl.data("w", cl.make_memory(eng, w)),
-                    cl.data("q", vec_mem(eng, np.ones(Cn, np.float32))), cl.data("c", vec_mem(eng, cal)), cl.data("e", vec_mem(eng, ecal)),
-                    cl.convolution("conv", "input", ["w"], None, ["q"], ["c"], groups=G),
+                    cl.data("e", vec_mem(eng, ecal)),
+                    cl.convolution("conv", "input", ["w"]),
                     cl.eltwise("sum", "input", "conv", cl.eltwise_mode.sum, True, 0.0, output_calibration_factors="e"),
                     cl.reorder("out", "sum", F.bfyx))
     net, outs = run(eng, t, {"input": cl.make_memory(eng, x)}, optimize)
-    conv = rc.conv(x, w, None, wqf=np.ones(Cn, np.float32), calib=cal, groups=G, out_dt="s8")
-    assert np.count_nonzero(np.abs(conv) == 127) + np.count_nonzero(conv == -128) > conv.size // 10  # it does saturate
+    conv = rc.conv(x, w, None)  # 8-bit accumulation
+    exact = np.einsum("bchw,fc->bfhw", x.astype(np.int64), w[:, :, 0, 0].astype(np.int64))
+    assert np.count_nonzero(conv.astype(np.int64) != exact) > conv.size // 4  # it does wrap around
     expected = rc.eltwise_sum(x, conv, calib=ecal, relu=True)
-    fused_form = rc.conv(x, w, None, wqf=np.ones(Cn, np.float32), calib=cal, groups=G, out_dt="s8", eltw=x, eltw_act="relu", eltw_calib=ecal)
-    assert np.count_nonzero(fused_form != expected) > 0  # the two arithmetics do differ on this data
     np.testing.assert_array_equal(outs["out"].get_memory().read(), expected)
     executed = net.get_executed_primitive_ids()
     assert "conv" in executed and "sum" in executed
+
+
+@pytest.mark.parametrize("optimize", OPT, ids=["plain", "optimize_data"])
+def test_grouped_quantized_convolution_through_network(eng, optimize):
+    """groups = 4 with quantization: as written on the plain-layout kernel, with optimize_data blocked on the matrix-core
+    kernels (block-diagonal weights); same numbers, those of the oracle's grouped convolution"""
+    r = np.random.default_rng(29)
+    B, Cn, OFM, H, W, G = 2, 64, 96, 9, 8, 4
+    x = r.integers(-128, 128, (B, Cn, H, W)).astype(np.int8)
+    w = r.integers(-127, 128, (OFM, Cn // G, 3, 3)).astype(np.int8)
+    bias = r.integers(-1000, 1001, OFM).astype(np.int32)
+    cal = (40.0 / (np.sqrt(Cn // G * 9) * 73.9 * 73.3) * r.uniform(0.5, 2.0, OFM)).astype(np.float32)
+    t = cl.topology(cl.input_layout("input", cl.layout(DT.i8, F.bfyx, cl.tensor(B, Cn, W, H))), cl.data("w", cl.make_memory(eng, w)),
+                    cl.data("b", vec_mem(eng, bias)), cl.data("q", vec_mem(eng, np.ones(OFM, np.float32))), cl.data("c", vec_mem(eng, cal)),
+                    cl.convolution("conv", "input", ["w"], ["b"], ["q"], ["c"], groups=G, input_offset=cl.tensor(0, 0, -1, -1, 0),
+                                   with_activation=True),
+                    cl.reorder("out", "conv", F.bfyx))
+    net, outs = run(eng, t, {"input": cl.make_memory(eng, x)}, optimize)
+    expected = rc.conv(x, w, bias, wqf=np.ones(OFM, np.float32), calib=cal, groups=G, pad=(1, 1), out_dt="s8", act="relu")
+    np.testing.assert_array_equal(outs["out"].get_memory().read(), expected)
+    kernel = net.get_primitive_info("conv")["kernel"]
+    assert kernel.startswith("conv_ref") != bool(optimize), kernel
 
 
 def test_closer_writes_over_its_shortcut_without_a_memory_pool():
