@@ -36,6 +36,29 @@ class Layer:
     pass
 
 
+def chain_groups(layers, fuse_residual):
+    """The launches a stack is cut into: a spatial layer (a dense convolution on multiples of 64 features, or a
+    depthwise 3x3) together with the one or two 1x1 / stride-1 layers that read its result in the network
+    (follows_prev), else the layer alone.  Whether the library accepts a group as a chain is decided when it is built."""
+    out, i = [], 0
+    while i < len(layers):
+        n = 1
+        h = layers[i]
+        dense_head = h["groups"] == 1 and h["ifm"] % 64 == 0
+        dw_head = h["k"] == 3 and h["groups"] == h["ifm"] == h["ofm"]
+        if h["k"] > 1 and (dense_head or dw_head):
+            while n < 3 and i + n < len(layers):
+                l, q = layers[i + n], layers[i + n - 1]
+                ok = l["follows_prev"] and l["k"] == 1 and l["stride"] == 1 and l["groups"] == 1 and l["ifm"] == q["ofm"] \
+                    and l["in_hw"] == q["out_hw"] and (not q["closes_block"] or fuse_residual)
+                if not ok:
+                    break
+                n += 1
+        out.append(layers[i:i + n])
+        i += n
+    return out
+
+
 def build_stack(eng, layers, batch, fuse_residual, seed=1337, tile=0, in_dt=np.uint8, chains=True):
     """Create device tensors and convolution objects for every layer (seeded synthetic data).
 
@@ -47,20 +70,11 @@ def build_stack(eng, layers, batch, fuse_residual, seed=1337, tile=0, in_dt=np.u
     follows = set()  # indices of layers that run as stage 1 / 2 of a chain
     if chains and not tile:
         i = 0
-        while i < len(layers):
-            n = 1
-            if layers[i]["k"] > 1 and layers[i]["groups"] == 1 and layers[i]["ifm"] % 64 == 0:
-                while n < 3 and i + n < len(layers):
-                    l, q = layers[i + n], layers[i + n - 1]
-                    ok = l["follows_prev"] and l["k"] == 1 and l["stride"] == 1 and l["groups"] == 1 and l["ifm"] == q["ofm"] \
-                        and l["in_hw"] == q["out_hw"] and (not q["closes_block"] or fuse_residual)
-                    if not ok:
-                        break
-                    n += 1
-            if n > 1:
-                layers[i] = dict(layers[i], chain_len=n)
-                follows.update(range(i + 1, i + n))
-            i += n
+        for group in chain_groups(layers, fuse_residual):
+            if len(group) > 1:
+                layers[i] = dict(layers[i], chain_len=len(group))
+                follows.update(range(i + 1, i + len(group)))
+            i += len(group)
     for i, l in enumerate(layers):
         r = np.random.default_rng(seed + i)
         L = Layer()

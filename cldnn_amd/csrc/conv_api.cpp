@@ -424,12 +424,15 @@ cldnn_hip_status cldnn_hip_conv_chain_create(cldnn_hip_engine e, int32_t count, 
                                                                   calib ? calib[k] : nullptr, eltw_calib ? eltw_calib[k] : nullptr, &c);
                 if (st != CLDNN_HIP_SUCCESS) throw error(st, std::string("stage ") + std::to_string(k) + ": " + cldnn_hip_last_error());
                 ch->stage[k] = c;
-                CHIP_REQUIRE(c->impl == CLDNN_HIP_IMPL_MFMA, CLDNN_HIP_UNSUPPORTED_FORMAT,
-                             "stage " + std::to_string(k) + " of a chain must be a dense int8 convolution in fs_b_yx_fsv16");
+                const bool dw_head = k == 0 && c->impl == CLDNN_HIP_IMPL_DEPTHWISE && c->w_masked;
+                CHIP_REQUIRE(c->impl == CLDNN_HIP_IMPL_MFMA || dw_head, CLDNN_HIP_UNSUPPORTED_FORMAT,
+                             "stage " + std::to_string(k) + " of a chain must be a dense int8 convolution in fs_b_yx_fsv16 (the first "
+                             "stage may be a depthwise 3x3)");
                 CHIP_REQUIRE(!descs[k].second_input_in_output, CLDNN_HIP_UNSUPPORTED_FORMAT, "a chained stage cannot read its residual from its own output");
-                CHIP_REQUIRE(descs[k].groups == 1, CLDNN_HIP_UNSUPPORTED_FORMAT, "a chained stage cannot be a grouped convolution");
+                CHIP_REQUIRE(descs[k].groups == 1 || dw_head, CLDNN_HIP_UNSUPPORTED_FORMAT, "a chained stage cannot be a grouped convolution");
                 ch->keep[k] = keep_output ? (keep_output[k] != 0) : 1;
-                ch->in[k] = ChainStageIn{&c->p, &c->epi, &c->fe, c->fast, (const int32_t*)c->acc_init};
+                ch->in[k] = ChainStageIn{&c->p, &c->epi, &c->fe, c->fast, (const int32_t*)c->acc_init,
+                                         dw_head ? (const int32_t*)c->w_masked : nullptr};
             }
             CHIP_REQUIRE(ch->keep[count - 1], CLDNN_HIP_INVALID_ARG, "the last stage of a chain always writes its output");
             const int cus = e->props.multiProcessorCount;
@@ -454,7 +457,7 @@ cldnn_hip_status cldnn_hip_conv_chain_create(cldnn_hip_engine e, int32_t count, 
             CHIP_CHECK(hipMemcpyAsync(ch->packed, packed.data(), packed.size(), hipMemcpyHostToDevice, e->stream));
             CHIP_CHECK(hipStreamSynchronize(e->stream));
             cldnn_hip_conv_info& inf = ch->info;
-            inf.impl = CLDNN_HIP_IMPL_MFMA, inf.tile_index = -1, inf.tile_pixels = 64 * ch->plan.nt, inf.tile_ofm = 64;
+            inf.impl = CLDNN_HIP_IMPL_MFMA, inf.tile_index = -1, inf.tile_pixels = 64 * (ch->plan.dw ? 4 : ch->plan.nt), inf.tile_ofm = 64;
             inf.grid = ch->plan.grid, inf.block = 256, inf.lds_bytes = ch->plan.lds_bytes;
             std::snprintf(inf.kernel_name, sizeof(inf.kernel_name), "%s", ch->plan.name);
             // algorithmic work of the chain: every stage's operations; bytes of what has to cross the memory interface,

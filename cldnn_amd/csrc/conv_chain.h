@@ -14,10 +14,14 @@ struct ChainStageIn {
     const FastEpi* fe;
     bool fast;                 // the short int8 epilogue applies
     const int32_t* acc_init;   // device
+    // a depthwise first stage (3x3, masked weights of the stand-alone depthwise kernel): device pointers, else nullptr
+    const int32_t* dw_wmask = nullptr;
 };
 
 struct ChainPlan {
     int stages;
+    int dw;                    // 1: the first stage is a depthwise 3x3 on the vector ALU (granules of 64 pixels), the LDS
+                               // image holds the units and vectors of the later stages only
     int nt;                    // 16-pixel fragments per wave and granule
     int depth;                 // activation look-ahead of stage 0 in K-steps
     int ksteps0;               // K-steps of stage 0 (padded to a multiple of depth)

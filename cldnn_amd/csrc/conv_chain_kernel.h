@@ -95,6 +95,9 @@ __device__ __forceinline__ void chain_scales(const ChainStage& st, const int32_t
 {
     if constexpr (EPI == EPI_KIND_RELU || EPI == EPI_KIND_LINEAR) {
         chain_vec16(ldsV, st.vec0 + spans * 64 + f0, sc.cal);
+    } else if constexpr (EPI == EPI_KIND_CLAMPQ) {
+        chain_vec16(ldsV, st.vec0 + spans * 64 + f0, sc.cal);
+        chain_vec16(ldsV, st.vec0 + 3 * spans * 64 + f0, sc.wq);
     } else if constexpr (EPI == EPI_KIND_FUSED) {
         chain_vec16(ldsV, st.vec0 + spans * 64 + f0, sc.cal);
         chain_vec16(ldsV, st.vec0 + 2 * spans * 64 + f0, sc.ecal);

@@ -82,7 +82,9 @@ struct MfmaArgs {
 //   RELU   clamp(acc * cal, 0, hi)                                    (relu, scales >= 0, unit wqf)
 //   FUSED  clamp((round(acc * cal) + residual) * ecal, 0, hi)         (residual relu, scales >= 0)
 //   LINEAR clamp(acc * cal, lo, hi)                                   (no activation, unit wqf)
-enum { EPI_KIND_GENERIC = 0, EPI_KIND_FAST = 1, EPI_KIND_RELU = 2, EPI_KIND_FUSED = 3, EPI_KIND_LINEAR = 4 };
+//   CLAMPQ clamp(acc * wqf, m, n) * cal, rounded                      (folded clamp{m, n} with 0 <= m, e.g. ReLU6 on the
+//                                                                      dequantised value; unit input factor; chain kernels)
+enum { EPI_KIND_GENERIC = 0, EPI_KIND_FAST = 1, EPI_KIND_RELU = 2, EPI_KIND_FUSED = 3, EPI_KIND_LINEAR = 4, EPI_KIND_CLAMPQ = 5 };
 template <int EPI> struct epi_is_short { static constexpr bool value = EPI != EPI_KIND_GENERIC; };
 
 // Workgroup barrier that orders LDS traffic only.  __syncthreads() also drains every outstanding
@@ -203,6 +205,26 @@ __device__ __forceinline__ v4i epilogue_fast16(const Args& a, const v4i (&acc)[4
         }
 #pragma unroll
         for (int d = 0; d < 4; ++d) packed[d] = pack_signed(v + d * 4);
+        if (valid < 16) {
+#pragma unroll
+            for (int d = 0; d < 4; ++d) {
+                unsigned keep = 0;
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                    if (d * 4 + i < valid) keep |= 255u << (8 * i);
+                packed[d] &= (int)keep;
+            }
+        }
+        return packed;
+    }
+    if constexpr (EPI == EPI_KIND_CLAMPQ) {
+        // clamp{m, n} on the dequantised value, then the calibration: the result lies in [0, n * factor], which the host
+        // has checked to be inside the output range (the clamp_folded case of the run-time form below)
+        v4i packed;
+#pragma unroll
+        for (int c = 0; c < 16; ++c) v[c] = med3(v[c] * wq[c], F.act_m, F.act_n) * cal[c] + 0.49999997f;
+#pragma unroll
+        for (int d = 0; d < 4; ++d) packed[d] = pack_nonneg(v + d * 4);
         if (valid < 16) {
 #pragma unroll
             for (int d = 0; d < 4; ++d) {

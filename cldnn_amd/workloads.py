@@ -57,13 +57,14 @@ def mobilenet_v2():
             stride = s if i == 0 else 1
             idx += 1
             mid = cin * t
+            # the stack has no residual sums, so every layer reads what the one before it writes
             if t != 1:
-                L.append(_layer("b%d_expand" % idx, cin, mid, 1, 1, 0, hw, act="relu6"))
-            L.append(_layer("b%d_dw" % idx, mid, mid, 3, stride, 1, hw, groups=mid, act="relu6"))
+                L.append(_layer("b%d_expand" % idx, cin, mid, 1, 1, 0, hw, act="relu6", follows_prev=True))
+            L.append(_layer("b%d_dw" % idx, mid, mid, 3, stride, 1, hw, groups=mid, act="relu6", follows_prev=True))
             hw = (hw + 2 - 3) // stride + 1
-            L.append(_layer("b%d_project" % idx, mid, c, 1, 1, 0, hw, act="none"))
+            L.append(_layer("b%d_project" % idx, mid, c, 1, 1, 0, hw, act="none", follows_prev=True))
             cin = c
-    L.append(_layer("conv_last", cin, 1280, 1, 1, 0, hw, act="relu6"))
+    L.append(_layer("conv_last", cin, 1280, 1, 1, 0, hw, act="relu6", follows_prev=True))
     assert len(L) == 52, len(L)
     return L
 

@@ -146,3 +146,66 @@ def test_chain_refusals(eng):
     with pytest.raises(hip.HipError) as err:
         hip.ConvChain(eng, spec, [False, True, True])
     assert err.value.status == -6 and "LDS" in str(err.value)
+
+
+# ------------------------------------------------------------------ depthwise chains (MobileNet blocks)
+def relu6_layer(r, ofm, ifm_g, k, act):
+    """factors as the benchmark's MobileNet stack has them: a clamp{0, 6} acts on the dequantised value"""
+    w = r.integers(-127, 128, (ofm, ifm_g, k, k)).astype(np.int8)
+    bias = r.integers(-1000, 1001, ofm).astype(np.int32)
+    if act == "relu6":
+        sig = np.sqrt(ifm_g * k * k) * 100.0 * 73.3
+        wqf = (3.0 / sig * r.uniform(0.5, 2.0, ofm)).astype(np.float32)
+        calib = np.full(ofm, 127.0 / 6.0, np.float32)
+        kw = dict(act="clamp", act_m=0.0, act_n=6.0)
+    else:
+        wqf = np.ones(ofm, np.float32)
+        calib = (40.0 / (np.sqrt(ifm_g * k * k) * 60.0 * 73.3) * r.uniform(0.5, 2.0, ofm)).astype(np.float32)
+        kw = dict(act="none")
+    return w, bias, wqf, calib, kw
+
+
+@pytest.mark.parametrize("in_dt", [np.uint8, np.int8], ids=["u8", "s8"])
+@pytest.mark.parametrize("mid,proj,stride,stages", [(32, 16, 1, 3), (96, 24, 2, 3), (144, 32, 1, 3), (192, 64, 2, 3), (384, 64, 1, 3),
+                                                    (144, 24, 1, 2)],
+                         ids=["b1", "b2_s2", "b4", "b7_s2", "b8", "two_stages"])
+def test_depthwise_chain_matches_the_oracle(eng, mid, proj, stride, stages, in_dt):
+    """depthwise 3x3 -> 1x1 projection -> 1x1 expansion of the next block in one launch, against the three
+    convolutions of the oracle; feature counts that do not fill slices of 64 (or, for the projection, of 16), stride 2,
+    pixel counts that do not fill a 64-pixel granule, every result kept and only the needed ones"""
+    r = np.random.default_rng(33)
+    B, H, W = 3, 13, 10
+    OH, OW = (H + 2 - 3) // stride + 1, (W + 2 - 3) // stride + 1
+    lo, hi = (0, 256) if in_dt == np.uint8 else (-128, 128)
+    x = r.integers(lo, hi, (B, mid, H, W)).astype(in_dt)
+    shapes = [(mid, 1, 3, "relu6", mid), (proj, mid, 1, "none", 1), (6 * proj, proj, 1, "relu6", 1)][:stages]
+    xin = hip.upload(eng, x, "fs_b_yx_fsv16", (1, 1))
+    spec, refs, bufs = [], [], []
+    prev_t, ref_in = xin.tensor, x
+    for k, (ofm, ifm_g, fk, act, groups) in enumerate(shapes):
+        w, bias, wqf, calib, akw = relu6_layer(r, ofm, ifm_g, fk, act)
+        s = stride if k == 0 else 1
+        d = hip.conv_desc(prev_t, w.shape, "s8", stride=(s, s), pad=(fk // 2,) * 2, groups=groups, bias_dt=hip.I32, has_wqf=True,
+                          has_calib=True, **akw)
+        spec.append((d, w, bias, wqf, calib, None))
+        bufs.append(hip.Buffer(eng, d.output))
+        ref = rc.conv(ref_in, w, bias, wqf=wqf, calib=calib, stride=(s, s), pad=(fk // 2,) * 2, groups=groups, out_dt="s8", **akw)
+        refs.append(ref)
+        ref_in, prev_t = ref, hip.Tensor.make(hip.S8, hip.FS_B_YX_FSV16, B, ofm, OH, OW)
+    for keep in ([False] + [True] * (stages - 1), None):
+        ch = hip.ConvChain(eng, spec, keep)
+        assert b"conv_dwchain" in ch.info().kernel_name
+        for b in bufs:
+            b.write_raw(np.full(b.nbytes, 0x55, np.uint8))
+        ch.enqueue(xin, [b if (keep is None or keep[k]) else None for k, b in enumerate(bufs)])
+        eng.finish()
+        for k in range(stages):
+            if keep is None or keep[k]:
+                got = hip.download(eng, bufs[k])
+                bad = np.argwhere(got != refs[k])
+                assert bad.size == 0, "stage %d: %d of %d differ, first at %s" % (k, len(bad), got.size, bad[0])
+        ch.close()
+    assert len(np.unique(refs[-1])) > 8  # the data does exercise the requantisation
+    xin.close()
+    for b in bufs:
+        b.close()

@@ -32,27 +32,10 @@ EXPECTED = {
     ("resnet50_b32_fused", "res5a_branch2b"): "conv_bdir<bdir_k2_p64_f64",
     ("vgg16_b16", "conv6"): "conv_mfma<p256_f128",
     ("vgg16_b16", "conv9"): "conv_bdir<bdir_p128_f128",
-    ("mobilenet_v2_b32", "b2_dw"): "conv_dw3x3_kernel",
-    ("mobilenet_v2_b32", "b2_expand"): "conv_stream<stream_p32",
+    ("mobilenet_v2_b32", "b2_dw"): "conv_dwchain<3 stages",
+    ("mobilenet_v2_b32", "b17_dw"): "conv_dw3x3_kernel",
     ("c1", "c1"): "conv_bdir<bdir_p64_f64",
 }
-
-
-def groups_of(layers, fuse):
-    """the launches bench.py forms: a spatial layer with the 1x1 followers that may chain behind it, else single layers"""
-    out, i = [], 0
-    while i < len(layers):
-        n = 1
-        if layers[i]["k"] > 1 and layers[i]["groups"] == 1 and layers[i]["ifm"] % 64 == 0:
-            while n < 3 and i + n < len(layers):
-                l, q = layers[i + n], layers[i + n - 1]
-                if not (l["follows_prev"] and l["k"] == 1 and l["stride"] == 1 and l["groups"] == 1 and l["ifm"] == q["ofm"]
-                        and l["in_hw"] == q["out_hw"] and (not q["closes_block"] or fuse)):
-                    break
-                n += 1
-        out.append(layers[i:i + n])
-        i += n
-    return out
 
 
 def signature(group, fuse):
@@ -64,7 +47,7 @@ def cases():
     out = []
     for wl, (layers, batch, fuse, images) in CONFIGS.items():
         seen = set()
-        for g in groups_of(layers, fuse):
+        for g in bench.chain_groups(layers, fuse):
             s = signature(g, fuse)
             if s in seen and (wl, g[0]["name"]) not in EXPECTED:
                 continue
