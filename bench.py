@@ -378,30 +378,36 @@ def network_workload(args):
         "requests_in_flight": in_flight, "cpu_baseline": None, "distinct_logit_values": int(len(np.unique(logits)))}), flush=True)
 
 
+def kernel_sources_digest():
+    """sha256 over the library's sources (cldnn_amd/csrc: *.hip, *.h, *.cpp, Makefile) in name order: what a counter
+    summary under profiles/ is stamped with."""
+    import hashlib
+    d = os.path.join(ROOT, "cldnn_amd", "csrc")
+    h = hashlib.sha256()
+    for name in sorted(os.listdir(d)):
+        if name.endswith((".hip", ".h", ".cpp")) or name == "Makefile":
+            h.update(name.encode() + b"\0")
+            with open(os.path.join(d, name), "rb") as f:
+                h.update(f.read())
+    return h.hexdigest()
+
+
 def measured_traffic(workload):
     """HBM bytes per launch from the committed counter summary of this workload.  None when there is none, or when
-    the summary is older than the kernels: it carries the commit it was taken at, and any later commit that touches
-    cldnn_amd/csrc/ makes it stale."""
+    the summary is older than the kernels: it carries the digest of the library sources it was taken with (and the
+    commit, for the reader), and any change to cldnn_amd/csrc/ since makes it stale."""
     path = os.path.join(ROOT, "profiles", "conv_stack_%s_hbm_traffic.txt" % workload)
     if not os.path.exists(path):
         return None
-    value = commit = None
+    value = digest = None
     with open(path) as f:
         for line in f:
             if line.startswith("traffic_bytes_per_launch:"):
                 value = int(line.split(":")[1])
-            if line.startswith("taken_at_commit:"):
-                commit = line.split(":")[1].strip()
-    if value is None or not commit:
+            if line.startswith("kernel_sources_sha256:"):
+                digest = line.split(":")[1].strip()
+    if value is None or not digest or digest != kernel_sources_digest():
         return None
-    try:
-        import subprocess
-        later = subprocess.run(["git", "-C", ROOT, "log", "--oneline", "%s..HEAD" % commit, "--", "cldnn_amd/csrc"],
-                               stdout=subprocess.PIPE, stderr=subprocess.DEVNULL, text=True, timeout=20)
-        if later.returncode != 0 or later.stdout.strip():
-            return None
-    except Exception:
-        return None  # no git history at hand (a bare copy of the tree): the stamp cannot be checked
     return value
 
 
