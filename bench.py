@@ -366,12 +366,20 @@ def network_workload(args):
             ofm, ifm, fx, fy = plan[n["deps"][1 if n["type"] == "convolution" else 2]]["size"]
             ops += 2.0 * np.prod(n["size"]) * ifm * fx * fy
     name = "ResNet-50" if resnet else ("VGG-16" if vgg else "MobileNet-v2")
+    # what the built network launches: members of a convolution chain are written by the launch of the chain's head
+    infos = {i: net.get_primitive_info(i) for i in net.get_all_primitive_ids()}
+    followers = [i for i, inf in infos.items() if str(inf.get("kernel", "")).startswith("in the chain of")]
+    executed = [i for i, inf in infos.items() if inf.get("type") not in ("data", "input_layout")]
+    if args.per_layer:
+        for i in executed:
+            log("%-40s %s" % (i, infos[i].get("kernel", infos[i].get("type"))))
     print(json.dumps({
         "metric": "%s int8 network images/sec @b%d (whole topology through the clDNN API)" % (name, batch), "value": batch * args.steps / dt,
         "unit": "images/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": dt / args.steps * 1e3,
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "i8xi8->i32 (f32 requantisation)", "data": "synthetic",
         "config": {"workload": args.workload, "batch": batch, "primitives": primitives,
-                   "build": "optimize_data" + (", tuning cache" if args.tuning_cache else "") + (", second stream" if args.second_stream else ""), "kernels_per_execute": len([n for n in plan.values() if n["type"] not in ("data", "input_layout")]),
+                   "build": "optimize_data" + (", tuning cache" if args.tuning_cache else "") + (", second stream" if args.second_stream else ""), "primitives_per_execute": len(executed), "launches_per_execute": len(executed) - len(followers),
+                   "chained_convolutions": len(followers) + len({str(infos[i]["kernel"]) for i in followers}),
                    "executed_ops_per_step": ops, "nominal_ops_per_step": nominal},
         "roofline": {"bound": "mfma", "achieved": ops * args.steps / dt / 1e12, "peak": PEAK_INT8_OPS / 1e12, "unit": "TOP/s",
                      "frac": ops * args.steps / dt / PEAK_INT8_OPS, "traffic": None, "kernel": "all kernels of one network.execute()"},

@@ -24,6 +24,7 @@ int epilogue_kind(const ChainStageIn& s)
         if (!f.fused && f.relu_folded) kind = EPI_KIND_RELU;
         if (!f.fused && f.act == CLDNN_HIP_ACT_NONE) kind = EPI_KIND_LINEAR;
         if (f.fused && f.act == CLDNN_HIP_ACT_NONE && f.eltw_relu_folded && s.epi->eltw_calib && !f.conv_sat) kind = EPI_KIND_FUSED;
+        if (f.fused && f.act == CLDNN_HIP_ACT_NONE && f.eltw_act == CLDNN_HIP_ACT_NONE && !f.eltw_relu_folded) kind = EPI_KIND_SUMLIN;
     }
     return kind;
 }
@@ -208,12 +209,14 @@ static void launch_dwchain(hipStream_t s, const ChainStageIn* st, const ChainPla
     for (int k = 0; k < pl.stages; ++k) fill_stage(a.st[k], st[k], pl, k, outs[k], eltws ? eltws[k] : nullptr);
     // the branch-free epilogue forms of a MobileNet block (clamp on the dequantised value, linear projection, clamp), else
     // the run-time form for every stage
-    constexpr int CQ = EPI_KIND_CLAMPQ, LIN = EPI_KIND_LINEAR, ANY = EPI_KIND_FAST;
-    const bool block = pl.epi[0] == CQ && pl.epi[1] == LIN && (pl.stages < 3 || pl.epi[2] == CQ);
-#define DWCHAIN_LAUNCH(NT, HAS2)                                                                        \
-    {                                                                                                   \
-        if (block) launch_dwchain_instance<NT, 1, HAS2, CQ, LIN, CQ>(s, a, pl.grid, pl.lds_bytes);      \
-        else launch_dwchain_instance<NT, 1, HAS2, ANY, ANY, ANY>(s, a, pl.grid, pl.lds_bytes);          \
+    constexpr int CQ = EPI_KIND_CLAMPQ, LIN = EPI_KIND_LINEAR, SUM = EPI_KIND_SUMLIN, ANY = EPI_KIND_FAST;
+    const bool ends = pl.epi[0] == CQ && (pl.stages < 3 || pl.epi[2] == CQ);
+    const bool block = ends && pl.epi[1] == LIN, block_sum = ends && pl.epi[1] == SUM;  // projection without / with the block's sum
+#define DWCHAIN_LAUNCH(NT, HAS2)                                                                           \
+    {                                                                                                      \
+        if (block) launch_dwchain_instance<NT, 1, HAS2, CQ, LIN, CQ>(s, a, pl.grid, pl.lds_bytes);         \
+        else if (block_sum) launch_dwchain_instance<NT, 1, HAS2, CQ, SUM, CQ>(s, a, pl.grid, pl.lds_bytes); \
+        else launch_dwchain_instance<NT, 1, HAS2, ANY, ANY, ANY>(s, a, pl.grid, pl.lds_bytes);             \
     }
     if (pl.nt == 2) {
         if (pl.stages > 2) DWCHAIN_LAUNCH(2, true) else DWCHAIN_LAUNCH(2, false)

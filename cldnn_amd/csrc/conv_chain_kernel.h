@@ -98,7 +98,7 @@ __device__ __forceinline__ void chain_scales(const ChainStage& st, const int32_t
     } else if constexpr (EPI == EPI_KIND_CLAMPQ) {
         chain_vec16(ldsV, st.vec0 + spans * 64 + f0, sc.cal);
         chain_vec16(ldsV, st.vec0 + 3 * spans * 64 + f0, sc.wq);
-    } else if constexpr (EPI == EPI_KIND_FUSED) {
+    } else if constexpr (EPI == EPI_KIND_FUSED || EPI == EPI_KIND_SUMLIN) {
         chain_vec16(ldsV, st.vec0 + spans * 64 + f0, sc.cal);
         chain_vec16(ldsV, st.vec0 + 2 * spans * 64 + f0, sc.ecal);
     } else {  // EPI_KIND_FAST: absent vectors were filled with their neutral values by the host
@@ -111,7 +111,7 @@ __device__ __forceinline__ void chain_scales(const ChainStage& st, const int32_t
 template <int EPI>
 constexpr bool chain_reads_residual()
 {
-    return EPI == EPI_KIND_FUSED || EPI == EPI_KIND_FAST;
+    return EPI == EPI_KIND_FUSED || EPI == EPI_KIND_FAST || EPI == EPI_KIND_SUMLIN;
 }
 
 // SP0 / SP1 / SP2: 64-feature spans of the three stages (SP2 == 0: two stages).  D: activation look-ahead of stage 0.

@@ -84,7 +84,11 @@ struct MfmaArgs {
 //   LINEAR clamp(acc * cal, lo, hi)                                   (no activation, unit wqf)
 //   CLAMPQ clamp(acc * wqf, m, n) * cal, rounded                      (folded clamp{m, n} with 0 <= m, e.g. ReLU6 on the
 //                                                                      dequantised value; unit input factor; chain kernels)
-enum { EPI_KIND_GENERIC = 0, EPI_KIND_FAST = 1, EPI_KIND_RELU = 2, EPI_KIND_FUSED = 3, EPI_KIND_LINEAR = 4, EPI_KIND_CLAMPQ = 5 };
+//   SUMLIN clamp((sat(round(acc * cal)) + residual) * ecal, lo, hi)    (residual sum without activation, the rounded
+//                                                                      convolution result optionally saturated first, unit
+//                                                                      wqf; a MobileNet projection; chain kernels)
+enum { EPI_KIND_GENERIC = 0, EPI_KIND_FAST = 1, EPI_KIND_RELU = 2, EPI_KIND_FUSED = 3, EPI_KIND_LINEAR = 4, EPI_KIND_CLAMPQ = 5,
+       EPI_KIND_SUMLIN = 6 };
 template <int EPI> struct epi_is_short { static constexpr bool value = EPI != EPI_KIND_GENERIC; };
 
 // Workgroup barrier that orders LDS traffic only.  __syncthreads() also drains every outstanding
@@ -201,6 +205,33 @@ __device__ __forceinline__ v4i epilogue_fast16(const Args& a, const v4i (&acc)[4
 #pragma unroll
         for (int c = 0; c < 16; ++c) {
             const float y = med3(v[c] * cal[c], F.lo, F.hi);
+            v[c] = y + copysignf(0.49999997f, y);
+        }
+#pragma unroll
+        for (int d = 0; d < 4; ++d) packed[d] = pack_signed(v + d * 4);
+        if (valid < 16) {
+#pragma unroll
+            for (int d = 0; d < 4; ++d) {
+                unsigned keep = 0;
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                    if (d * 4 + i < valid) keep |= 255u << (8 * i);
+                packed[d] &= (int)keep;
+            }
+        }
+        return packed;
+    }
+    if constexpr (EPI == EPI_KIND_SUMLIN) {
+        // the run-time form's steps for a sum without activation, in the same order; ecal[] holds ones where the sum has
+        // no calibration factors
+        v4i packed;
+#pragma unroll
+        for (int c = 0; c < 16; ++c) {
+            float r = rha(v[c] * cal[c]);
+            if (F.conv_sat) r = med3(r, F.conv_lo, F.conv_hi);
+            const unsigned word = (unsigned)ev4[c >> 2];
+            const float e = F.eltw_u8 ? (float)((word >> (8 * (c & 3))) & 255u) : (float)(int)(int8_t)(word >> (8 * (c & 3)));
+            const float y = med3((r + e) * ecal[c], F.lo, F.hi);
             v[c] = y + copysignf(0.49999997f, y);
         }
 #pragma unroll

@@ -155,7 +155,7 @@ static void submit(cldnn_network_impl* net, cldnn_event* deps, size_t ndeps, cld
             HOST_REQUIRE(it != net->mem.end() && it->second, CLDNN_ERROR, "no memory for primitive " + d->p->id);
             return it->second.get();
         };
-        cldnn_memory_impl* out = mem_of(n);
+        cldnn_memory_impl* out = n->chain_unkept() ? nullptr : mem_of(n);
         // a primitive on the second stream starts when everything issued before it on the first has finished (its
         // inputs, and whatever used its output buffer before); its user waits for it
         cldnn_hip_engine where = eng->h;
@@ -221,7 +221,19 @@ static void submit(cldnn_network_impl* net, cldnn_event* deps, size_t ndeps, cld
         }
         case prim_type::convolution:
         case prim_type::fused_conv_eltwise: {
+            if (n->chain_head) break;  // written by the launch of its chain's head
             cldnn_memory_impl* in = mem_of(n->deps[0]);
+            if (n->chain) {
+                void* outs[3] = {nullptr, nullptr, nullptr};
+                const void* eltws[3] = {nullptr, nullptr, nullptr};
+                for (size_t k = 0; k < n->chain_members.size(); ++k) {
+                    node* m = n->chain_members[k];
+                    if (n->chain_keep[k]) outs[k] = mem_of(m)->device_ptr();
+                    if (m->p->type == prim_type::fused_conv_eltwise) eltws[k] = mem_of(m->deps[1])->device_ptr();
+                }
+                hip_check(cldnn_hip_conv_chain_enqueue(n->chain, in->device_ptr(), outs, eltws));
+                break;
+            }
             const void* eltw = nullptr;
             if (p.type == prim_type::fused_conv_eltwise && !p.second_input_in_output) eltw = mem_of(n->deps[1])->device_ptr();
             hip_check(cldnn_hip_conv_enqueue(n->conv, in->device_ptr(), out->device_ptr(), eltw));
@@ -364,8 +376,10 @@ cldnn_network_impl::~cldnn_network_impl()
 }
 cldnn_program_impl::~cldnn_program_impl()
 {
-    for (auto& n : nodes)
+    for (auto& n : nodes) {
         if (n->conv) cldnn_hip_conv_release(n->conv);
+        if (n->chain) cldnn_hip_conv_chain_release(n->chain);
+    }
 }
 
 struct cldnn_primitive_type {
@@ -798,6 +812,14 @@ cldnn_network cldnn_allocate_network(cldnn_program program, cldnn_status* status
         for (auto& u : program->nodes)
             if (u->side_stream)
                 for (node* d : u->deps) last_use[d] = std::max(last_use[d], index[u->users.at(0)]);
+        // a convolution chain reads and writes everything its members touch in the ONE launch at its head: whatever a
+        // member reads stays reserved until the last member, so that no member's output can take that buffer over
+        for (auto& u : program->nodes) {
+            if (u->chain_members.empty()) continue;
+            const size_t tail = index[u->chain_members.back()];
+            for (node* m : u->chain_members)
+                for (node* d : m->deps) last_use[d] = std::max(last_use[d], tail);
+        }
         const bool pool = e->memory_pool && !aliasing;
         std::vector<std::pair<size_t, ref<cldnn_memory_impl>>> in_flight;  // (index of the last consumer, buffer)
         std::vector<ref<cldnn_memory_impl>> idle;
@@ -818,6 +840,7 @@ cldnn_network cldnn_allocate_network(cldnn_program program, cldnn_status* status
                     if (f.second.get() == net->mem[n].get() && last_use.count(n)) f.first = std::max(f.first, last_use[n]);
                 continue;
             }
+            if (n->chain_unkept()) continue;  // never written: the next member of the chain takes it in registers
             // buffers whose tensors nobody reads at or after this primitive become idle
             for (auto it = in_flight.begin(); it != in_flight.end();) {
                 if (it->first < i) {

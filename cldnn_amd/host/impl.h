@@ -177,6 +177,21 @@ struct node {
     // compiled convolution
     cldnn_hip_conv conv = nullptr;
     cldnn_hip_conv_info conv_info{};
+    // convolution chain: the head holds the chain object and its members (itself first); a follower points at its
+    // head and is not launched on its own.  Members are consecutive in the execution order.
+    cldnn_hip_conv_chain chain = nullptr;
+    std::vector<node*> chain_members;
+    std::vector<int32_t> chain_keep;
+    node* chain_head = nullptr;
+    // member of a chain whose result stays in registers: it has no buffer and nobody but the next member reads it
+    bool chain_unkept() const
+    {
+        const node* head = chain ? this : chain_head;
+        if (!head) return false;
+        for (size_t k = 0; k < head->chain_members.size(); ++k)
+            if (head->chain_members[k] == this) return head->chain_keep[k] == 0;
+        return false;
+    }
     ref<cldnn_memory_impl> eltw_calib_dev;  // device copy of eltwise calibration (stand-alone eltwise)
 };
 

@@ -767,8 +767,22 @@ cldnn_hip_pooling_desc pooling_descriptor(const node* n)
 }
 
 // convolution / fused_conv_eltwise -> one cldnn_hip_conv object (reference convolution_gpu.cpp:71-162)
-static void compile_conv(cldnn_program_impl* prog, node* n)
+// descriptor and host copies of the constants of one convolution node
+struct conv_build {
+    cldnn_hip_conv_desc d{};
+    std::vector<uint8_t> wv, bv, qv, cv, ev;
+    const void* weights() const { return wv.data(); }
+    const void* bias() const { return bv.empty() ? nullptr : bv.data(); }
+    const float* wqf() const { return qv.empty() ? nullptr : (const float*)qv.data(); }
+    const float* calib() const { return cv.empty() ? nullptr : (const float*)cv.data(); }
+    const float* eltw_calib() const { return ev.empty() ? nullptr : (const float*)ev.data(); }
+};
+
+static void prepare_conv(cldnn_program_impl* prog, node* n, conv_build& cb)
 {
+    (void)prog;
+    cldnn_hip_conv_desc& d = cb.d;
+    std::vector<uint8_t>&wv = cb.wv, &bv = cb.bv, &qv = cb.qv, &cv = cb.cv, &ev = cb.ev;
     prim& p = *n->p;
     const bool fused = p.type == prim_type::fused_conv_eltwise;
     node* in = n->deps[0];
@@ -776,7 +790,6 @@ static void compile_conv(cldnn_program_impl* prog, node* n)
     conv_geom g = conv_geometry(p, in->out, w->out);
     const int ifm_g = g.IFM / g.groups;
 
-    cldnn_hip_conv_desc d{};
     d.input = to_hip(in->out);
     // a positive input offset: the same buffer, seen as the smaller tensor with what is left out counted as border
     d.input.y = g.IH, d.input.x = g.IW;
@@ -811,7 +824,7 @@ static void compile_conv(cldnn_program_impl* prog, node* n)
         return all;
     };
     size_t wdt = w->out.data_type, bdt = cldnn_f32, fdt = cldnn_f32;
-    std::vector<uint8_t> wv = gather(p.weights, wcount, "weights", &wdt), bv, qv, cv, ev;
+    wv = gather(p.weights, wcount, "weights", &wdt);
     for (const std::string& id : p.weights) {
         const cldnn_layout& wl = dep_named(n, id)->out;
         HOST_REQUIRE(wl.format == cldnn_format_bfyx && wl.size.sizes[0] == w->out.size.sizes[0] && wl.size.sizes[1] == w->out.size.sizes[1]
@@ -844,7 +857,6 @@ static void compile_conv(cldnn_program_impl* prog, node* n)
         d.activation = hip_act(n->fused_act);
         d.activation_m = n->fused_a, d.activation_n = n->fused_b;
     }
-    const void* eltw_calib = nullptr;
     if (fused) {
         HOST_REQUIRE(p.eltw_mode == cldnn_eltwise_sum, CLDNN_INVALID_ARG, "fused_conv_eltwise supports the sum mode only");
         d.fused = 1;
@@ -862,13 +874,21 @@ static void compile_conv(cldnn_program_impl* prog, node* n)
             node* c = dep_named(n, p.eltw_calib);
             ev = read_constant(c, g.OFM, "eltwise output_calibration_factors");
             d.has_eltw_calib = 1;
-            eltw_calib = ev.data();
         }
     }
     d.impl = CLDNN_HIP_IMPL_AUTO;
-    const void* bias_ptr = bv.empty() ? nullptr : bv.data();
-    const float* wqf_ptr = qv.empty() ? nullptr : (const float*)qv.data();
-    const float* calib_ptr = cv.empty() ? nullptr : (const float*)cv.data();
+}
+
+static void compile_conv(cldnn_program_impl* prog, node* n)
+{
+    conv_build cb;
+    prepare_conv(prog, n, cb);
+    cldnn_hip_conv_desc& d = cb.d;
+    const void* bias_ptr = cb.bias();
+    const float* wqf_ptr = cb.wqf();
+    const float* calib_ptr = cb.calib();
+    const void* eltw_calib = cb.eltw_calib();
+    std::vector<uint8_t>& wv = cb.wv;
     if (prog->tuning.mode != cldnn_tuning_disabled) {
         // reference src/gpu/convolution_gpu.cpp:147-154, kernel_selector/core/kernel_selector.cpp GetAutoTuneBestKernel: take
         // the cached choice; in tune_and_cache mode measure what the cache does not hold and add it
@@ -889,10 +909,109 @@ static void compile_conv(cldnn_program_impl* prog, node* n)
             ++prog->tuned_now;
         }
     }
-    hip_check(cldnn_hip_conv_create(n->side_stream ? prog->engine->side : prog->engine->h, &d, wv.data(), bv.empty() ? nullptr : bv.data(),
-                                    qv.empty() ? nullptr : (const float*)qv.data(), cv.empty() ? nullptr : (const float*)cv.data(),
+    hip_check(cldnn_hip_conv_create(n->side_stream ? prog->engine->side : prog->engine->h, &d, wv.data(), bias_ptr, wqf_ptr, calib_ptr,
                                     (const float*)eltw_calib, &n->conv));
     hip_check(cldnn_hip_conv_get_info(n->conv, &n->conv_info));
+}
+
+// ------------------------------------------------------------------------------------------ convolution chains
+// A convolution and the one or two 1x1 / stride-1 / unpadded convolutions that read its result run as ONE launch
+// (cldnn_hip_conv_chain): the tail of a ResNet bottleneck (3x3 -> 1x1 + sum -> the next block's 1x1) or of a MobileNet
+// block (depthwise 3x3 -> 1x1 -> the next block's 1x1).  The reference launches every node
+// (src/gpu/primitive_gpu_base.h:117-168); results are the same bits.  A follower moves up in the execution order to
+// sit right behind its predecessor, which is allowed when everything else it reads (the residual operand) is produced
+// before the head; results that other nodes read, or that are outputs, are written (keep), the rest never leaves
+// the registers.  Whether the kernels can run the group as a chain is decided by cldnn_hip_conv_chain_create (feature
+// counts, weights that fit into LDS ...); what it refuses runs node by node.
+static bool chain_follower(cldnn_program_impl* prog, node* prev, node* c, size_t head_pos)
+{
+    const prim& p = *c->p;
+    if (p.type != prim_type::convolution && p.type != prim_type::fused_conv_eltwise) return false;
+    if (p.fully_connected || p.second_input_in_output || c->side_stream || c->first_layer || c->deps[0] != prev) return false;
+    node* w = dep_named(c, p.weights.at(0));
+    const conv_geom g = conv_geometry(p, prev->out, w->out);
+    if (g.FY != 1 || g.FX != 1 || g.sy != 1 || g.sx != 1 || g.py != 0 || g.px != 0 || g.groups != 1) return false;
+    for (size_t i = 1; i < c->deps.size(); ++i)  // the residual operand has to exist when the head starts
+        if (!c->deps[i]->constant && position(prog, c->deps[i]) >= head_pos) return false;
+    return true;
+}
+
+static void group_chains(cldnn_program_impl* prog)
+{
+    for (size_t i = 0; i < prog->nodes.size(); ++i) {
+        node* head = prog->nodes[i].get();
+        const prim& hp = *head->p;
+        if (head->chain_head || (hp.type != prim_type::convolution && hp.type != prim_type::fused_conv_eltwise)) continue;
+        if (hp.fully_connected || hp.second_input_in_output || head->side_stream || head->first_layer) continue;
+        if (head->out.format != cldnn_format_fs_b_yx_fsv16 || head->deps[0]->out.format != cldnn_format_fs_b_yx_fsv16) continue;
+        std::vector<node*> members{head};
+        while (members.size() < 3) {
+            node* prev = members.back();
+            node* next = nullptr;
+            for (node* u : prev->users)
+                if (!u->chain_head && chain_follower(prog, prev, u, i)) {
+                    next = u;
+                    break;
+                }
+            if (!next) break;
+            members.push_back(next);
+        }
+        if (members.size() < 2) continue;
+        // followers move up behind the head
+        for (size_t k = 1; k < members.size(); ++k) {
+            const size_t from = position(prog, members[k]);
+            std::unique_ptr<node> moved = std::move(prog->nodes[from]);
+            prog->nodes.erase(prog->nodes.begin() + from);
+            prog->nodes.insert(prog->nodes.begin() + i + k, std::move(moved));
+            members[k]->chain_head = head;
+        }
+        head->chain_members = members;
+        for (size_t k = 0; k < members.size(); ++k) {
+            bool keep = members[k]->is_output || k + 1 == members.size();
+            for (node* u : members[k]->users) keep = keep || k + 1 >= members.size() || u != members[k + 1];
+            head->chain_keep.push_back(keep ? 1 : 0);
+        }
+    }
+}
+
+// Create the chain of a head node; members the kernels refuse as a chain are compiled one by one (a group of three is
+// tried as its first two members as well).
+static void compile_chain(cldnn_program_impl* prog, node* head)
+{
+    std::vector<node*> members = head->chain_members;
+    std::vector<conv_build> cb(members.size());
+    for (size_t k = 0; k < members.size(); ++k) prepare_conv(prog, members[k], cb[k]);
+    for (size_t count = members.size(); count >= 2 && !head->chain; --count) {
+        std::vector<cldnn_hip_conv_desc> descs;
+        std::vector<const void*> w, b;
+        std::vector<const float*> q, c, e;
+        std::vector<int32_t> keep(head->chain_keep.begin(), head->chain_keep.begin() + count);
+        keep[count - 1] = 1;
+        for (size_t k = 0; k < count; ++k) {
+            descs.push_back(cb[k].d);
+            w.push_back(cb[k].weights()), b.push_back(cb[k].bias()), q.push_back(cb[k].wqf()), c.push_back(cb[k].calib());
+            e.push_back(cb[k].eltw_calib());
+        }
+        const cldnn_hip_status st = cldnn_hip_conv_chain_create(prog->engine->h, (int32_t)count, descs.data(), w.data(), b.data(), q.data(),
+                                                                c.data(), e.data(), keep.data(), &head->chain);
+        if (st == CLDNN_HIP_SUCCESS) {
+            head->chain_keep = keep;
+            for (size_t k = count; k < members.size(); ++k) members[k]->chain_head = nullptr;
+            members.resize(count);
+            head->chain_members = members;
+            hip_check(cldnn_hip_conv_chain_get_info(head->chain, &head->conv_info));
+            for (size_t k = 1; k < count; ++k) {
+                members[k]->conv_info = cldnn_hip_conv_info{};
+                std::snprintf(members[k]->conv_info.kernel_name, sizeof(members[k]->conv_info.kernel_name), "in the chain of %s",
+                              head->p->id.substr(0, 40).c_str());
+            }
+            return;
+        }
+        if (st != CLDNN_HIP_UNSUPPORTED_FORMAT) hip_check(st);
+    }
+    for (node* m : members) m->chain_head = nullptr;
+    head->chain_members.clear();
+    head->chain_keep.clear();
 }
 
 // enable_parallelisation (reference api/C/cldnn.h:152, "parallel execution of primitives which don't depend on each
@@ -1008,9 +1127,16 @@ void build_program(cldnn_program_impl* prog, cldnn_topology_impl* topo, const st
     if (prog->optimize_data && prog->engine && !prog->engine->memory_pool) conv_eltw_read_write_opt(prog);
     if (!prog->engine) return;  // planning only: the graph is inspected, nothing is compiled
     if (prog->engine->side) assign_streams(prog);
+    // chains with the graph optimisations only; a tuned program keeps one launch per node (its cache is per node)
+    if (prog->optimize_data && prog->tuning.mode == cldnn_tuning_disabled) group_chains(prog);
     for (auto& u : prog->nodes) {
         node* n = u.get();
-        if (n->p->type == prim_type::convolution || n->p->type == prim_type::fused_conv_eltwise) compile_conv(prog, n);
+        if (!n->chain_members.empty()) compile_chain(prog, n);
+    }
+    for (auto& u : prog->nodes) {
+        node* n = u.get();
+        const bool conv = n->p->type == prim_type::convolution || n->p->type == prim_type::fused_conv_eltwise;
+        if (conv && !n->chain && !n->chain_head) compile_conv(prog, n);
     }
     prog->tuning.save();
 }
@@ -1049,7 +1175,7 @@ std::string describe_node(const node* n)
         s += "]";
     }
     if (n->side_stream) s += ",\"stream\":1";
-    if (n->conv)
+    if (n->conv || n->chain || n->chain_head)
         s += std::string(",\"kernel\":\"") + n->conv_info.kernel_name + "\",\"grid\":" + std::to_string(n->conv_info.grid)
              + ",\"ops\":" + std::to_string(n->conv_info.ops) + ",\"bytes\":" + std::to_string(n->conv_info.bytes);
     return s + "}";

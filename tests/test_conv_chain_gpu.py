@@ -209,3 +209,56 @@ def test_depthwise_chain_matches_the_oracle(eng, mid, proj, stride, stages, in_d
     xin.close()
     for b in bufs:
         b.close()
+
+
+@pytest.mark.parametrize("saturate,eltw_dt", [(0, np.int8), (1, np.int8), (0, np.uint8)], ids=["sum", "sum_saturated", "sum_u8"])
+def test_depthwise_chain_with_the_blocks_sum_on_the_projection(eng, saturate, eltw_dt):
+    """MobileNet block with a shortcut: depthwise 3x3 -> 1x1 projection + residual sum (no activation; with the
+    convolution's own int8 saturation kept or not) -> next expansion; the projection's compile-time form of the sum"""
+    r = np.random.default_rng(57)
+    B, H, W, mid, proj = 2, 14, 9, 192, 32
+    x = r.integers(0, 256, (B, mid, H, W)).astype(np.uint8)
+    xin = hip.upload(eng, x, "fs_b_yx_fsv16", (1, 1))
+    lo, hi = (0, 256) if eltw_dt == np.uint8 else (-128, 128)
+    e = r.integers(lo, hi, (B, proj, H, W)).astype(eltw_dt)
+    ecal = r.uniform(0.5, 1.0, proj).astype(np.float32)
+    ebuf = hip.upload(eng, e, "fs_b_yx_fsv16")
+    shapes = [(mid, 1, 3, "relu6", mid), (proj, mid, 1, "none", 1), (6 * proj, proj, 1, "relu6", 1)]
+    spec, refs, bufs = [], [], []
+    prev_t, ref_in = xin.tensor, x
+    for k, (ofm, ifm_g, fk, act, groups) in enumerate(shapes):
+        w, bias, wqf, calib, akw = relu6_layer(r, ofm, ifm_g, fk, act)
+        kw = dict(stride=(1, 1), pad=(fk // 2,) * 2, groups=groups, bias_dt=hip.I32, has_wqf=True, has_calib=True, **akw)
+        okw = dict(stride=(1, 1), pad=(fk // 2,) * 2, groups=groups, out_dt="s8", **akw)
+        if k == 1:
+            kw.update(eltw_t=ebuf.tensor, eltw_act="none", has_eltw_calib=True, conv_saturate=saturate)
+            okw.update(eltw=e, eltw_act="none", eltw_calib=ecal)
+        d = hip.conv_desc(prev_t, w.shape, "s8", **kw)
+        spec.append((d, w, bias, wqf, calib, ecal if k == 1 else None))
+        bufs.append(hip.Buffer(eng, d.output))
+        if k == 1:
+            calib = calib * 3  # a share of the convolution results beyond +-127
+            spec[-1] = (d, w, bias, wqf, calib, ecal)
+        if k == 1 and saturate:
+            # the kept saturation equals a convolution writing s8 followed by the stand-alone quantized sum
+            plain = {key: val for key, val in okw.items() if not key.startswith("eltw")}
+            refs.append(rc.eltwise([e, rc.conv(ref_in, w, bias, wqf=wqf, calib=calib, **plain)], "sum", calib=ecal))
+        else:
+            refs.append(rc.conv(ref_in, w, bias, wqf=wqf, calib=calib, **okw))
+        ref_in, prev_t = refs[-1], hip.Tensor.make(hip.S8, hip.FS_B_YX_FSV16, B, ofm, H, W)
+    ch = hip.ConvChain(eng, spec, [False, True, True])
+    assert b"conv_dwchain" in ch.info().kernel_name
+    ch.enqueue(xin, [None, bufs[1], bufs[2]], [None, ebuf, None])
+    eng.finish()
+    for k in (1, 2):
+        got = hip.download(eng, bufs[k])
+        bad = np.argwhere(got != refs[k])
+        assert bad.size == 0, "stage %d: %d of %d differ, first at %s" % (k, len(bad), got.size, bad[0])
+    if saturate:  # the data does reach the saturation
+        unsat = rc.conv(refs[0], spec[1][1], spec[1][2], wqf=spec[1][3], calib=spec[1][4], out_dt="s8", act="none", eltw=e, eltw_act="none",
+                        eltw_calib=ecal)
+        assert (unsat != refs[1]).any()
+    ch.close()
+    xin.close(), ebuf.close()
+    for b in bufs:
+        b.close()

@@ -134,6 +134,13 @@ def test_memory_pool_shares_buffers_without_changing_results():
         in_place = sorted(i.split("_fused_")[1] for i in net.get_all_primitive_ids()
                           if "_fused_" in i and net.get_primitive_info(i).get("second_input_in_output"))
         assert in_place == ([] if pool else sorted(b for b in BLOCKS if b not in ("res2c", "res3d", "res4f"))), in_place
+        # convolution chains: the 3x3, the closer with its sum and the next block's opener of stage 2 are one launch
+        # (not where the closer writes over its shortcut, i.e. not without a pool)
+        kernels = {i: net.get_primitive_info(i).get("kernel", "") for i in net.get_all_primitive_ids()}
+        followers = sorted(i for i, k in kernels.items() if k.startswith("in the chain of"))
+        if pool:
+            assert followers == ["res2a_branch2c_fused_res2a", "res2b_branch2a", "res2b_branch2c_fused_res2b", "res2c_branch2a"], followers
+            assert kernels["res2a_branch2b"].startswith("conv_chain<3 stages") and kernels["res2b_branch2a"] == "in the chain of res2a_branch2b"
         net.set_input_data("input", cl.make_memory(eng, x))
         for _ in range(2):  # a second run reuses the same buffers
             logits[pool] = net.execute()["fc1000"].get_memory().read()
@@ -141,8 +148,12 @@ def test_memory_pool_shares_buffers_without_changing_results():
         del net
     np.testing.assert_array_equal(logits[True], logits[False])
     np.testing.assert_array_equal(logits[True], run_oracle(x, params, fused=BLOCKS)["fc1000"])
-    # 26 MB of either figure are weights; without a pool the 13 closers that write over their shortcuts save nearly as much
-    assert used[True] < used[False] < 40e6, used
+    # 26 MB of either figure are weights; without a pool the 13 closers that write over their shortcuts save nearly as
+    # much as the pool does.  With the pool the two convolution chains of stage 2 (pooled engines only: a closer that
+    # writes over its shortcut is not chained) cost one 64-feature tensor each, because a chain's last member is written
+    # by the launch that still reads the head's input and cannot take that buffer over: at this batch the two figures
+    # meet within a percent
+    assert max(used.values()) < 40e6 and used[True] < 1.01 * used[False], used
 
 
 @pytest.mark.gpu

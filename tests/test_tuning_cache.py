@@ -99,7 +99,13 @@ def test_tune_and_cache_then_use_cache(tmp_path):
     assert used_kernels == tuned_kernels
     # the file decides: name another row for the second convolution and it runs on that row; a stale name is ignored
     key_b = [k for k in entries if "256x64x1x1" in k][0]
-    default_kernel = run(plain_eng, cl.build_options(optimize_data=True))[1]["b_fsv16"]
+    # the table's own choice: a program with a tuning cache keeps one launch per node (the cache is per node), an untuned
+    # one runs these two convolutions as a chain
+    empty = str(tmp_path / "empty.json")
+    json.dump({}, open(empty, "w"))
+    default_kernel = run(plain_eng, cl.build_options(optimize_data=True, tuning_config=(cl.tuning_mode.tuning_use_cache, empty)))[1]["b_fsv16"]
+    assert run(plain_eng, cl.build_options(optimize_data=True))[1] == {"a": run(plain_eng, cl.build_options(optimize_data=True))[1]["a"],
+                                                                        "b_fsv16": "in the chain of a"}
     forced = None
     for row in range(tile_config_count()):
         entries[key_b] = [tile_config_name(row), row]
