@@ -253,6 +253,7 @@ SIGNATURES = {
     "cldnn_convolution_type_id": (C.c_void_p, [_ST]),
     "cldnn_fused_conv_eltwise_type_id": (C.c_void_p, [_ST]),
     "cldnn_pooling_type_id": (C.c_void_p, [_ST]),
+    "cldnn_concatenation_type_id": (C.c_void_p, [_ST]),
     "cldnn_fully_connected_type_id": (C.c_void_p, [_ST]),
 }
 
@@ -539,6 +540,24 @@ class activation(_primitive):  # noqa: N801
         d.activation_func = func
         d.additional_params = c_act_params(*params)
         d.additional_params_input = b""
+
+
+class concatenation_axis:  # noqa: N801
+    along_b, along_f, along_x, along_y = 0, 1, 2, 3
+
+
+class c_concatenation_desc(C.Structure):
+    _fields_ = _BASE + [("axis", C.c_int32)]
+
+
+class concatenation(_primitive):  # noqa: N801
+    """concatenation(id, inputs, axis) (reference api/CPP/concatenation.hpp:54-92)."""
+    type_fn = "cldnn_concatenation_type_id"
+
+    def __init__(self, prim_id, inputs, axis, output_padding=None):
+        d = c_concatenation_desc()
+        self._base(d, prim_id, list(inputs), output_padding)
+        d.axis = axis
 
 
 class pooling(_primitive):  # noqa: N801

@@ -650,6 +650,16 @@ cldnn_hip_status cldnn_hip_reorder(cldnn_hip_engine e, const void* src_dev, cons
     });
 }
 
+cldnn_hip_status cldnn_hip_copy_region(cldnn_hip_engine e, const void* src_dev, const cldnn_hip_tensor* src, void* dst_dev,
+                                       const cldnn_hip_tensor* dst, int32_t offset_b, int32_t offset_f, int32_t offset_y, int32_t offset_x)
+{
+    return guarded([&] {
+        CHIP_REQUIRE(e && src_dev && src && dst_dev && dst, CLDNN_HIP_INVALID_ARG, "null argument");
+        e->make_current();
+        launch_copy_region(e->stream, *src, src_dev, *dst, dst_dev, offset_b, offset_f, offset_y, offset_x);
+    });
+}
+
 cldnn_hip_status cldnn_hip_activation(cldnn_hip_engine e, const void* src_dev, const cldnn_hip_tensor* src, void* dst_dev,
                                       const cldnn_hip_tensor* dst, int32_t activation, float m, float n)
 {

@@ -19,6 +19,9 @@ void launch_conv_ref(hipStream_t s, const ConvProblem& p, const Epilogue& epi, c
 void launch_eltwise(hipStream_t s, const cldnn_hip_eltwise_desc& d, const void* const* inputs, const float* calib, void* dst);
 void launch_pooling(hipStream_t s, const cldnn_hip_pooling_desc& d, const void* in, void* out);
 void launch_reorder(hipStream_t s, const cldnn_hip_tensor& st, const void* src, const cldnn_hip_tensor& dt, void* dst);
+// src copied into dst with its element (0, 0, 0, 0) at (ob, of, oy, ox): one input of a concatenation
+void launch_copy_region(hipStream_t s, const cldnn_hip_tensor& st, const void* src, const cldnn_hip_tensor& dt, void* dst, int ob, int of,
+                        int oy, int ox);
 // dst = act(a [+ b]); quantized: round((a + b) * (calib[f] or oqf)) saturated to char before the activation
 void launch_pointwise(hipStream_t s, const cldnn_hip_tensor& at, const void* a, const cldnn_hip_tensor* bt, const void* b,
                       const cldnn_hip_tensor& dt, void* dst, int quantized, const float* calib, float oqf, int act, float m,

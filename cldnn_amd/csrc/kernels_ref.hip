@@ -225,6 +225,62 @@ __global__ void __launch_bounds__(256) reorder_kernel(ReorderArgs a, const void*
     }
 }
 
+// ------------------------------------------------------------------------------------------ concatenation
+// One input of a concatenation copied to its place in the output: one work-item per element, any two layouts of one
+// element type (reference kernel_selector/core/cl_kernels/concatenation_gpu_ref.cl:18-46, one kernel per input with
+// the offset along the concatenation axis as its argument).
+struct CopyRegionArgs {
+    Pitch src, dst;
+    int B, F, Y, X;      // logical size of the source
+    int ob, of, oy, ox;  // where its element (0, 0, 0, 0) lies in the destination
+    int wide;            // 4-byte elements
+};
+
+__global__ void __launch_bounds__(256) copy_region_kernel(CopyRegionArgs a, const void* __restrict__ src, void* __restrict__ dst)
+{
+    const int64_t total = (int64_t)a.B * a.F * a.Y * a.X;
+    const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= total) return;
+    int b, f, y, x;
+    if (a.dst.fsv > 1 || a.dst.pf == 1) {  // features innermost in the destination
+        f = (int)(idx % a.F);
+        int64_t r = idx / a.F;
+        x = (int)(r % a.X);
+        r /= a.X;
+        y = (int)(r % a.Y);
+        b = (int)(r / a.Y);
+    } else {
+        x = (int)(idx % a.X);
+        int64_t r = idx / a.X;
+        y = (int)(r % a.Y);
+        r /= a.Y;
+        f = (int)(r % a.F);
+        b = (int)(r / a.F);
+    }
+    const int64_t si = a.src.at(b, f, y, x), di = a.dst.at(b + a.ob, f + a.of, y + a.oy, x + a.ox);
+    if (a.wide) ((uint32_t*)dst)[di] = ((const uint32_t*)src)[si];
+    else ((uint8_t*)dst)[di] = ((const uint8_t*)src)[si];
+}
+
+void launch_copy_region(hipStream_t s, const cldnn_hip_tensor& st, const void* src, const cldnn_hip_tensor& dt, void* dst, int ob, int of,
+                        int oy, int ox)
+{
+    CHIP_REQUIRE(dtype_size(st.dtype) == dtype_size(dt.dtype), CLDNN_HIP_INVALID_ARG, "concatenation: element sizes differ");
+    CHIP_REQUIRE(ob >= 0 && of >= 0 && oy >= 0 && ox >= 0 && ob + st.b <= dt.b && of + st.f <= dt.f && oy + st.y <= dt.y && ox + st.x <= dt.x,
+                 CLDNN_HIP_DIMENSION_MISMATCH, "concatenation: the input does not fit into the output at this offset");
+    CopyRegionArgs a{};
+    a.src = make_pitch(st), a.dst = make_pitch(dt);
+    a.B = st.b, a.F = st.f, a.Y = st.y, a.X = st.x;
+    a.ob = ob, a.of = of, a.oy = oy, a.ox = ox;
+    a.wide = dtype_size(st.dtype) == 4;
+    const int64_t total = (int64_t)a.B * a.F * a.Y * a.X;
+    if (total == 0) return;
+    const int64_t blocks = (total + 255) / 256;
+    CHIP_REQUIRE(blocks < (1ll << 31), CLDNN_HIP_UNSUPPORTED_SIZE, "tensor too large for the copy grid");
+    hipLaunchKernelGGL(copy_region_kernel, dim3((unsigned)blocks), dim3(256), 0, s, a, src, dst);
+    CHIP_CHECK(hipGetLastError());
+}
+
 // ------------------------------------------------------------------------------------------ eltwise / activation
 // Stand-alone forms of what the convolution epilogue fuses (reference
 // kernel_selector/core/cl_kernels/generic_eltwise_ref.cl:311-328 for the sum, activation_ref.cl for the

@@ -149,6 +149,8 @@ SIGNATURES = {
     "cldnn_hip_tensor_bytes": (C.c_size_t, [C.POINTER(Tensor)]),
     "cldnn_hip_tensor_offset": (C.c_int64, [C.POINTER(Tensor), C.c_int32, C.c_int32, C.c_int32, C.c_int32]),
     "cldnn_hip_reorder": (C.c_int32, [C.c_void_p, C.c_void_p, C.POINTER(Tensor), C.c_void_p, C.POINTER(Tensor)]),
+    "cldnn_hip_copy_region": (C.c_int32, [C.c_void_p, C.c_void_p, C.POINTER(Tensor), C.c_void_p, C.POINTER(Tensor), C.c_int32, C.c_int32,
+                                          C.c_int32, C.c_int32]),
     "cldnn_hip_activation": (C.c_int32, [C.c_void_p, C.c_void_p, C.POINTER(Tensor), C.c_void_p, C.POINTER(Tensor),
                                          C.c_int32, C.c_float, C.c_float]),
     "cldnn_hip_eltwise_sum": (C.c_int32, [C.c_void_p, C.c_void_p, C.POINTER(Tensor), C.c_void_p, C.POINTER(Tensor),

@@ -180,6 +180,17 @@ static void submit(cldnn_network_impl* net, cldnn_event* deps, size_t ndeps, cld
             hip_check(cldnn_hip_reorder(eng->h, in->device_ptr(), &it, out->device_ptr(), &ot));
             break;
         }
+        case prim_type::concatenation: {
+            if (n->concat_in_place) break;  // its inputs wrote into this buffer themselves
+            // reference src/gpu/concatenation_gpu.cpp:64-90: one copy per input, at its offset along the axis
+            int at[4] = {0, 0, 0, 0};  // b, f, x, y
+            for (size_t i = 0; i < p.inputs.size(); ++i) {
+                const cldnn_hip_tensor it = to_hip(n->deps[i]->out);
+                hip_check(cldnn_hip_copy_region(eng->h, mem_of(n->deps[i])->device_ptr(), &it, out->device_ptr(), &ot, at[0], at[1], at[3], at[2]));
+                at[p.concat_axis] += n->deps[i]->out.size.sizes[p.concat_axis];
+            }
+            break;
+        }
         case prim_type::pooling: {
             cldnn_memory_impl* in = mem_of(n->deps[0]);
             cldnn_hip_pooling_desc pd = pooling_descriptor(n);
@@ -392,6 +403,7 @@ static const cldnn_primitive_type g_types[] = {
     {prim_type::fused_conv_eltwise, "fused_conv_eltwise"}, {prim_type::pooling, "pooling"},
     // kept as a convolution node whose filter covers the input plane
     {prim_type::convolution, "fully_connected"},
+    {prim_type::concatenation, "concatenation"},
 };
 
 extern "C" {
@@ -411,6 +423,7 @@ TYPE_ID_FN(convolution, 5)
 TYPE_ID_FN(fused_conv_eltwise, 6)
 TYPE_ID_FN(pooling, 7)
 TYPE_ID_FN(fully_connected, 8)
+TYPE_ID_FN(concatenation, 9)
 
 const char* cldnn_get_last_error_message() { return g_last_error.c_str(); }
 
@@ -470,6 +483,14 @@ void cldnn_add_primitive(cldnn_topology topology, const struct cldnn_primitive_d
             HOST_REQUIRE((!d->mean_subtract || !*d->mean_subtract) && d->subtract_per_feature.size == 0, CLDNN_INVALID_ARG,
                          "reorder with mean subtraction is not supported by this library");
             p->reorder_format = d->output_format;
+            break;
+        }
+        case prim_type::concatenation: {
+            auto* d = reinterpret_cast<const cldnn_concatenation_desc*>(dto);
+            HOST_REQUIRE(d->axis == cldnn_concatenation_along_b || d->axis == cldnn_concatenation_along_f || d->axis == cldnn_concatenation_along_x
+                             || d->axis == cldnn_concatenation_along_y,
+                         CLDNN_INVALID_ARG, "concatenation axis must be b, f, x or y (no five-dimensional tensors in this library)");
+            p->concat_axis = (int32_t)d->axis;
             break;
         }
         case prim_type::pooling: {
@@ -841,6 +862,24 @@ cldnn_network cldnn_allocate_network(cldnn_program program, cldnn_status* status
                 continue;
             }
             if (n->chain_unkept()) continue;  // never written: the next member of the chain takes it in registers
+            if (n->concat_in_place || n->concat_into) {
+                // an in-place concatenation owns one buffer of its own (outside the pool); its inputs, which come earlier
+                // in the order, are windows into it
+                node* c = n->concat_in_place ? n : n->concat_into;
+                if (!net->mem.count(c)) {
+                    net->mem[c] = allocate(e, c->out);
+                    net->allocated_bytes += layout_bytes(c->out);
+                }
+                if (n->concat_into) {
+                    ref<cldnn_memory_impl> w(new cldnn_memory_impl(), false);
+                    w->layout = n->out;
+                    w->engine = ref<cldnn_engine_impl>(e, true);
+                    w->view_of = net->mem[c];
+                    w->view_offset = n->concat_offset;
+                    net->mem[n] = w;
+                }
+                continue;
+            }
             // buffers whose tensors nobody reads at or after this primitive become idle
             for (auto it = in_flight.begin(); it != in_flight.end();) {
                 if (it->first < i) {

@@ -64,7 +64,7 @@ struct ref {  // owning smart pointer for refcounted objects
     explicit operator bool() const { return p != nullptr; }
 };
 
-enum class prim_type { input_layout, data, reorder, activation, eltwise, convolution, fused_conv_eltwise, pooling };
+enum class prim_type { input_layout, data, reorder, activation, eltwise, convolution, fused_conv_eltwise, pooling, concatenation };
 
 // which row of the tile-config table a convolution runs on, measured once and kept in a JSON file (tuning_cache.cpp)
 struct tuning_cache {
@@ -96,8 +96,14 @@ struct cldnn_memory_impl : host::refcounted {
     cldnn_hip_buffer buf = nullptr;
     void* attached = nullptr;
     size_t attached_bytes = 0;
+    host::ref<cldnn_memory_impl> view_of;  // a window into another memory's buffer (input of an in-place concatenation)
+    size_t view_offset = 0;
     ~cldnn_memory_impl() override;
-    void* device_ptr() const { return buf ? cldnn_hip_buffer_device_ptr(buf) : nullptr; }
+    void* device_ptr() const
+    {
+        if (view_of) return (char*)view_of->device_ptr() + view_offset;
+        return buf ? cldnn_hip_buffer_device_ptr(buf) : nullptr;
+    }
 };
 
 struct cldnn_event_impl : host::refcounted {
@@ -128,6 +134,8 @@ struct prim {
     int32_t pool_mode = cldnn_pooling_max;
     bool pool_global = false;
     cldnn_tensor pool_size{};
+    // concatenation: index into cldnn_tensor::sizes (0 batch, 1 feature, 2 x, 3 y)
+    int32_t concat_axis = 1;
     // eltwise / fused eltw part
     std::string eltw_calib;
     float eltw_oqf = 1.f;
@@ -183,6 +191,11 @@ struct node {
     std::vector<node*> chain_members;
     std::vector<int32_t> chain_keep;
     node* chain_head = nullptr;
+    // in-place concatenation (reference prepare_buffer_fusing.cpp:38-140): this node writes straight into the buffer of
+    // the concatenation `concat_into`, `concat_offset` bytes from its start; the concatenation itself then does nothing
+    node* concat_into = nullptr;
+    size_t concat_offset = 0;
+    bool concat_in_place = false;   // concatenation whose inputs all write into its buffer
     // member of a chain whose result stays in registers: it has no buffer and nobody but the next member reads it
     bool chain_unkept() const
     {

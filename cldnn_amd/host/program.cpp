@@ -251,6 +251,23 @@ static void calc_layout(node* n)
         n->out.size = make_tensor(in.size.sizes[0], in.size.sizes[1], g.OW, g.OH);
         break;
     }
+    case prim_type::concatenation: {
+        // reference src/concatenation.cpp:31-54 (layout) and :85-120 (every other axis must agree, one format)
+        HOST_REQUIRE(!p.out_dt.enabled, CLDNN_INVALID_ARG, "output data type forcing is not supported for concatenation");
+        HOST_REQUIRE(p.concat_axis >= 0 && p.concat_axis <= 3, CLDNN_INVALID_ARG, "concatenation axis must be b, f, x or y");
+        const cldnn_layout& first = n->deps[0]->out;
+        n->out = first;
+        n->out.size.sizes[p.concat_axis] = 0;
+        for (size_t k = 0; k < p.inputs.size(); ++k) {
+            const cldnn_layout& in = n->deps[k]->out;
+            for (int i = 0; i < 4; ++i)
+                HOST_REQUIRE(i == p.concat_axis || in.size.sizes[i] == first.size.sizes[i], CLDNN_DIMENSION_MISMATCH,
+                             "concatenation: every input must have the same size along the other axes");
+            HOST_REQUIRE(in.data_type == first.data_type, CLDNN_INVALID_ARG, "concatenation: the inputs differ in data type");
+            n->out.size.sizes[p.concat_axis] += in.size.sizes[p.concat_axis];
+        }
+        break;
+    }
     case prim_type::eltwise: {
         const size_t count = p.inputs.size();
         HOST_REQUIRE(count >= 2 && n->deps.size() >= count, CLDNN_INVALID_ARG, "eltwise needs two inputs");
@@ -741,6 +758,56 @@ static void prepare_borders(cldnn_program_impl* prog)
 }
 
 // ------------------------------------------------------------------------------------------ compile
+// prepare_buffer_fusing (reference src/graph_optimizer/prepare_buffer_fusing.cpp:38-140): the inputs of a concatenation
+// write straight into the concatenation's buffer and the concatenation itself does nothing.  The reference expresses an
+// input's place as output padding along the concatenation axis, which its kernels honour on every axis; the kernels
+// here take borders in y and x only, so the pass applies where an input's place is one CONTIGUOUS piece of the buffer
+// with the input's own layout: the concatenation axis is the outermost axis of the memory order that has more than one
+// element -- feature slices in fs_b_yx_fsv16 (every input but the last a multiple of 16 features), the batch in bfyx, the
+// features in bfyx at batch 1 -- and all tensors carry the same border.  As in the reference an input must not be an
+// output or user memory, and (stricter) belongs to one in-place concatenation only and is no concatenation itself.
+static void prepare_buffer_fusing(cldnn_program_impl* prog)
+{
+    for (auto& u : prog->nodes) {
+        node* c = u.get();
+        if (c->p->type != prim_type::concatenation) continue;
+        const int axis = c->p->concat_axis;
+        const cldnn_layout& out = c->out;
+        const int B = out.size.sizes[0];
+        bool outermost = false;
+        if (out.format == cldnn_format_fs_b_yx_fsv16) outermost = axis == 1;
+        else if (out.format == cldnn_format_bfyx) outermost = axis == 0 || (axis == 1 && B == 1);
+        if (!outermost) continue;
+        const size_t count = c->p->inputs.size();
+        // one border for the whole group: the widest any member needs
+        cldnn_padding pad = out.padding;
+        bool ok = true;
+        for (size_t k = 0; k < count && ok; ++k) {
+            node* in = c->deps[k];
+            ok = !in->constant && !in->is_output && in->p->type != prim_type::input_layout && in->p->type != prim_type::concatenation
+                 && !in->concat_into && in->out.format == out.format && !in->side_stream
+                 && !(in->p->type == prim_type::fused_conv_eltwise && in->p->second_input_in_output);
+            for (size_t j = 0; j < k && ok; ++j) ok = c->deps[j] != in;  // the same tensor twice needs two copies
+            if (ok && out.format == cldnn_format_fs_b_yx_fsv16 && k + 1 < count) ok = in->out.size.sizes[1] % 16 == 0;
+            for (int i = 0; i < 4 && ok; ++i) {
+                pad.lower_size.sizes[i] = std::max(pad.lower_size.sizes[i], in->out.padding.lower_size.sizes[i]);
+                pad.upper_size.sizes[i] = std::max(pad.upper_size.sizes[i], in->out.padding.upper_size.sizes[i]);
+            }
+        }
+        if (!ok) continue;
+        c->out.padding = pad;
+        size_t offset = 0;
+        for (size_t k = 0; k < count; ++k) {
+            node* in = c->deps[k];
+            in->out.padding = pad;
+            in->concat_into = c;
+            in->concat_offset = offset;
+            offset += layout_bytes(in->out);
+        }
+        c->concat_in_place = true;
+    }
+}
+
 static int hip_act(int32_t f)
 {
     switch (f) {
@@ -1057,9 +1124,9 @@ static void conv_eltw_read_write_opt(cldnn_program_impl* prog)
 {
     for (size_t i = 0; i < prog->nodes.size(); ++i) {
         node* n = prog->nodes[i].get();
-        if (n->p->type != prim_type::fused_conv_eltwise || n->p->second_input_in_output || n->is_output) continue;
+        if (n->p->type != prim_type::fused_conv_eltwise || n->p->second_input_in_output || n->is_output || n->concat_into) continue;
         node* r = n->deps[1];
-        if (r->constant || r->is_output || r->p->type == prim_type::input_layout) continue;
+        if (r->constant || r->is_output || r->p->type == prim_type::input_layout || r->concat_into || r->concat_in_place) continue;
         if (!layouts_equal(r->out, n->out)) continue;
         bool last_reader = true;
         for (node* u : r->users) last_reader = last_reader && (u == n || position(prog, u) < i);
@@ -1122,6 +1189,7 @@ void build_program(cldnn_program_impl* prog, cldnn_topology_impl* topo, const st
     }
     for (auto& u : prog->nodes) calc_layout(u.get());
     prepare_borders(prog);
+    if (prog->optimize_data) prepare_buffer_fusing(prog);
     // with the memory pool on, buffers are recycled anyway and the in-place form measures 1.7 % slower on ResNet-50
     // (same kernels; reads and writes of one launch then share their cache lines), so the pass serves engines without a pool
     if (prog->optimize_data && prog->engine && !prog->engine->memory_pool) conv_eltw_read_write_opt(prog);
@@ -1150,7 +1218,8 @@ static std::string four(const int32_t* s)
 // one node as JSON; sizes and paddings are [b, f, x, y] like cldnn_tensor::sizes
 std::string describe_node(const node* n)
 {
-    static const char* tn[] = {"input_layout", "data", "reorder", "activation", "eltwise", "convolution", "fused_conv_eltwise", "pooling"};
+    static const char* tn[] = {"input_layout", "data", "reorder", "activation", "eltwise", "convolution", "fused_conv_eltwise", "pooling",
+                               "concatenation"};
     const prim& p = *n->p;
     std::string s = "{\"id\":\"" + p.id + "\",\"type\":\"" + tn[(int)p.type] + "\",\"org_id\":\"" + n->org_id + "\",\"deps\":[";
     for (size_t i = 0; i < n->deps.size(); ++i) s += std::string(i ? "," : "") + "\"" + n->deps[i]->p->id + "\"";
@@ -1174,6 +1243,8 @@ std::string describe_node(const node* n)
         for (size_t i = 0; i < p.eltw_stride.size(); ++i) s += (i ? "," : "") + four(p.eltw_stride[i].sizes);
         s += "]";
     }
+    if (p.type == prim_type::concatenation) s += ",\"axis\":" + std::to_string(p.concat_axis) + ",\"in_place\":" + (n->concat_in_place ? "true" : "false");
+    if (n->concat_into) s += ",\"concat_into\":\"" + n->concat_into->p->id + "\",\"concat_offset\":" + std::to_string(n->concat_offset);
     if (n->side_stream) s += ",\"stream\":1";
     if (n->conv || n->chain || n->chain_head)
         s += std::string(",\"kernel\":\"") + n->conv_info.kernel_name + "\",\"grid\":" + std::to_string(n->conv_info.grid)

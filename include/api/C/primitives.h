@@ -1,7 +1,7 @@
 /*
  * Descriptor structures ("dto") of the primitives a convolution topology needs.  Field order and
  * meaning follow the reference headers: api/C/input_layout.h, data.h, reorder.h, activation.h,
- * eltwise.h, pooling.h, convolution.h:36-74 and api_extension/C/fused_conv_eltwise.h:35-97.
+ * eltwise.h, pooling.h, concatenation.h, convolution.h:36-74 and api_extension/C/fused_conv_eltwise.h:35-97.
  */
 #ifndef CLDNN_PRIMITIVES_H
 #define CLDNN_PRIMITIVES_H
@@ -56,6 +56,21 @@ uint32_t with_output_size;
 cldnn_tensor output_size;
 CLDNN_END_PRIMITIVE_DESC(pooling)
 CLDNN_DECLARE_PRIMITIVE_TYPE_ID(pooling);
+
+/* concatenation (reference api/C/concatenation.h:31-50): the inputs side by side along one axis; every other axis must
+ * agree.  along_z belongs to five-dimensional tensors, which this library does not have. */
+typedef enum {
+    cldnn_concatenation_along_b = 0,
+    cldnn_concatenation_along_f = CLDNN_TENSOR_BATCH_DIM_MAX,
+    cldnn_concatenation_along_x = CLDNN_TENSOR_BATCH_DIM_MAX + CLDNN_TENSOR_FEATURE_DIM_MAX,
+    cldnn_concatenation_along_y = cldnn_concatenation_along_x + 1,
+    cldnn_concatenation_along_z = cldnn_concatenation_along_y + 1
+} cldnn_concatenation_axis;
+
+CLDNN_BEGIN_PRIMITIVE_DESC(concatenation)
+cldnn_concatenation_axis axis;
+CLDNN_END_PRIMITIVE_DESC(concatenation)
+CLDNN_DECLARE_PRIMITIVE_TYPE_ID(concatenation);
 
 /* fully_connected (reference api/C/fully_connected.h:33-59): the convolution whose filter covers the whole input
  * plane; weights [ofm][ifm][y][x] in bfyx.  Quantized (weights_quantization_factors given) it has the epilogue of the

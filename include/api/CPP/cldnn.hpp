@@ -588,6 +588,31 @@ private:
     mutable id_list _in;
 };
 
+// concatenation(id, inputs, axis) (reference api/CPP/concatenation.hpp:54-92); along_z is not available
+struct concatenation : primitive {
+    enum concatenation_axis {
+        along_b = cldnn_concatenation_along_b,
+        along_f = cldnn_concatenation_along_f,
+        along_x = cldnn_concatenation_along_x,
+        along_y = cldnn_concatenation_along_y
+    };
+    concatenation_axis axis;
+    concatenation(const primitive_id& id, const std::vector<primitive_id>& input, const concatenation_axis axis,
+                  const padding& output_padding = padding())
+        : primitive(id, input, output_padding), axis(axis) {}
+    CLDNN_CPP_TYPE_ID(concatenation)
+    const ::cldnn_primitive_desc* get_dto() const override
+    {
+        fill_base(_d, type_id(), _in);
+        _d.axis = static_cast<cldnn_concatenation_axis>(axis);
+        return reinterpret_cast<const ::cldnn_primitive_desc*>(&_d);
+    }
+
+private:
+    mutable cldnn_concatenation_desc _d{};
+    mutable id_list _in;
+};
+
 // fully_connected(id, input, weights, bias, with_activation, slope) and the quantized forms with
 // w_quantization_factor [, output_calibration_factors], i_quantization_factor [, o_quantization_factor]
 // (reference api/CPP/fully_connected.hpp:60-150)

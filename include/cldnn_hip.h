@@ -163,6 +163,13 @@ cldnn_hip_status cldnn_hip_reorder(cldnn_hip_engine e, const void* src_dev, cons
 
 enum { CLDNN_HIP_ACT_NONE = 0, CLDNN_HIP_ACT_RELU = 1, CLDNN_HIP_ACT_RELU_SLOPE = 2, CLDNN_HIP_ACT_CLAMP = 3 };
 
+/* One input of a concatenation copied to its place in the output: the source's element (0, 0, 0, 0) lands at the given
+ * logical offset of the destination; any two layouts, same element size (reference
+ * kernel_selector/core/cl_kernels/concatenation_gpu_ref.cl:18-46 and src/gpu/concatenation_gpu.cpp:64-90: one kernel per
+ * input).  Asynchronous on the engine stream. */
+cldnn_hip_status cldnn_hip_copy_region(cldnn_hip_engine e, const void* src_dev, const cldnn_hip_tensor* src, void* dst_dev,
+                                       const cldnn_hip_tensor* dst, int32_t offset_b, int32_t offset_f, int32_t offset_y, int32_t offset_x);
+
 /* stand-alone activation and element-wise sum (what the convolution epilogue fuses when it can);
  * replace the reference's activation / eltwise kernels for the cases a convolution topology needs
  * (reference src/gpu/activation_gpu.cpp, src/gpu/eltwise_gpu.cpp,

@@ -533,3 +533,90 @@ def test_border_for_strided_window_covers_the_last_tap():
     OW = o["conv_fsv16"]["size"][2]
     last = (OW - 1) * 2 - 1 + 2  # leftmost tap of the last window + filter reach
     assert r["pad_lower"][2] == 1 and r["pad_upper"][2] == max(0, last - 8)
+
+
+# ------------------------------------------------------------------------------------------ concatenation
+def two_branch_topology(f1=32, f2=16, axis=cl.concatenation_axis.along_f, quantized=True, in_fmt=F.bfyx, batch=2, tail=True, out=None):
+    """in -> conv a (f1 features), conv b (f2 features) -> concatenation -> [1x1 conv]"""
+    Cn, H, W = 16, 6, 5
+    q = dict(w_quantization_factor=None, output_calibration_factors=None)
+    prims = [cl.input_layout("in", cl.layout(DT.i8, in_fmt, cl.tensor(batch, Cn, W, H)))]
+    for name, f in (("a", f1), ("b", f2)):
+        prims += [cl.data("w" + name, attach(np.ones((f, Cn, 3, 3), np.int8))), cl.data("q" + name, vec(f)), cl.data("c" + name, vec(f))]
+        q = dict(w_quantization_factor=["q" + name], output_calibration_factors=["c" + name]) if quantized else {}
+        prims.append(cl.convolution(name, "in", ["w" + name], input_offset=cl.tensor(0, 0, -1, -1, 0), with_activation=True, **q))
+    prims.append(cl.concatenation("cat", ["a", "b"], axis))
+    if tail:
+        n = f1 + f2 if axis == cl.concatenation_axis.along_f else f1
+        prims += [cl.data("wt", attach(np.ones((8, n, 1, 1), np.int8))), cl.data("qt", vec(8)), cl.data("ct", vec(8)),
+                  cl.convolution("tail", "cat", ["wt"], w_quantization_factor=["qt"], output_calibration_factors=["ct"])]
+    return cl.topology(*prims)
+
+
+@pytest.mark.parametrize("axis,sizes,want", [(cl.concatenation_axis.along_f, [(2, 3, 5, 4), (2, 7, 5, 4), (2, 1, 5, 4)], [2, 11, 5, 4]),
+                                             (cl.concatenation_axis.along_b, [(1, 3, 5, 4), (4, 3, 5, 4)], [5, 3, 5, 4]),
+                                             (cl.concatenation_axis.along_x, [(2, 3, 5, 4), (2, 3, 2, 4)], [2, 3, 7, 4]),
+                                             (cl.concatenation_axis.along_y, [(2, 3, 5, 4), (2, 3, 5, 9)], [2, 3, 5, 13])],
+                         ids=["f", "b", "x", "y"])
+def test_concatenation_layout(axis, sizes, want):
+    """reference src/concatenation.cpp:31-54: the sizes add up along the axis, format and type follow the first input"""
+    prims = [cl.input_layout("i%d" % k, cl.layout(DT.f32, F.bfyx, cl.tensor(*s))) for k, s in enumerate(sizes)]
+    prims.append(cl.concatenation("cat", ["i%d" % k for k in range(len(sizes))], axis))
+    n = by_id(cl.plan(cl.topology(*prims)))["cat"]
+    assert n["type"] == "concatenation" and n["size"] == want and n["format"] == F.bfyx and n["data_type"] == DT.f32
+    assert n["deps"] == ["i%d" % k for k in range(len(sizes))] and n["in_place"] is False
+
+
+def test_concatenation_inputs_must_agree():
+    a = cl.input_layout("a", cl.layout(DT.f32, F.bfyx, cl.tensor(2, 3, 5, 4)))
+    with pytest.raises(cl.error, match="same size along the other axes") as e:
+        cl.plan(cl.topology(a, cl.input_layout("b", cl.layout(DT.f32, F.bfyx, cl.tensor(2, 3, 6, 4))),
+                            cl.concatenation("cat", ["a", "b"], cl.concatenation_axis.along_f)))
+    assert e.value.status == cl.DIMENSION_MISMATCH
+    with pytest.raises(cl.error, match="differ in data type"):
+        cl.plan(cl.topology(a, cl.input_layout("b", cl.layout(DT.i8, F.bfyx, cl.tensor(2, 3, 5, 4))),
+                            cl.concatenation("cat", ["a", "b"], cl.concatenation_axis.along_f)))
+    with pytest.raises(cl.error, match="axis must be b, f, x or y"):
+        cl.plan(cl.topology(a, cl.concatenation("cat", ["a"], 4)))  # along_z: five-dimensional tensors only
+
+
+def test_concatenation_in_place_of_blocked_convolutions():
+    """reference prepare_buffer_fusing.cpp:38-140: the producers write into the concatenation's buffer.  Here that holds
+    where an input's place is one contiguous piece of the buffer: feature slices of fs_b_yx_fsv16"""
+    opt = by_id(cl.plan(two_branch_topology(), cl.build_options(optimize_data=True)))
+    cat, a, b = opt["cat"], opt["a"], opt["b"]
+    assert cat["format"] == F.fs_b_yx_fsv16 and cat["in_place"] is True and cat["size"] == [2, 48, 5, 6]
+    assert a["concat_into"] == "cat" and a["concat_offset"] == 0
+    # b starts behind a's two feature slices: 2 slices x batch 2 x 6 rows x 5 pixels x 16 bytes (no border: the tail is 1x1)
+    assert b["concat_into"] == "cat" and b["concat_offset"] == 2 * 2 * 6 * 5 * 16
+    # without the graph optimisations nothing is shared
+    plain = by_id(cl.plan(two_branch_topology()))
+    assert plain["cat"]["in_place"] is False and "concat_into" not in plain["a"]
+
+
+@pytest.mark.parametrize("kw,why", [(dict(f1=24), "24 features do not fill their last slice"),
+                                    (dict(axis=cl.concatenation_axis.along_x, f2=32), "x is not the outermost axis"),
+                                    (dict(quantized=False), "plain kernel, bfyx at batch 2: features are not outermost")],
+                         ids=["ragged_slice", "along_x", "bfyx_batch2"])
+def test_concatenation_not_in_place(kw, why):
+    opt = by_id(cl.plan(two_branch_topology(**kw), cl.build_options(optimize_data=True)))
+    assert opt["cat"]["in_place"] is False, why
+    assert "concat_into" not in opt["a"] and "concat_into" not in opt["b"]
+
+
+def test_concatenation_in_place_needs_private_intermediate_inputs():
+    # an input that is an output keeps its own buffer (reference :95-99)
+    t = two_branch_topology(in_fmt=F.fs_b_yx_fsv16)
+    opt = by_id(cl.plan(t, cl.build_options(optimize_data=True, outputs=["a", "tail"])))
+    assert opt["a"]["is_output"] and opt["cat"]["in_place"] is False
+    # ... unless the application sees a copy in its own format: then the blocked tensor behind it is an intermediate one
+    opt = by_id(cl.plan(two_branch_topology(), cl.build_options(optimize_data=True, outputs=["a", "tail"])))
+    assert opt["a"]["type"] == "reorder" and opt["a_fsv16"]["concat_into"] == "cat" and opt["cat"]["in_place"] is True
+    # bfyx at batch 1: the features are the outermost axis, so the plain path shares too; one border for the whole group
+    opt = by_id(cl.plan(two_branch_topology(quantized=False, batch=1), cl.build_options(optimize_data=True)))
+    assert opt["cat"]["in_place"] is True and opt["b"]["concat_offset"] == 32 * 6 * 5
+    assert opt["a"]["pad_lower"] == opt["b"]["pad_lower"] == opt["cat"]["pad_lower"]
+    # user memory is never a window into something else
+    prims = [cl.input_layout("i%d" % k, cl.layout(DT.i8, F.bfyx, cl.tensor(1, 16, 5, 4))) for k in range(2)]
+    prims.append(cl.concatenation("cat", ["i0", "i1"], cl.concatenation_axis.along_f))
+    assert by_id(cl.plan(cl.topology(*prims), cl.build_options(optimize_data=True)))["cat"]["in_place"] is False

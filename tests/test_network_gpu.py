@@ -6,6 +6,8 @@ tests/test_cases/fused_conv_eltwise_gpu_test.cpp:31-236, tests/test_cases/memory
 tests/test_cases/topology_test.cpp): build a topology from input_layout / data / convolution primitives,
 run a network, read the output memory.
 """
+import ctypes as C
+
 import numpy as np
 import pytest
 
@@ -675,3 +677,106 @@ def test_unsupported_requests_fail_loudly(eng):
     with pytest.raises(cl.error) as e:
         net.execute()
     assert "not supported" in str(e.value)
+
+
+# ------------------------------------------------------------------------------------------ concatenation
+def inception_like(eng, seed, B=2, C=32, H=9, W=7, f=(32, 48, 16)):
+    """three quantized branches (1x1, 3x3, 3x3) side by side along the features, a 3x3 convolution behind them: what an
+    inception block hands to the next one.  The 3x3 behind the concatenation needs a zero border, which the in-place
+    form has to give to every branch."""
+    r = np.random.default_rng(seed)
+    x = r.integers(0, 256, (B, C, H, W)).astype(np.uint8)
+    ks = (1, 3, 3)
+    L = [rand_layer(r, f[i], C, ks[i]) for i in range(3)] + [rand_layer(r, 24, sum(f), 3)]
+    prims = [cl.input_layout("input", cl.layout(DT.u8, F.bfyx, cl.tensor(B, C, W, H)))]
+    for i, (w, b, q, c) in enumerate(L):
+        prims += [cl.data(f"w{i}", cl.make_memory(eng, w)), cl.data(f"b{i}", vec_mem(eng, b)), cl.data(f"q{i}", vec_mem(eng, q)),
+                  cl.data(f"c{i}", vec_mem(eng, c))]
+    for i in range(3):
+        prims.append(cl.convolution(f"br{i}", "input", [f"w{i}"], [f"b{i}"], [f"q{i}"], [f"c{i}"], with_activation=True,
+                                    input_offset=cl.tensor(0, 0, -(ks[i] // 2), -(ks[i] // 2), 0), output_data_type=DT.u8))
+    prims += [cl.concatenation("cat", ["br0", "br1", "br2"], cl.concatenation_axis.along_f),
+              cl.convolution("next", "cat", ["w3"], ["b3"], ["q3"], ["c3"], with_activation=True, input_offset=cl.tensor(0, 0, -1, -1, 0),
+                             output_data_type=DT.u8)]
+
+    def oracle():
+        br = [rc.conv(x, L[i][0], L[i][1], wqf=L[i][2], calib=L[i][3], pad=(ks[i] // 2,) * 2, out_dt="u8", act="relu") for i in range(3)]
+        cat = np.concatenate(br, axis=1)
+        return cat, rc.conv(cat, L[3][0], L[3][1], wqf=L[3][2], calib=L[3][3], pad=(1, 1), out_dt="u8", act="relu")
+
+    return cl.topology(*prims), x, oracle
+
+
+@pytest.mark.parametrize("optimize", OPT, ids=["plain", "optimize_data"])
+def test_concatenation_of_quantized_branches(eng, optimize):
+    topo, x, oracle = inception_like(eng, 11)
+    net = cl.network(eng, topo, cl.build_options(optimize_data=optimize, outputs=["cat", "next"]) if not optimize
+                     else cl.build_options(optimize_data=True))
+    net.set_input_data("input", cl.make_memory(eng, x))
+    outs = net.execute()
+    cat, nxt = oracle()
+    np.testing.assert_array_equal(outs["next"].get_memory().read(), nxt)
+    info = net.get_primitive_info("cat")
+    if optimize:
+        # the branches wrote straight into the concatenation's buffer (reference prepare_buffer_fusing.cpp:38-140), each with
+        # the border the convolution behind the concatenation needs
+        assert info["in_place"] is True and info["format"] == F.fs_b_yx_fsv16 and info["pad_lower"][2:] == [1, 1]
+        offs = [net.get_primitive_info(f"br{i}")["concat_offset"] for i in range(3)]
+        plane = 2 * (9 + 2) * (7 + 2) * 16  # batch x padded rows x padded pixels x 16 features
+        assert offs == [0, 2 * plane, 5 * plane]
+        for _ in range(2):  # again: same buffers
+            np.testing.assert_array_equal(net.execute()["next"].get_memory().read(), nxt)
+    else:
+        assert info["in_place"] is False
+        np.testing.assert_array_equal(outs["cat"].get_memory().read(), cat)
+
+
+def test_concatenation_as_an_output_is_in_place_too(eng):
+    """the concatenation's own buffer is what the application reads (through the reorder back to its format)"""
+    topo, x, oracle = inception_like(eng, 12, B=1, f=(16, 16, 32))
+    net = cl.network(eng, topo, cl.build_options(optimize_data=True, outputs=["cat", "next"]))
+    net.set_input_data("input", cl.make_memory(eng, x))
+    outs = net.execute()
+    cat, nxt = oracle()
+    np.testing.assert_array_equal(outs["cat"].get_memory().read(), cat)
+    np.testing.assert_array_equal(outs["next"].get_memory().read(), nxt)
+    assert net.get_primitive_info("cat_fsv16")["in_place"] is True
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.int8], ids=["f32", "i8"])
+@pytest.mark.parametrize("axis", ["b", "f", "x", "y"])
+def test_concatenation_copies_along_every_axis(eng, axis, dtype):
+    """inputs that are user memory: one copy per input at its offset (reference src/gpu/concatenation_gpu.cpp:64-90,
+    concatenation_gpu_ref.cl:18-46); three inputs of different extent along the axis"""
+    r = np.random.default_rng(5)
+    ax = "bfyx".index(axis)
+    shapes = []
+    for extent in (2, 5, 1):
+        s = [3, 4, 6, 5]
+        s[ax] = extent
+        shapes.append(tuple(s))
+    arrs = [(r.standard_normal(s) * 50).astype(dtype) for s in shapes]
+    dt = DT.f32 if dtype == np.float32 else DT.i8
+    prims = [cl.input_layout(f"i{k}", cl.layout(dt, F.bfyx, cl.tensor(s[0], s[1], s[3], s[2]))) for k, s in enumerate(shapes)]
+    prims.append(cl.concatenation("cat", ["i0", "i1", "i2"], getattr(cl.concatenation_axis, "along_" + axis)))
+    for optimize in OPT:
+        net, outs = run(eng, cl.topology(*prims), {f"i{k}": cl.make_memory(eng, a) for k, a in enumerate(arrs)}, optimize)
+        np.testing.assert_array_equal(outs["cat"].get_memory().read(), np.concatenate(arrs, axis=ax))
+        assert net.get_primitive_info("cat")["in_place"] is False
+
+
+def test_copy_region_between_layouts():
+    """the C-ABI entry behind the copies: a bfyx block into the middle of a padded blocked tensor and back"""
+    from cldnn_amd import hip
+    e = hip.Engine()
+    r = np.random.default_rng(8)
+    big = r.integers(-128, 128, (2, 40, 7, 6)).astype(np.int8)
+    part = r.integers(-128, 128, (1, 19, 3, 4)).astype(np.int8)
+    dst = hip.upload(e, big, "fs_b_yx_fsv16", (1, 2))
+    src = hip.upload(e, part, "bfyx")
+    hip.check(hip.lib().cldnn_hip_copy_region(e.h, src.ptr, C.byref(src.tensor), dst.ptr, C.byref(dst.tensor), 1, 17, 2, 1))
+    want = big.copy()
+    want[1:2, 17:36, 2:5, 1:5] = part
+    np.testing.assert_array_equal(hip.download(e, dst), want)
+    assert hip.lib().cldnn_hip_copy_region(e.h, src.ptr, C.byref(src.tensor), dst.ptr, C.byref(dst.tensor), 1, 22, 2, 1) == -7  # does not fit
+    src.close(), dst.close(), e.close()
