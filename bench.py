@@ -130,12 +130,19 @@ def build_stack(eng, layers, batch, fuse_residual, seed=1337, tile=0, in_dt=np.u
         L.info = L.conv.info()
         L.kept = True
         out.append(L)
-    # the chains: three stages where the library takes them, else two, else the layers run one by one
-    for i, L in enumerate(out):
-        n = L.spec.get("chain_len", 1)
+    # the chains: as many stages as the library takes (three, else two); where it refuses a head, that layer runs
+    # alone and the layers behind it are tried as a chain of their own (a block's closing 1x1 with the next block's
+    # opening 1x1)
+    i = 0
+    while i < len(out):
+        L = out[i]
+        want = L.spec.get("chain_len", 1)
+        n = want
         while n > 1:
             members = out[i:i + n]
-            keep = [False] + [True] * (n - 1)  # only the next stage reads the first stage's result
+            # the first stage's result is read by the next stage only, unless it closes a block (then the next
+            # block's sum reads it too)
+            keep = [bool(L.spec["closes_block"])] + [True] * (n - 1)
             try:
                 L.chain = hip.ConvChain(eng, [(M.desc, M.w, M.bias, M.wqf, M.calib, M.ecal) for M in members], keep)
             except hip.HipError as e:
@@ -146,18 +153,19 @@ def build_stack(eng, layers, batch, fuse_residual, seed=1337, tile=0, in_dt=np.u
             L.members = members
             L.chain_args = L.chain.pointers([M.out if k else None for M, k in zip(members, keep)], [M.ein for M in members])
             L.info = L.chain.info()
-            L.kept = False
+            L.kept = keep[0]
             for M in members[1:]:
                 M.info = None  # counted in the chain head
             break
-        if L.chain is None and n == 1 and L.spec.get("chain_len", 1) > 1:
-            log("bench.py: %s and its followers do not chain on this device, running them one by one" % L.spec["name"])
-        if L.chain is None or len(L.members) < L.spec.get("chain_len", 1):
-            # followers that did not make it into a chain need a real input tensor: the layer before them writes it
-            first_loose = i + (len(L.members) if L.chain is not None else 1)
-            for j in range(first_loose, i + L.spec.get("chain_len", 1)):
-                M = out[j]
-                M.follows, M.xin_from = False, out[j - 1]
+        if n < want:
+            # the first layer left out needs a real input tensor: the layer before it writes it
+            M = out[i + n]
+            M.follows, M.xin_from = False, out[i + n - 1]
+            if want - n > 1:
+                M.spec = dict(M.spec, chain_len=want - n)
+            if n == 1:
+                log("bench.py: %s does not head a chain on this device, it runs alone" % L.spec["name"])
+        i += n
     return out
 
 
@@ -168,10 +176,10 @@ def launches(stack):
     for L in stack:
         if L.follows:
             continue
+        src = L.xin.ptr if L.xin is not None else L.xin_from.out.ptr
         if L.chain is not None:
-            seq.append((lib.cldnn_hip_conv_chain_enqueue, (L.chain.h, L.xin.ptr, L.chain_args[0], L.chain_args[1])))
+            seq.append((lib.cldnn_hip_conv_chain_enqueue, (L.chain.h, src, L.chain_args[0], L.chain_args[1])))
         else:
-            src = L.xin.ptr if L.xin is not None else L.xin_from.out.ptr
             seq.append((lib.cldnn_hip_conv_enqueue, (L.conv.h, src, L.out.ptr, L.ein.ptr if L.ein is not None else None)))
     return seq
 

@@ -185,6 +185,27 @@ __device__ __forceinline__ int pack_signed(const float* v)
     return (int)(q0 | (q1 << 8) | (q2 << 16) | (q3 << 24));
 }
 
+// Placed at the top of a conditional block of plain arithmetic, this keeps the branch a branch.  Without it the
+// compiler evaluates the block for every value whatever the condition says and selects afterwards: three extra
+// instructions per output for the two residual types, two and a half for the mask below.
+__device__ __forceinline__ void keep_branch() { asm volatile(""); }
+
+// partly filled last feature slice: the padding features stay zero
+__device__ __forceinline__ void zero_padding_features(v4i& packed, int valid)
+{
+    if (valid < 16) {
+        keep_branch();
+#pragma unroll
+        for (int d = 0; d < 4; ++d) {
+            unsigned keep = 0;
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+                if (d * 4 + i < valid) keep |= 255u << (8 * i);
+            packed[d] &= (int)keep;
+        }
+    }
+}
+
 // ---------------------------------------------------------------------------------------------------
 // Short epilogue for int8 outputs in the float-requantisation mode.  Same operations in the same
 // order as the long form, with three exact rewrites: "round then saturate" becomes "clamp then round"
@@ -209,43 +230,34 @@ __device__ __forceinline__ v4i epilogue_fast16(const Args& a, const v4i (&acc)[4
         }
 #pragma unroll
         for (int d = 0; d < 4; ++d) packed[d] = pack_signed(v + d * 4);
-        if (valid < 16) {
-#pragma unroll
-            for (int d = 0; d < 4; ++d) {
-                unsigned keep = 0;
-#pragma unroll
-                for (int i = 0; i < 4; ++i)
-                    if (d * 4 + i < valid) keep |= 255u << (8 * i);
-                packed[d] &= (int)keep;
-            }
-        }
+        zero_padding_features(packed, valid);
         return packed;
     }
     if constexpr (EPI == EPI_KIND_SUMLIN) {
         // the run-time form's steps for a sum without activation, in the same order; ecal[] holds ones where the sum has
         // no calibration factors
         v4i packed;
+        // without the saturation the bounds are infinite: one instruction that changes nothing instead of a select
+        const float clo = F.conv_sat ? F.conv_lo : -__builtin_inff(), chi = F.conv_sat ? F.conv_hi : __builtin_inff();
+        float e[16];
+        if (F.eltw_u8) {
+            keep_branch();
+#pragma unroll
+            for (int c = 0; c < 16; ++c) e[c] = (float)(((unsigned)ev4[c >> 2] >> (8 * (c & 3))) & 255u);
+        } else {
+            keep_branch();
+#pragma unroll
+            for (int c = 0; c < 16; ++c) e[c] = (float)(int)(int8_t)((unsigned)ev4[c >> 2] >> (8 * (c & 3)));
+        }
 #pragma unroll
         for (int c = 0; c < 16; ++c) {
-            float r = rha(v[c] * cal[c]);
-            if (F.conv_sat) r = med3(r, F.conv_lo, F.conv_hi);
-            const unsigned word = (unsigned)ev4[c >> 2];
-            const float e = F.eltw_u8 ? (float)((word >> (8 * (c & 3))) & 255u) : (float)(int)(int8_t)(word >> (8 * (c & 3)));
-            const float y = med3((r + e) * ecal[c], F.lo, F.hi);
+            const float r = med3(rha(v[c] * cal[c]), clo, chi);
+            const float y = med3((r + e[c]) * ecal[c], F.lo, F.hi);
             v[c] = y + copysignf(0.49999997f, y);
         }
 #pragma unroll
         for (int d = 0; d < 4; ++d) packed[d] = pack_signed(v + d * 4);
-        if (valid < 16) {
-#pragma unroll
-            for (int d = 0; d < 4; ++d) {
-                unsigned keep = 0;
-#pragma unroll
-                for (int i = 0; i < 4; ++i)
-                    if (d * 4 + i < valid) keep |= 255u << (8 * i);
-                packed[d] &= (int)keep;
-            }
-        }
+        zero_padding_features(packed, valid);
         return packed;
     }
     if constexpr (EPI == EPI_KIND_CLAMPQ) {
@@ -256,16 +268,7 @@ __device__ __forceinline__ v4i epilogue_fast16(const Args& a, const v4i (&acc)[4
         for (int c = 0; c < 16; ++c) v[c] = med3(v[c] * wq[c], F.act_m, F.act_n) * cal[c] + 0.49999997f;
 #pragma unroll
         for (int d = 0; d < 4; ++d) packed[d] = pack_nonneg(v + d * 4);
-        if (valid < 16) {
-#pragma unroll
-            for (int d = 0; d < 4; ++d) {
-                unsigned keep = 0;
-#pragma unroll
-                for (int i = 0; i < 4; ++i)
-                    if (d * 4 + i < valid) keep |= 255u << (8 * i);
-                packed[d] &= (int)keep;
-            }
-        }
+        zero_padding_features(packed, valid);
         return packed;
     }
     if constexpr (EPI == EPI_KIND_RELU || EPI == EPI_KIND_FUSED) {
@@ -275,10 +278,12 @@ __device__ __forceinline__ v4i epilogue_fast16(const Args& a, const v4i (&acc)[4
             for (int c = 0; c < 16; ++c) v[c] = med3(v[c] * cal[c], 0.0f, F.hi) + 0.49999997f;
         } else {
             if (F.eltw_u8) {
+                keep_branch();
 #pragma unroll
                 for (int c = 0; c < 16; ++c)
                     v[c] = rha(v[c] * cal[c]) + (float)(((unsigned)ev4[c >> 2] >> (8 * (c & 3))) & 255u);
             } else {
+                keep_branch();
 #pragma unroll
                 for (int c = 0; c < 16; ++c)
                     v[c] = rha(v[c] * cal[c]) + (float)(int)(int8_t)((unsigned)ev4[c >> 2] >> (8 * (c & 3)));
@@ -288,16 +293,7 @@ __device__ __forceinline__ v4i epilogue_fast16(const Args& a, const v4i (&acc)[4
         }
 #pragma unroll
         for (int d = 0; d < 4; ++d) packed[d] = pack_nonneg(v + d * 4);
-        if (valid < 16) {
-#pragma unroll
-            for (int d = 0; d < 4; ++d) {
-                unsigned keep = 0;
-#pragma unroll
-                for (int i = 0; i < 4; ++i)
-                    if (d * 4 + i < valid) keep |= 255u << (8 * i);
-                packed[d] &= (int)keep;
-            }
-        }
+        zero_padding_features(packed, valid);
         return packed;
     }
     if (F.has_wqf) {
@@ -391,16 +387,7 @@ __device__ __forceinline__ v4i epilogue_fast16(const Args& a, const v4i (&acc)[4
             for (int d = 0; d < 4; ++d) packed[d] = pack_signed(v + d * 4);
         }
     }
-    if (valid < 16) {  // partly filled last feature slice: the padding features stay zero
-#pragma unroll
-        for (int d = 0; d < 4; ++d) {
-            unsigned keep = 0;
-#pragma unroll
-            for (int i = 0; i < 4; ++i)
-                if (d * 4 + i < valid) keep |= 255u << (8 * i);
-            packed[d] &= (int)keep;
-        }
-    }
+    zero_padding_features(packed, valid);
     return packed;
 }
 
