@@ -59,13 +59,17 @@ def chain_groups(layers, fuse_residual):
     return out
 
 
-def build_stack(eng, layers, batch, fuse_residual, seed=1337, tile=0, in_dt=np.uint8, chains=True):
+def build_stack(eng, layers, batch, fuse_residual, seed=1337, tile=0, in_dt=np.uint8, chains=True, siblings=None):
     """Create device tensors and convolution objects for every layer (seeded synthetic data).
 
     chains: neighbouring layers that feed each other in the network (follows_prev) run as ONE launch of the
     convolution chain kernel where the library accepts them (a spatial convolution followed by one or two 1x1
     convolutions); a chained layer reads what the layer before it produced instead of a fresh random tensor, and the
-    result of a chain's first stage, which only the second stage reads, is never written."""
+    result of a chain's first stage, which only the second stage reads, is never written.
+    siblings (default: as chains): a layer that reads the same tensor as the one before it (shares_input: a block's
+    opening 1x1 beside the shortcut projection) runs in that layer's launch; its result is the tail of the launch's
+    output buffer.  Such a layer reads the same input data as its neighbour either way."""
+    siblings = chains if siblings is None else siblings
     out = []
     follows = set()  # indices of layers that run as stage 1 / 2 of a chain
     if chains and not tile:
@@ -84,7 +88,14 @@ def build_stack(eng, layers, batch, fuse_residual, seed=1337, tile=0, in_dt=np.u
         lo, hi = (0, 256) if in_dt == np.uint8 else (-128, 128)
         L.follows = i in follows
         L.chain = None
-        L.x = None if L.follows else r.integers(lo, hi, (batch, ifm, hw, hw), dtype=np.int16).astype(in_dt)
+        L.shares = bool(l.get("shares_input")) and i > 0 and not out[-1].follows
+        L.sibling = None
+        if L.follows:
+            L.x = None
+        elif L.shares:
+            L.x = out[-1].x
+        else:
+            L.x = r.integers(lo, hi, (batch, ifm, hw, hw), dtype=np.int16).astype(in_dt)
         L.w = r.integers(-127, 128, (ofm, ifm // g, k, k), dtype=np.int16).astype(np.int8)
         L.bias = r.integers(-1000, 1001, ofm).astype(np.int32)
         L.wqf = np.ones(ofm, np.float32)
@@ -106,6 +117,9 @@ def build_stack(eng, layers, batch, fuse_residual, seed=1337, tile=0, in_dt=np.u
         if L.follows:  # reads the int8 tensor of the stage before it, which stays in registers
             L.xin = None
             in_tensor = hip.Tensor.make(hip.S8, hip.FS_B_YX_FSV16, batch, ifm, hw, hw)
+        elif L.shares:
+            L.xin = out[-1].xin
+            in_tensor = L.xin.tensor
         else:
             L.xin = hip.upload(eng, L.x, "b_fs_yx_fsv4" if first else "fs_b_yx_fsv16", (l["pad"], l["pad"]))
             in_tensor = L.xin.tensor
@@ -166,6 +180,30 @@ def build_stack(eng, layers, batch, fuse_residual, seed=1337, tile=0, in_dt=np.u
             if n == 1:
                 log("bench.py: %s does not head a chain on this device, it runs alone" % L.spec["name"])
         i += n
+    # two convolutions of one input in one launch, where the library has a short epilogue for the pair
+    for H, M in zip(out, out[1:]):
+        if not (siblings and not tile and M.shares and H.chain is None and M.chain is None and not H.fused and not M.fused
+                and H.spec["ofm"] % 16 == 0):
+            continue
+        cat = lambda a, b: np.concatenate([a, b])
+        w = cat(H.w, M.w)
+        kw = dict(H.kw, sibling_split=H.spec["ofm"], sibling_act=M.kw["act"], sibling_act_m=M.kw.get("act_m", 0.0),
+                  sibling_act_n=M.kw.get("act_n", 0.0))
+        desc = hip.conv_desc(H.xin.tensor, w.shape, "s8", **kw)
+        try:
+            both = hip.Conv(eng, desc, w, cat(H.bias, M.bias), cat(H.wqf, M.wqf), cat(H.calib, M.calib), None)
+        except hip.HipError as e:
+            if e.status != -6:
+                raise
+            continue
+        if b"generic" in both.info().kernel_name:  # no short epilogue for this pair: two launches are faster
+            both.close()
+            continue
+        H.conv.close(), M.conv.close(), H.out.close(), M.out.close()
+        H.conv, H.desc, H.info, H.sibling = both, desc, both.info(), M
+        H.whole = hip.Buffer(eng, desc.output)
+        H.out, M.out = hip.Window(H.whole, 0, H.spec["ofm"]), hip.Window(H.whole, H.spec["ofm"], M.spec["ofm"])
+        M.conv, M.info, M.follows = None, None, True  # written by the launch of H
     return out
 
 
@@ -377,16 +415,18 @@ def network_workload(args):
     # what the built network launches: members of a convolution chain are written by the launch of the chain's head
     infos = {i: net.get_primitive_info(i) for i in net.get_all_primitive_ids()}
     followers = [i for i, inf in infos.items() if str(inf.get("kernel", "")).startswith("in the chain of")]
+    paired = [i for i, inf in infos.items() if "launched_by" in inf]  # written by the launch of a convolution of the same input
     executed = [i for i, inf in infos.items() if inf.get("type") not in ("data", "input_layout")]
     if args.per_layer:
         for i in executed:
-            log("%-40s %s" % (i, infos[i].get("kernel", infos[i].get("type"))))
+            log("%-40s %s" % (i, "in the launch of " + infos[i]["launched_by"] if i in paired else infos[i].get("kernel", infos[i].get("type"))))
     print(json.dumps({
         "metric": "%s int8 network images/sec @b%d (whole topology through the clDNN API)" % (name, batch), "value": batch * args.steps / dt,
         "unit": "images/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": dt / args.steps * 1e3,
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "i8xi8->i32 (f32 requantisation)", "data": "synthetic",
         "config": {"workload": args.workload, "batch": batch, "primitives": primitives,
-                   "build": "optimize_data" + (", tuning cache" if args.tuning_cache else "") + (", second stream" if args.second_stream else ""), "primitives_per_execute": len(executed), "launches_per_execute": len(executed) - len(followers),
+                   "build": "optimize_data" + (", tuning cache" if args.tuning_cache else "") + (", second stream" if args.second_stream else ""), "primitives_per_execute": len(executed), "launches_per_execute": len(executed) - len(followers) - len(paired),
+                   "convolutions_in_a_neighbours_launch": len(paired),
                    "chained_convolutions": len(followers) + len({str(infos[i]["kernel"]) for i in followers}),
                    "executed_ops_per_step": ops, "nominal_ops_per_step": nominal},
         "roofline": {"bound": "mfma", "achieved": ops * args.steps / dt / 1e12, "peak": PEAK_INT8_OPS / 1e12, "unit": "TOP/s",
@@ -441,7 +481,11 @@ def release_stack(stack):
     for L in stack:
         if L.chain is not None:
             L.chain.close()
-        L.conv.close(), L.out.close()
+        if L.conv is not None:
+            L.conv.close()
+        L.out.close()
+        if L.sibling is not None:
+            L.whole.close()
         if L.xin is not None:
             L.xin.close()
         if L.ein is not None:
@@ -584,7 +628,7 @@ def measure_stack(args, wl, steps, warmup, in_flight_n, cpu_seconds, extras):
         for L, dt in zip(stk, times):
             tops, gbs = L.info.ops / dt / 1e12, L.info.bytes / dt / 1e9
             t_m, t_h = L.info.ops / PEAK_INT8_OPS, L.info.bytes / PEAK_HBM
-            name = L.spec["name"] + ("+%d" % (len(L.members) - 1) if L.chain is not None else "")
+            name = L.spec["name"] + ("+%d" % (len(L.members) - 1) if L.chain is not None else "") + ("|1" if L.sibling is not None else "")
             log("%-18s %-52s %6d %9.1f %8.1f %8.0f %7s %5.1f%%" % (
                 name, L.info.kernel_name.decode(), L.info.grid, dt * 1e6, tops, gbs,
                 "mfma" if t_m > t_h else "hbm", 100 * max(t_m, t_h) / dt))
@@ -630,6 +674,7 @@ def measure_stack(args, wl, steps, warmup, in_flight_n, cpu_seconds, extras):
         "ms_per_step": t_wall / steps * 1e3,
         "config": {"workload": wl, "batch": batch, "layers": len(stack), "launches_per_step": len(seq),
                    "chained_layers": sum(len(L.members) for L in stack if L.chain is not None),
+                   "layers_in_a_neighbours_launch": sum(1 for L in stack if L.sibling is not None),
                    "layout": "fs_b_yx_fsv16",
                    "variant": "stride on the first 1x1 (Caffe form)" if wl.startswith("resnet50") else wl,
                    "fused_residual_layers": sum(1 for L in stack if L.fused)},
@@ -695,7 +740,7 @@ def main():
                     choices=["resnet50_b32_fused", "resnet50_b32", "resnet50_b1", "vgg16_b16", "mobilenet_v2_b32", "c1",
                              "copy_256m", "resnet50_b32_network", "mobilenet_v2_b32_network", "vgg16_b16_network"])
     ap.add_argument("--tile", type=int, default=0, help="force one row (index+1) of the tile table on every layer (no chains)")
-    ap.add_argument("--no-chains", action="store_true", help="every layer is a launch of its own (no convolution chains)")
+    ap.add_argument("--no-chains", action="store_true", help="every layer is a launch of its own (no convolution chains, no two convolutions of one input in one launch)")
     ap.add_argument("--per-layer", action="store_true", help="print the per-launch table to stderr")
     ap.add_argument("--tune", action="store_true", help="try every row of the tile table on every layer, print the best")
     ap.add_argument("--only", default="", help="comma-separated layer names: run just these layers of the workload "

@@ -71,6 +71,9 @@ struct Epilogue {
     int32_t round_even;
     int32_t fc;              // quantized fully_connected form (see cldnn_hip_conv_desc.fully_connected)
     int32_t conv_sat;        // fused form: 1 / 2 = the rounded convolution result is saturated to s8 / u8 before the sum
+    int32_t split_f;         // > 0: features from here on take act2 (two convolutions of one input in one launch)
+    int32_t act2;
+    float act2_m, act2_n;
 };
 
 }  // namespace chip

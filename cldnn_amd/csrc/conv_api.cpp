@@ -159,6 +159,17 @@ void build(cldnn_hip_conv c, const void* weights, const void* bias, const float*
     CHIP_REQUIRE(d.conv_saturate >= 0 && d.conv_saturate <= 2 && (!d.conv_saturate || (d.fused && d.has_wqf)), CLDNN_HIP_INVALID_ARG,
                  "conv_saturate is 0, 1 (s8) or 2 (u8) and goes with the quantized fused form");
     e.conv_sat = d.conv_saturate;
+    if (d.sibling_split) {
+        CHIP_REQUIRE(d.sibling_split > 0 && d.sibling_split < d.ofm && d.sibling_split % 16 == 0, CLDNN_HIP_INVALID_ARG,
+                     "sibling_split is a multiple of 16 inside (0, ofm)");
+        CHIP_REQUIRE(d.groups == 1 && d.has_wqf && !d.fused && !d.fully_connected, CLDNN_HIP_UNSUPPORTED_FORMAT,
+                     "two convolutions in one launch: one group, the quantized form, no fused second input");
+        // one convolution as far as the arithmetic goes when both sides take the same activation
+        const bool same = d.sibling_activation == d.activation
+                          && (d.activation == CLDNN_HIP_ACT_NONE || d.activation == CLDNN_HIP_ACT_RELU
+                              || (d.sibling_activation_m == d.activation_m && d.sibling_activation_n == d.activation_n));
+        if (!same) e.split_f = d.sibling_split, e.act2 = d.sibling_activation, e.act2_m = d.sibling_activation_m, e.act2_n = d.sibling_activation_n;
+    }
     if (e.fc) {
         CHIP_REQUIRE(p.OH == 1 && p.OW == 1 && p.FY == p.IH && p.FX == p.IW && p.py == 0 && p.px == 0, CLDNN_HIP_INVALID_ARG,
                      "fully_connected: the filter must cover the whole input plane");
@@ -429,6 +440,7 @@ cldnn_hip_status cldnn_hip_conv_chain_create(cldnn_hip_engine e, int32_t count, 
                              "stage " + std::to_string(k) + " of a chain must be a dense int8 convolution in fs_b_yx_fsv16 (the first "
                              "stage may be a depthwise 3x3)");
                 CHIP_REQUIRE(!descs[k].second_input_in_output, CLDNN_HIP_UNSUPPORTED_FORMAT, "a chained stage cannot read its residual from its own output");
+                CHIP_REQUIRE(!descs[k].sibling_split, CLDNN_HIP_UNSUPPORTED_FORMAT, "a chained stage cannot be two convolutions in one");
                 CHIP_REQUIRE(descs[k].groups == 1 || dw_head, CLDNN_HIP_UNSUPPORTED_FORMAT, "a chained stage cannot be a grouped convolution");
                 ch->keep[k] = keep_output ? (keep_output[k] != 0) : 1;
                 ch->in[k] = ChainStageIn{&c->p, &c->epi, &c->fe, c->fast, (const int32_t*)c->acc_init,

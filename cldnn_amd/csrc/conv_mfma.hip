@@ -148,6 +148,7 @@ int mfma_choose(const ConvProblem& p, int cus)
     if (ksteps <= 8) {
         if (m >= 16384) return ROW_WSL_P64;                       // 1x1 reductions at 56x56 and 28x28
         if (m >= 4096) {
+            if (p.OFM > 1024) return ROW_P64_F128;  // a 14x14 projection together with the block's opening 1x1
             if (p.OFM >= 512) return ksteps <= 4 ? ROW_WSL_P128 : ROW_BDIR_P128_F128;  // 14x14 expansions / projections
             return stream_fits ? stream_row : ROW_BDIR_P64_F64;
         }
@@ -165,6 +166,7 @@ int mfma_choose(const ConvProblem& p, int cus)
     }
     if (m >= 4096) return ROW_BDIR_P64_F64;                        // 14x14
     if (ksteps >= 32) return m >= 2048 ? ROW_BDIR_K2_P128_F64 : ROW_BDIR_K2_P64_F64;  // few pixels, K >= 2048: split K
+    if (p.OFM > 2048 && m >= 512) return ROW_P64_F128;  // a 7x7 projection together with the block's opening 1x1
     if (p.OFM >= 1024 && m >= 512) return ROW_P128_F128;
     return ROW_BDIR_P64_F64;
 }
@@ -347,6 +349,28 @@ bool mfma_fast_epilogue(const ConvProblem& p, const Epilogue& e, const float* ca
         return false;  // an int32 bias is folded into the accumulator start; a float bias takes the long path
     }
     if (!(e.out_dt == CLDNN_HIP_S8 || e.out_dt == CLDNN_HIP_U8)) return false;
+    if (e.split_f > 0) {
+        // Two convolutions in one launch: only the branch-free clamp form is written for it.  It needs per-feature
+        // output factors that are finite (and not negative where a relu is folded into the clamp), unit weight factors,
+        // and none / relu on both sides.
+        auto plain = [](int act) { return act == CLDNN_HIP_ACT_NONE || act == CLDNN_HIP_ACT_RELU; };
+        if (e.fc || e.fused || !calib || !plain(e.act) || !plain(e.act2) || !tame(calib, p.OFM)) return false;
+        if (e.iqf != 1.0f) return false;
+        if (wqf)
+            for (int f = 0; f < p.OFM; ++f)
+                if (wqf[f] != 1.0f) return false;
+        for (int f = 0; f < p.OFM; ++f)
+            if ((f < e.split_f ? e.act : e.act2) == CLDNN_HIP_ACT_RELU && !(calib[f] >= 0.0f)) return false;
+        F.hi = e.out_dt == CLDNN_HIP_S8 ? 127.0f : 255.0f;
+        const float type_lo = e.out_dt == CLDNN_HIP_S8 ? -128.0f : 0.0f;
+        F.lo = e.act == CLDNN_HIP_ACT_RELU ? 0.0f : type_lo;
+        F.lo2 = e.act2 == CLDNN_HIP_ACT_RELU ? 0.0f : type_lo;
+        F.split_valid = p.OFM - e.split_f;
+        F.act = CLDNN_HIP_ACT_NONE;  // what is left of the activations is in the bounds
+        F.iqf = 1.0f, F.iqf_one = 1;
+        *out = F;
+        return true;
+    }
     if (!(e.act == CLDNN_HIP_ACT_NONE || e.act == CLDNN_HIP_ACT_RELU || e.act == CLDNN_HIP_ACT_CLAMP)) return false;
     if (e.act == CLDNN_HIP_ACT_CLAMP && !(e.act_m <= e.act_n)) return false;  // the median form needs ordered bounds
     // factors small enough that no product can overflow into inf * 0

@@ -81,7 +81,8 @@ struct MfmaArgs {
 // VGG stacks consist of, with nothing left to decide at run time:
 //   RELU   clamp(acc * cal, 0, hi)                                    (relu, scales >= 0, unit wqf)
 //   FUSED  clamp((round(acc * cal) + residual) * ecal, 0, hi)         (residual relu, scales >= 0)
-//   LINEAR clamp(acc * cal, lo, hi)                                   (no activation, unit wqf)
+//   LINEAR clamp(acc * cal, lo, hi)                                   (no activation, unit wqf; with two convolutions in one
+//                                                                      launch lo is 0 for the features of the one with a relu)
 //   CLAMPQ clamp(acc * wqf, m, n) * cal, rounded                      (folded clamp{m, n} with 0 <= m, e.g. ReLU6 on the
 //                                                                      dequantised value; unit input factor; chain kernels)
 //   SUMLIN clamp((sat(round(acc * cal)) + residual) * ecal, lo, hi)    (residual sum without activation, the rounded
@@ -223,9 +224,10 @@ __device__ __forceinline__ v4i epilogue_fast16(const Args& a, const v4i (&acc)[4
     for (int c = 0; c < 16; ++c) v[c] = (float)acc[c >> 2][nt][c & 3];
     if constexpr (EPI == EPI_KIND_LINEAR) {
         v4i packed;
+        const float lo = valid <= F.split_valid ? F.lo2 : F.lo;
 #pragma unroll
         for (int c = 0; c < 16; ++c) {
-            const float y = med3(v[c] * cal[c], F.lo, F.hi);
+            const float y = med3(v[c] * cal[c], lo, F.hi);
             v[c] = y + copysignf(0.49999997f, y);
         }
 #pragma unroll

@@ -122,7 +122,8 @@ __device__ __forceinline__ EpiOut epilogue_generic(const Epilogue& e, int acc, i
             deq = deq * e.iqf;
         }
         if (e.bias_after) deq = deq + ((const float*)e.bias)[f];
-        float a = act_f(e.act, e.act_m, e.act_n, deq);
+        const bool second = e.split_f > 0 && f >= e.split_f;  // the sibling convolution's features
+        float a = second ? act_f(e.act2, e.act2_m, e.act2_n, deq) : act_f(e.act, e.act_m, e.act_n, deq);
         float cal = a;
         if (e.calib) cal = a * e.calib[f];
         else if (e.oqf_on) cal = a * e.oqf;

@@ -99,6 +99,11 @@ struct FastEpi {
     int32_t conv_sat;     // fused: the rounded convolution result is limited to [conv_lo, conv_hi] before the sum
     float conv_lo, conv_hi;
     int32_t fc;           // the fully_connected form: float bias after the dequantisation, conversion to char keeps the low byte
+    // two convolutions of one input in one launch: a 16-feature group with at most split_valid features from its start
+    // to the end of the output belongs to the second one and clamps from lo2 instead of lo (0 for a folded relu, the
+    // type's lower bound without activation).  split_valid == 0: one convolution.
+    int32_t split_valid;
+    float lo2;
 };
 // true (and *out filled) when the short epilogue reproduces the long one bit for bit
 bool mfma_fast_epilogue(const ConvProblem& p, const Epilogue& e, const float* calib, const float* ecal, const float* wqf,

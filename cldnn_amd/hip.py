@@ -68,6 +68,10 @@ class ConvDesc(C.Structure):
         ("impl", C.c_int32), ("tile_override", C.c_int32),
         ("pad_end_delta_y", C.c_int32), ("pad_end_delta_x", C.c_int32), ("fully_connected", C.c_int32),
         ("conv_saturate", C.c_int32),
+        ("sibling_split", C.c_int32),
+        ("sibling_activation", C.c_int32),
+        ("sibling_activation_m", C.c_float),
+        ("sibling_activation_n", C.c_float),
     ]
 
 
@@ -268,6 +272,27 @@ class Buffer:
             self.close()
         except Exception:
             pass
+
+
+class Window:
+    """Feature slices [first / 16, (first + features) / 16) of an fs_b_yx_fsv16 Buffer as a tensor of its own: the feature
+    slice is the outermost axis of that layout, so a range of slices is contiguous memory."""
+
+    def __init__(self, buf, first, features):
+        t = buf.tensor
+        assert t.format == FS_B_YX_FSV16 and first % 16 == 0 and first + features <= t.f and not (t.pad_lo_f or t.pad_hi_f)
+        assert first + features == t.f or features % 16 == 0
+        self.buf, self.engine = buf, buf.engine
+        self.tensor = Tensor.make(t.dtype, t.format, t.b, features, t.y, t.x, t.pad_lo_y, t.pad_lo_x, t.pad_hi_y, t.pad_hi_x)
+        self.nbytes = lib().cldnn_hip_tensor_bytes(C.byref(self.tensor))
+        self.offset = (first // 16) * (buf.nbytes // (-(-t.f // 16)))
+
+    @property
+    def ptr(self):
+        return self.buf.ptr + self.offset
+
+    def close(self):
+        pass  # the Buffer owns the memory
 
 
 def reorder(engine, src, dst):
@@ -498,7 +523,8 @@ def conv_desc(x_t, w_shape, out_dt, *, stride=(1, 1), pad=(0, 0), dilation=(1, 1
               out_pad=(0, 0), bias_dt=NO_TYPE, w_dt=S8, has_wqf=False, has_calib=False, iqf=1.0, oqf=1.0,
               act="none", act_m=0.0, act_n=0.0, eltw_t=None, non_conv_scale=1.0, eltw_act="none", eltw_m=0.0,
               eltw_n=0.0, has_eltw_calib=False, eltw_stride=(1, 1), in_place=False, round_even=False,
-              impl=IMPL_AUTO, tile=0, pad_end=None, fc=False, conv_saturate=0):
+              impl=IMPL_AUTO, tile=0, pad_end=None, fc=False, conv_saturate=0, sibling_split=0, sibling_act="none",
+              sibling_act_m=0.0, sibling_act_n=0.0):
     """Fill a ConvDesc from an input Tensor and the weight shape [OFM, IFM/groups, FY, FX].
     pad = zero padding on the low side (y, x); pad_end = on the high side (default: the same)."""
     L = lib()
@@ -531,6 +557,9 @@ def conv_desc(x_t, w_shape, out_dt, *, stride=(1, 1), pad=(0, 0), dilation=(1, 1
     d.pad_end_delta_y, d.pad_end_delta_x = pad_end[0] - pad[0], pad_end[1] - pad[1]
     d.fully_connected = int(fc)
     d.conv_saturate = int(conv_saturate)
+    d.sibling_split = int(sibling_split)
+    d.sibling_activation = ACT_NAME[sibling_act] if isinstance(sibling_act, str) else sibling_act
+    d.sibling_activation_m, d.sibling_activation_n = sibling_act_m, sibling_act_n
     return d
 
 
@@ -544,7 +573,8 @@ def conv_forward(engine, x, w, bias=None, wqf=None, calib=None, *, stride=(1, 1)
                  groups=1, out_dt=None, iqf=1.0, oqf=1.0, act="none", act_m=0.0, act_n=0.0, eltw=None,
                  non_conv_scale=1.0, eltw_act="none", eltw_m=0.0, eltw_n=0.0, eltw_calib=None, eltw_stride=(1, 1),
                  round_even=False, fmt="bfyx", in_pad=(0, 0), out_pad=(0, 0), impl=IMPL_AUTO, tile=0,
-                 want_acc=False, want_info=False, pad_end=None, fc=False, in_place=False, conv_saturate=0):
+                 want_acc=False, want_info=False, pad_end=None, fc=False, in_place=False, conv_saturate=0, sibling_split=0,
+                 sibling_act="none", sibling_act_m=0.0, sibling_act_n=0.0):
     """numpy in, numpy out: upload (reordering to `fmt`), run the HIP convolution, download.
 
     Argument meaning follows oracle.refconv.conv so that parity tests can call both alike.  in_place: the residual
@@ -568,7 +598,8 @@ def conv_forward(engine, x, w, bias=None, wqf=None, calib=None, *, stride=(1, 1)
                   eltw_t=None if e_buf is None else e_buf.tensor, non_conv_scale=non_conv_scale, eltw_act=eltw_act,
                   eltw_m=eltw_m, eltw_n=eltw_n, has_eltw_calib=eltw_calib is not None, eltw_stride=eltw_stride,
                   round_even=round_even, impl=impl, tile=tile, pad_end=pad_end, fc=fc, in_place=in_place,
-                  conv_saturate=conv_saturate)
+                  conv_saturate=conv_saturate, sibling_split=sibling_split, sibling_act=sibling_act,
+                  sibling_act_m=sibling_act_m, sibling_act_n=sibling_act_n)
     c = Conv(engine, d, w, bias, wqf, calib, eltw_calib)
     if in_place:
         out = upload(engine, np.ascontiguousarray(eltw), "fs_b_yx_fsv16" if first_layer else fmt, out_pad)

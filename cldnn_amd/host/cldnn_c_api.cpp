@@ -233,6 +233,7 @@ static void submit(cldnn_network_impl* net, cldnn_event* deps, size_t ndeps, cld
         case prim_type::convolution:
         case prim_type::fused_conv_eltwise: {
             if (n->chain_head) break;  // written by the launch of its chain's head
+            if (n->sibling_head) break;  // written by the launch of the convolution it is paired with
             cldnn_memory_impl* in = mem_of(n->deps[0]);
             if (n->chain) {
                 void* outs[3] = {nullptr, nullptr, nullptr};
@@ -862,6 +863,7 @@ cldnn_network cldnn_allocate_network(cldnn_program program, cldnn_status* status
                 continue;
             }
             if (n->chain_unkept()) continue;  // never written: the next member of the chain takes it in registers
+            if (n->sibling_head) continue;  // a window into the pair's buffer, made when the pair's first node came up
             if (n->concat_in_place || n->concat_into) {
                 // an in-place concatenation owns one buffer of its own (outside the pool); its inputs, which come earlier
                 // in the order, are windows into it
@@ -889,10 +891,12 @@ cldnn_network cldnn_allocate_network(cldnn_program program, cldnn_status* status
                     ++it;
                 }
             }
+            cldnn_layout want = n->out;
+            if (n->sibling) want.size.sizes[1] += n->sibling->out.size.sizes[1];
             ref<cldnn_memory_impl> m;
             if (pool && !n->is_output) {
                 for (auto it = idle.begin(); it != idle.end(); ++it)
-                    if (same_layout((*it)->layout, n->out)) {
+                    if (same_layout((*it)->layout, want)) {
                         m = *it;
                         idle.erase(it);
                         net->pooled_tensors++;
@@ -900,8 +904,26 @@ cldnn_network cldnn_allocate_network(cldnn_program program, cldnn_status* status
                     }
             }
             if (!m) {
-                m = allocate(e, n->out);
-                net->allocated_bytes += layout_bytes(n->out);
+                m = allocate(e, want);
+                net->allocated_bytes += layout_bytes(want);
+            }
+            if (n->sibling) {
+                // the pair's buffer is one tensor as far as the pool goes; the two nodes see windows
+                node* b = n->sibling;
+                size_t until = last_use.count(n) ? last_use[n] : i;
+                if (last_use.count(b)) until = std::max(until, last_use[b]);
+                if (pool) in_flight.emplace_back(until, m);
+                auto window = [&](const cldnn_layout& l, size_t offset) {
+                    ref<cldnn_memory_impl> w(new cldnn_memory_impl(), false);
+                    w->layout = l;
+                    w->engine = ref<cldnn_engine_impl>(e, true);
+                    w->view_of = m;
+                    w->view_offset = offset;
+                    return w;
+                };
+                net->mem[n] = window(n->out, 0);
+                net->mem[b] = window(b->out, layout_bytes(n->out));
+                continue;
             }
             net->mem[n] = m;
             if (pool && !n->is_output && last_use.count(n)) in_flight.emplace_back(last_use[n], m);

@@ -196,6 +196,11 @@ struct node {
     node* concat_into = nullptr;
     size_t concat_offset = 0;
     bool concat_in_place = false;   // concatenation whose inputs all write into its buffer
+    // two convolutions of one input in one launch: `sibling` (on the first in execution order) is the convolution whose
+    // features follow this one's in the launch; `sibling_head` (on the second) is the node that launches for both.  The
+    // two results share one buffer (the second is its contiguous tail: feature slices are the outermost axis).
+    node* sibling = nullptr;
+    node* sibling_head = nullptr;
     // member of a chain whose result stays in registers: it has no buffer and nobody but the next member reads it
     bool chain_unkept() const
     {

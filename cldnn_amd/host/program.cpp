@@ -981,6 +981,89 @@ static void compile_conv(cldnn_program_impl* prog, node* n)
     hip_check(cldnn_hip_conv_get_info(n->conv, &n->conv_info));
 }
 
+// ------------------------------------------------------------------------------------------ sibling convolutions
+// Two quantized convolutions that read the same tensor with the same filter size, stride, padding and dilation (a
+// residual block's shortcut projection and its opening 1x1; the 1x1 branches of an inception module) run as ONE launch
+// over the concatenated output features (cldnn_hip_conv_desc.sibling_split).  The reference launches every node
+// (src/gpu/primitive_gpu_base.h:117-168); the results per feature are the same.  In fs_b_yx_fsv16 the second result is the
+// contiguous tail of the pair's buffer, so both nodes keep output tensors of their own for their readers.  The pair
+// takes the wider of the two borders.  Whether the kernels have a short epilogue for the pair is decided when it is
+// compiled (compile_siblings); a pair they refuse is taken apart again.
+static bool sibling_candidate(const node* n)
+{
+    const prim& p = *n->p;
+    if (p.type != prim_type::convolution || p.fully_connected || p.split != 1 || p.groups != 1) return false;
+    if (n->is_output || n->side_stream || n->first_layer || n->concat_into || n->concat_in_place || n->sibling || n->sibling_head) return false;
+    if (n->chain_head || !n->chain_members.empty()) return false;
+    if (p.wqf.empty() || p.calib.empty() || p.iqf != 1.0f) return false;
+    for (const node* u : n->users)  // a sum written over this tensor needs it in a buffer of its own
+        if (u->p->type == prim_type::fused_conv_eltwise && u->p->second_input_in_output && u->deps.size() > 1 && u->deps[1] == n) return false;
+    const auto int8 = [](int32_t t) { return t == cldnn_i8 || t == cldnn_u8; };
+    return n->out.format == cldnn_format_fs_b_yx_fsv16 && n->deps[0]->out.format == cldnn_format_fs_b_yx_fsv16 && int8(n->out.data_type)
+           && int8(n->deps[0]->out.data_type);
+}
+
+static void pair_siblings(cldnn_program_impl* prog)
+{
+    for (size_t i = 0; i < prog->nodes.size(); ++i) {
+        node* a = prog->nodes[i].get();
+        if (!sibling_candidate(a) || a->out.size.sizes[1] % 16 != 0) continue;
+        const conv_geom ga = conv_geometry(*a->p, a->deps[0]->out, dep_named(a, a->p->weights.at(0))->out);
+        for (node* b : a->deps[0]->users) {
+            if (b == a || !sibling_candidate(b) || b->deps[0] != a->deps[0] || position(prog, b) < i) continue;
+            if (b->out.data_type != a->out.data_type || b->p->bias.empty() != a->p->bias.empty()) continue;
+            const conv_geom gb = conv_geometry(*b->p, b->deps[0]->out, dep_named(b, b->p->weights.at(0))->out);
+            if (gb.FY != ga.FY || gb.FX != ga.FX || gb.sy != ga.sy || gb.sx != ga.sx || gb.py != ga.py || gb.px != ga.px || gb.dy != ga.dy
+                || gb.dx != ga.dx || gb.ey != ga.ey || gb.ex != ga.ex || gb.vy != ga.vy || gb.vx != ga.vx || gb.OH != ga.OH || gb.OW != ga.OW)
+                continue;
+            for (int k = 0; k < 4; ++k) {
+                int32_t& la = a->out.padding.lower_size.sizes[k], &lb = b->out.padding.lower_size.sizes[k];
+                int32_t& ua = a->out.padding.upper_size.sizes[k], &ub = b->out.padding.upper_size.sizes[k];
+                la = lb = std::max(la, lb), ua = ub = std::max(ua, ub);
+            }
+            a->sibling = b, b->sibling_head = a;
+            break;
+        }
+    }
+}
+
+// One convolution object for a pair.  false: the kernels have no short form for this pair (the pair is taken apart).
+static bool compile_siblings(cldnn_program_impl* prog, node* a);
+
+static bool compile_siblings(cldnn_program_impl* prog, node* a)
+{
+    node* b = a->sibling;
+    conv_build ca, cb;
+    prepare_conv(prog, a, ca);
+    prepare_conv(prog, b, cb);
+    cldnn_hip_conv_desc d = ca.d;
+    const bool alike = ca.d.bias_dtype == cb.d.bias_dtype && ca.d.weights_dtype == cb.d.weights_dtype && cb.d.has_wqf && cb.d.has_calib
+                       && ca.d.has_wqf && ca.d.has_calib;
+    if (alike) {
+        d.sibling_split = ca.d.ofm;
+        d.sibling_activation = cb.d.activation, d.sibling_activation_m = cb.d.activation_m, d.sibling_activation_n = cb.d.activation_n;
+        d.ofm = ca.d.ofm + cb.d.ofm;
+        d.output.f = d.ofm;
+        auto join = [](std::vector<uint8_t>& x, const std::vector<uint8_t>& y) { x.insert(x.end(), y.begin(), y.end()); };
+        join(ca.wv, cb.wv), join(ca.bv, cb.bv), join(ca.qv, cb.qv), join(ca.cv, cb.cv);
+        cldnn_hip_conv c = nullptr;
+        const cldnn_hip_status st = cldnn_hip_conv_create(prog->engine->h, &d, ca.weights(), ca.bias(), ca.wqf(), ca.calib(), nullptr, &c);
+        if (st == CLDNN_HIP_SUCCESS) {
+            cldnn_hip_conv_info info{};
+            hip_check(cldnn_hip_conv_get_info(c, &info));
+            if (!std::strstr(info.kernel_name, "generic")) {
+                a->conv = c, a->conv_info = info;
+                return true;
+            }
+            cldnn_hip_conv_release(c);  // element by element two launches are faster
+        } else if (st != CLDNN_HIP_UNSUPPORTED_FORMAT && st != CLDNN_HIP_UNSUPPORTED_SIZE) {
+            hip_check(st);
+        }
+    }
+    a->sibling = nullptr, b->sibling_head = nullptr;
+    return false;
+}
+
 // ------------------------------------------------------------------------------------------ convolution chains
 // A convolution and the one or two 1x1 / stride-1 / unpadded convolutions that read its result run as ONE launch
 // (cldnn_hip_conv_chain): the tail of a ResNet bottleneck (3x3 -> 1x1 + sum -> the next block's 1x1) or of a MobileNet
@@ -995,6 +1078,7 @@ static bool chain_follower(cldnn_program_impl* prog, node* prev, node* c, size_t
     const prim& p = *c->p;
     if (p.type != prim_type::convolution && p.type != prim_type::fused_conv_eltwise) return false;
     if (p.fully_connected || p.second_input_in_output || c->side_stream || c->first_layer || c->deps[0] != prev) return false;
+    if (c->sibling || c->sibling_head) return false;
     node* w = dep_named(c, p.weights.at(0));
     const conv_geom g = conv_geometry(p, prev->out, w->out);
     if (g.FY != 1 || g.FX != 1 || g.sy != 1 || g.sx != 1 || g.py != 0 || g.px != 0 || g.groups != 1) return false;
@@ -1009,6 +1093,7 @@ static void group_chains(cldnn_program_impl* prog)
         node* head = prog->nodes[i].get();
         const prim& hp = *head->p;
         if (head->chain_head || (hp.type != prim_type::convolution && hp.type != prim_type::fused_conv_eltwise)) continue;
+        if (head->sibling || head->sibling_head) continue;  // launched as a pair
         if (hp.fully_connected || hp.second_input_in_output || head->side_stream || head->first_layer) continue;
         if (head->out.format != cldnn_format_fs_b_yx_fsv16 || head->deps[0]->out.format != cldnn_format_fs_b_yx_fsv16) continue;
         std::vector<node*> members{head};
@@ -1196,7 +1281,12 @@ void build_program(cldnn_program_impl* prog, cldnn_topology_impl* topo, const st
     if (!prog->engine) return;  // planning only: the graph is inspected, nothing is compiled
     if (prog->engine->side) assign_streams(prog);
     // chains with the graph optimisations only; a tuned program keeps one launch per node (its cache is per node)
-    if (prog->optimize_data && prog->tuning.mode == cldnn_tuning_disabled) group_chains(prog);
+    if (prog->optimize_data && prog->tuning.mode == cldnn_tuning_disabled) {
+        pair_siblings(prog);
+        for (auto& u : prog->nodes)
+            if (u->sibling) compile_siblings(prog, u.get());
+        group_chains(prog);
+    }
     for (auto& u : prog->nodes) {
         node* n = u.get();
         if (!n->chain_members.empty()) compile_chain(prog, n);
@@ -1204,7 +1294,7 @@ void build_program(cldnn_program_impl* prog, cldnn_topology_impl* topo, const st
     for (auto& u : prog->nodes) {
         node* n = u.get();
         const bool conv = n->p->type == prim_type::convolution || n->p->type == prim_type::fused_conv_eltwise;
-        if (conv && !n->chain && !n->chain_head) compile_conv(prog, n);
+        if (conv && !n->conv && !n->chain && !n->chain_head && !n->sibling_head) compile_conv(prog, n);
     }
     prog->tuning.save();
 }
@@ -1246,6 +1336,8 @@ std::string describe_node(const node* n)
     if (p.type == prim_type::concatenation) s += ",\"axis\":" + std::to_string(p.concat_axis) + ",\"in_place\":" + (n->concat_in_place ? "true" : "false");
     if (n->concat_into) s += ",\"concat_into\":\"" + n->concat_into->p->id + "\",\"concat_offset\":" + std::to_string(n->concat_offset);
     if (n->side_stream) s += ",\"stream\":1";
+    if (n->sibling) s += ",\"launches_also\":\"" + n->sibling->p->id + "\"";
+    if (n->sibling_head) s += ",\"launched_by\":\"" + n->sibling_head->p->id + "\"";
     if (n->conv || n->chain || n->chain_head)
         s += std::string(",\"kernel\":\"") + n->conv_info.kernel_name + "\",\"grid\":" + std::to_string(n->conv_info.grid)
              + ",\"ops\":" + std::to_string(n->conv_info.ops) + ",\"bytes\":" + std::to_string(n->conv_info.bytes);

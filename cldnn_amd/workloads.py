@@ -3,14 +3,17 @@
 Each entry is a dict: name, ifm, ofm, k (square filter), stride, pad, in_hw (input height = width),
 groups, act ("relu" / "none" / "relu6"), closes_block (the 1x1 that takes the residual add),
 follows_prev (in the network this layer reads the tensor the entry before it in the list writes, with nothing
-but a fused residual sum in between: such neighbours may run as one convolution chain).
+but a fused residual sum in between: such neighbours may run as one convolution chain), shares_input (in the network
+this layer reads the SAME tensor as the entry before it, with the same filter size, stride and padding: the two may run
+as one launch).
 """
 
 
-def _layer(name, ifm, ofm, k, stride, pad, in_hw, groups=1, act="relu", closes_block=False, follows_prev=False):
+def _layer(name, ifm, ofm, k, stride, pad, in_hw, groups=1, act="relu", closes_block=False, follows_prev=False,
+           shares_input=False):
     out_hw = (in_hw + 2 * pad - k) // stride + 1
     return dict(name=name, ifm=ifm, ofm=ofm, k=k, stride=stride, pad=pad, in_hw=in_hw, out_hw=out_hw, groups=groups,
-                act=act, closes_block=closes_block, follows_prev=follows_prev)
+                act=act, closes_block=closes_block, follows_prev=follows_prev, shares_input=shares_input)
 
 
 def resnet50(stride_on_3x3=False):
@@ -30,7 +33,8 @@ def resnet50(stride_on_3x3=False):
                 L.append(_layer(n + "_branch1", cin, width * 4, 1, s, 0, hw, act="none"))
             # a block's first 1x1 reads the sum the block before it closes with (not in a block with a projection, whose
             # list neighbour is that projection)
-            L.append(_layer(n + "_branch2a", cin, width, 1, s1, 0, hw, follows_prev=b > 0))
+            # ... and in such a block it reads what the projection reads
+            L.append(_layer(n + "_branch2a", cin, width, 1, s1, 0, hw, follows_prev=b > 0, shares_input=b == 0 and s1 == s))
             L.append(_layer(n + "_branch2b", width, width, 3, s3, 1, mid_hw, follows_prev=True))
             L.append(_layer(n + "_branch2c", width, width * 4, 1, 1, 0, out_hw, closes_block=True, follows_prev=True))
             cin = width * 4

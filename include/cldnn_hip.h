@@ -301,6 +301,17 @@ typedef struct {
      * fused_conv_eltwise itself does not have: it adds to the unsaturated value (fused_conv_eltwise_gpu_ref.cl:199-233).
      * Lets a sum the reference leaves stand-alone run inside the convolution with unchanged results. */
     int32_t conv_saturate;
+    /* Two convolutions of the same input in one launch ("siblings": same filter size, stride, padding and dilation, e.g.
+     * a residual block's shortcut projection and its opening 1x1).  sibling_split > 0: output features [0, sibling_split)
+     * belong to the first convolution and take `activation`, features [sibling_split, ofm) belong to the second and take
+     * sibling_activation; weights, bias and per-feature factors are the two convolutions' concatenated.  In
+     * fs_b_yx_fsv16 the second convolution's result is the contiguous tail of the output buffer (feature slices are the
+     * outermost axis), so a reader takes it as a tensor of its own.  Needs a multiple of 16, one group, the quantized
+     * non-fused form; not for fully_connected.  The reference enqueues the two primitives one after the other
+     * (src/gpu/primitive_gpu_base.h:117-168); the results per feature are the same. */
+    int32_t sibling_split;
+    int32_t sibling_activation;
+    float sibling_activation_m, sibling_activation_n;
 } cldnn_hip_conv_desc;
 
 /* Host pointers: weights [ofm][ifm/groups][fy][fx] dense, bias/wqf/calib/eltw_calib [ofm] or NULL.

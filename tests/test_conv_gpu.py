@@ -677,3 +677,68 @@ def test_grouped_convolution_on_the_matrix_core_kernels(eng, shape, in_dt):
     # plain layouts keep the one-thread-per-output kernel
     _, (go, ga, info) = both(eng, x, w, bias, wqf, calib, fmt="bfyx", stride=(1, 1), pad=(pad, pad), groups=G, out_dt="s8", act="relu")
     assert info.impl == hip.IMPL_REF
+
+
+# two convolutions of the same input in one launch (a block's shortcut projection and its opening 1x1): every output
+# feature must equal what its own convolution gives alone
+SIBLINGS = [
+    # B, IFM, H, W, OFM of the first, OFM of the second, filter, stride, padding
+    (2, 64, 14, 14, 256, 64, 1, 1, 0),
+    (2, 256, 14, 14, 128, 64, 1, 2, 0),
+    (1, 128, 9, 9, 64, 48, 3, 1, 1),
+    (3, 64, 7, 7, 80, 24, 1, 1, 0),    # a last feature slice that is partly filled
+]
+
+
+@pytest.mark.parametrize("acts", [("none", "relu"), ("relu", "none"), ("relu", "relu"), ("none", "none"), ("relu_slope", "relu"),
+                                  ("none", "clamp")], ids=lambda a: "-".join(a))
+@pytest.mark.parametrize("shape", SIBLINGS, ids=lambda s: "x".join(map(str, s)))
+@pytest.mark.parametrize("in_dt", [np.uint8, np.int8], ids=["u8", "s8"])
+def test_two_convolutions_of_one_input_in_one_launch(eng, shape, acts, in_dt):
+    B, IFM, H, W, F1, F2, FK, stride, pad = shape
+    x, w, bias, wqf, calib = problem(77, B, IFM, H, W, F1 + F2, FK, FK, in_dt)
+    par = {"none": (0.0, 0.0), "relu": (0.0, 0.0), "relu_slope": (0.25, 0.0), "clamp": (-3000.0, 2500.0)}
+    kw = dict(stride=(stride, stride), pad=(pad, pad), out_dt="s8")
+    halves = []
+    for (lo, hi), act in zip(((0, F1), (F1, F1 + F2)), acts):
+        halves.append(rc.conv(x, w[lo:hi], bias[lo:hi], wqf=wqf[lo:hi], calib=calib[lo:hi], act=act, act_m=par[act][0],
+                              act_n=par[act][1], **kw))
+    ref = np.concatenate(halves, axis=1)
+    short = all(a in ("none", "relu") for a in acts)
+    names = tile_names()
+    rows = [0] + [i + 1 for i, n in enumerate(names) if n in ("p64_f64", "bdir_p64_f64", "wsl_p64", "stream_p32", "bdir_k2_p64_f64")]
+    seen = set()
+    for tile in rows:
+        args = dict(fmt="fs_b_yx_fsv16", in_pad=(pad, pad), tile=tile, want_info=True, act=acts[0], act_m=par[acts[0]][0],
+                    act_n=par[acts[0]][1], sibling_split=F1, sibling_act=acts[1], **kw)
+        d_extra = dict(sibling_act_m=par[acts[1]][0], sibling_act_n=par[acts[1]][1])
+        try:
+            got, info = hip.conv_forward(eng, x, w, bias, wqf, calib, **args, **d_extra)
+        except hip.HipError:
+            assert tile != 0  # a forced row that does not fit the shape
+            continue
+        name = info.kernel_name.decode()
+        seen.add(name)
+        assert ("generic" in name) == (not short), name
+        assert_same(ref, got)
+    assert seen
+    # negative output factors under a relu: the clamp form does not apply, the element-wise epilogue takes over
+    if acts == ("none", "relu"):
+        calib2 = calib.copy()
+        calib2[F1 + 3] *= -1
+        ref2 = ref.copy()
+        ref2[:, F1 + 3] = rc.conv(x, w[F1 + 3:F1 + 4], bias[F1 + 3:F1 + 4], wqf=wqf[:1], calib=calib2[F1 + 3:F1 + 4], act="relu", **kw)[:, 0]
+        got, info = hip.conv_forward(eng, x, w, bias, wqf, calib2, fmt="fs_b_yx_fsv16", in_pad=(pad, pad), want_info=True, act="none",
+                                     sibling_split=F1, sibling_act="relu", **kw)
+        assert b"generic" in info.kernel_name
+        assert_same(ref2, got)
+
+
+def test_sibling_split_is_validated(eng):
+    x, w, bias, wqf, calib = problem(5, 1, 64, 6, 6, 96, 1, 1)
+    for bad in (8, 96, 100, -16):
+        with pytest.raises(hip.HipError):
+            hip.conv_forward(eng, x, w, bias, wqf, calib, fmt="fs_b_yx_fsv16", out_dt="s8", sibling_split=bad, sibling_act="relu")
+    e = np.zeros((1, 96, 6, 6), np.int8)
+    with pytest.raises(hip.HipError):  # not together with a fused second input
+        hip.conv_forward(eng, x, w, bias, wqf, calib, fmt="fs_b_yx_fsv16", out_dt="s8", sibling_split=32, sibling_act="relu", eltw=e)

@@ -30,6 +30,9 @@ EXPECTED = {
     ("resnet50_b32_fused", "res4a_branch2b"): "conv_bdir<bdir_p64_f64",
     ("resnet50_b32_fused", "res4a_branch2c"): "conv_wsl<wsl_p128",
     ("resnet50_b32_fused", "res5a_branch2b"): "conv_bdir<bdir_k2_p64_f64",
+    ("resnet50_b32_fused", "res2a_branch1|1"): "conv_stream<stream_p32",
+    ("resnet50_b32_fused", "res4a_branch1|1"): "conv_mfma<p64_f128",
+    ("resnet50_b32_fused", "res5a_branch1|1"): "conv_mfma<p64_f128",
     ("vgg16_b16", "conv6"): "conv_mfma<p256_f128",
     ("vgg16_b16", "conv9"): "conv_bdir<bdir_p128_f128",
     ("mobilenet_v2_b32", "b2_dw"): "conv_dwchain<3 stages",
@@ -53,6 +56,10 @@ def cases():
                 continue
             seen.add(s)
             out.append(pytest.param(wl, [dict(l) for l in g], id="%s-%s" % (wl, g[0]["name"] + ("+%d" % (len(g) - 1) if len(g) > 1 else ""))))
+        # two convolutions of one input in one launch (a projection and the block's opening 1x1)
+        for a, b in zip(layers, layers[1:]):
+            if b.get("shares_input") and not (fuse and (a["closes_block"] or b["closes_block"])):
+                out.append(pytest.param(wl, [dict(a), dict(b)], id="%s-%s|1" % (wl, a["name"])))
     return out
 
 
@@ -70,7 +77,10 @@ def test_layer_at_its_real_batch_matches_the_oracle(eng, wl, group):
     head = stack[0]
     name = head.info.kernel_name.decode()
     assert not name.startswith("conv_ref"), name  # every layer of the configurations runs on a fast kernel
-    want = EXPECTED.get((wl, group[0]["name"]))
+    pair = len(group) == 2 and bool(group[1].get("shares_input"))
+    if pair and batch > 1:
+        assert head.sibling is stack[1], "the two convolutions of one input run as two launches"
+    want = EXPECTED.get((wl, group[0]["name"] + ("|1" if pair else "")))
     if want:
         assert name.startswith(want), "%s runs on %s, the profile shows %s" % (group[0]["name"], name, want)
     bench.run_step(bench.launches(stack))

@@ -780,3 +780,68 @@ def test_copy_region_between_layouts():
     np.testing.assert_array_equal(hip.download(e, dst), want)
     assert hip.lib().cldnn_hip_copy_region(e.h, src.ptr, C.byref(src.tensor), dst.ptr, C.byref(dst.tensor), 1, 22, 2, 1) == -7  # does not fit
     src.close(), dst.close(), e.close()
+
+
+def projection_block(eng, seed, B=2, C=64, M=32, H=14, W=14, stride=2):
+    """a down-sampling ResNet block: the shortcut projection (1x1, no activation) and the opening 1x1 (relu) read the same
+    tensor with the same stride -> 3x3 -> 1x1 expand + projection, relu"""
+    r = np.random.default_rng(seed)
+    x = r.integers(-128, 128, (B, C, H, W)).astype(np.int8)
+    O = 4 * M
+    L = [rand_layer(r, O, C, 1, False), rand_layer(r, M, C, 1, False), rand_layer(r, M, M, 3, False), rand_layer(r, O, M, 1, False)]
+    ecal = r.uniform(0.4, 0.9, O).astype(np.float32)
+    prims = [cl.input_layout("input", cl.layout(DT.i8, F.bfyx, cl.tensor(B, C, W, H)))]
+    for i, (w, b, q, c) in enumerate(L):
+        prims += [cl.data(f"w{i}", cl.make_memory(eng, w)), cl.data(f"b{i}", vec_mem(eng, b)), cl.data(f"q{i}", vec_mem(eng, q)),
+                  cl.data(f"c{i}", vec_mem(eng, c))]
+    st = cl.tensor(1, 1, stride, stride)
+    prims += [cl.data("ecal", vec_mem(eng, ecal)),
+              cl.convolution("shortcut", "input", ["w0"], ["b0"], ["q0"], ["c0"], stride=st),
+              cl.convolution("reduce", "input", ["w1"], ["b1"], ["q1"], ["c1"], stride=st, with_activation=True),
+              cl.convolution("mid", "reduce", ["w2"], ["b2"], ["q2"], ["c2"], input_offset=cl.tensor(0, 0, -1, -1, 0), with_activation=True),
+              cl.convolution("expand", "mid", ["w3"], ["b3"], ["q3"], ["c3"], output_data_type=DT.i8),
+              cl.eltwise("sum", "shortcut", "expand", cl.eltwise_mode.sum, True, 0.0, output_calibration_factors="ecal"),
+              cl.reorder("out", "sum", F.bfyx)]
+
+    def oracle():
+        s = (stride, stride)
+        sc = rc.conv(x, L[0][0], L[0][1], wqf=L[0][2], calib=L[0][3], stride=s, out_dt="s8")
+        a = rc.conv(x, L[1][0], L[1][1], wqf=L[1][2], calib=L[1][3], stride=s, out_dt="s8", act="relu")
+        a = rc.conv(a, L[2][0], L[2][1], wqf=L[2][2], calib=L[2][3], pad=(1, 1), out_dt="s8", act="relu")
+        return sc, rc.conv(a, L[3][0], L[3][1], wqf=L[3][2], calib=L[3][3], out_dt="s8", eltw=sc, eltw_act="relu", eltw_calib=ecal)
+
+    return cl.topology(*prims), x, oracle
+
+
+@pytest.mark.parametrize("optimize", OPT, ids=["plain", "optimize_data"])
+@pytest.mark.parametrize("stride", [1, 2])
+def test_projection_and_opening_convolution_share_a_launch(eng, optimize, stride):
+    topo, x, oracle = projection_block(eng, 21, stride=stride)
+    net, outs = run(eng, topo, {"input": cl.make_memory(eng, x)}, optimize)
+    sc, expected = oracle()
+    np.testing.assert_array_equal(outs["out"].get_memory().read(), expected)
+    a, b = net.get_primitive_info("shortcut"), net.get_primitive_info("reduce")
+    if optimize:
+        # one launch for the two convolutions of `input`; `reduce` is the tail of the pair's buffer and both carry the
+        # border the 3x3 behind `reduce` needs
+        assert a["launches_also"] == "reduce" and b["launched_by"] == "shortcut" and "kernel" not in b
+        assert "generic" not in a["kernel"]
+        assert a["pad_lower"][2:] == [1, 1] and b["pad_lower"][2:] == [1, 1]
+        for _ in range(2):  # again, same buffers
+            np.testing.assert_array_equal(net.execute()["out"].get_memory().read(), expected)
+    else:
+        assert "launches_also" not in a and "launched_by" not in b
+
+
+def test_paired_convolution_that_is_an_output(eng):
+    """what the application reads is the reorder back to its own format, which takes the convolution's window of the pair's
+    buffer like any other reader"""
+    topo, x, oracle = projection_block(eng, 22, stride=1)
+    net = cl.network(eng, topo, cl.build_options(optimize_data=True, outputs=["shortcut", "reduce", "out"]))
+    net.set_input_data("input", cl.make_memory(eng, x))
+    outs = net.execute()
+    sc, expected = oracle()
+    np.testing.assert_array_equal(outs["out"].get_memory().read(), expected)
+    np.testing.assert_array_equal(outs["shortcut"].get_memory().read(), sc)
+    assert outs["reduce"].get_memory().read().min() == 0  # relu on the second convolution only
+    assert sc.min() < 0

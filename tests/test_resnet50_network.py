@@ -141,6 +141,10 @@ def test_memory_pool_shares_buffers_without_changing_results():
         if pool:
             assert followers == ["res2a_branch2c_fused_res2a", "res2b_branch2a", "res2b_branch2c_fused_res2b", "res2c_branch2a"], followers
             assert kernels["res2a_branch2b"].startswith("conv_chain<3 stages") and kernels["res2b_branch2a"] == "in the chain of res2a_branch2b"
+        # a projection block's shortcut convolution and its opening 1x1 read the same tensor: one launch for the two
+        # (not where the closer writes over the shortcut, which then needs a buffer of its own)
+        paired = sorted(i for i in net.get_all_primitive_ids() if "launched_by" in net.get_primitive_info(i))
+        assert paired == (["res%da_branch2a" % s for s in (2, 3, 4, 5)] if pool else []), paired
         net.set_input_data("input", cl.make_memory(eng, x))
         for _ in range(2):  # a second run reuses the same buffers
             logits[pool] = net.execute()["fc1000"].get_memory().read()
@@ -151,9 +155,10 @@ def test_memory_pool_shares_buffers_without_changing_results():
     # 26 MB of either figure are weights; without a pool the 13 closers that write over their shortcuts save nearly as
     # much as the pool does.  With the pool the two convolution chains of stage 2 (pooled engines only: a closer that
     # writes over its shortcut is not chained) cost one 64-feature tensor each, because a chain's last member is written
-    # by the launch that still reads the head's input and cannot take that buffer over: at this batch the two figures
-    # meet within a percent
-    assert max(used.values()) < 40e6 and used[True] < 1.01 * used[False], used
+    # by the launch that still reads the head's input and cannot take that buffer over; and the four buffers that hold a
+    # projection together with the block's opening 1x1 have layouts nothing else in the network has, so they are never
+    # taken over (4 MB at this batch)
+    assert max(used.values()) < 43e6 and used[True] < 1.12 * used[False], used
 
 
 @pytest.mark.gpu
