@@ -58,8 +58,10 @@ static const TileConfig g_tiles[] = {
     // few pixels, long K (fully_connected): a workgroup owns one 16-feature fragment of a 64-feature tile and 16
     // pixels; its waves split K and stream both operands straight from global memory
     {"gemv_p16_f16", 16, 64, 16},
+    // first layers with several K-steps (a 7x7 filter): 64 pixels per wave, so the weights are fetched half as often
+    {"stem_p64", 64, 64, 64},
 };
-enum { FIRST_STREAM_ROW = 6, FIRST_BDIR_ROW = 8, FIRST_WSL_ROW = 14, FIRST_BDIRK_ROW = 17, STEM_ROW = 20, GEMV_ROW = 21 };
+enum { FIRST_STREAM_ROW = 6, FIRST_BDIR_ROW = 8, FIRST_WSL_ROW = 14, FIRST_BDIRK_ROW = 17, STEM_ROW = 20, GEMV_ROW = 21, STEM_P64_ROW = 22 };
 enum { WSL_MAX_LDS = 160 * 1024 };
 enum { MFMA_SLACK_STEPS = 40 };  // >= weight look-ahead + activation look-ahead + 3
 static const tile_launcher g_launch[] = {launch_mfma_tile_0, launch_mfma_tile_1, launch_mfma_tile_2, launch_mfma_tile_3,
@@ -104,7 +106,7 @@ enum {
     ROW_STREAM_P16 = 6, ROW_STREAM_P32 = 7,
     ROW_BDIR_P64_F64 = 8, ROW_BDIR_P128_F64 = 9, ROW_BDIR_P256_F64 = 10, ROW_BDIR_P64_F128 = 11, ROW_BDIR_P128_F128 = 12,
     ROW_BDIR_P256_F128 = 13, ROW_WSL_P64 = 14, ROW_WSL_P128 = 15, ROW_WSL_P256 = 16,
-    ROW_BDIR_K2_P64_F64 = 17, ROW_BDIR_K4_P64_F64 = 18, ROW_BDIR_K2_P128_F64 = 19, ROW_STEM_P32 = 20, ROW_GEMV = 21
+    ROW_BDIR_K2_P64_F64 = 17, ROW_BDIR_K4_P64_F64 = 18, ROW_BDIR_K2_P128_F64 = 19, ROW_STEM_P32 = 20, ROW_GEMV = 21, ROW_STEM_P64 = 22
 };
 
 static int choose_lds_tile(const ConvProblem& p, int64_t m, int cus)
@@ -126,7 +128,8 @@ static int choose_lds_tile(const ConvProblem& p, int64_t m, int cus)
 
 int mfma_choose(const ConvProblem& p, int cus)
 {
-    if (p.in_t.format == CLDNN_HIP_FMT_B_FS_YX_FSV4) return ROW_STEM_P32;
+    if (p.in_t.format == CLDNN_HIP_FMT_B_FS_YX_FSV4)
+        return p.FY * ((p.FX + 3) / 4) > 8 ? ROW_STEM_P64 : ROW_STEM_P32;  // more than two K-steps of four 4-tap chunks
     const int64_t m = (int64_t)p.B * p.OH * p.OW;
     const int cb = (p.IFM + 15) / 16;
     const int ksteps = (p.FY * p.FX * cb + 3) / 4;
@@ -198,7 +201,7 @@ MfmaPlan mfma_plan(const ConvProblem& p, int tile, int cus)
     MfmaPlan pl{};
     pl.tile = tile;
     pl.checked = border_covers(p) ? 0 : 1;
-    pl.stem = tile == STEM_ROW ? 1 : 0;
+    pl.stem = tile == STEM_ROW || tile == STEM_P64_ROW ? 1 : 0;
     CHIP_REQUIRE(pl.stem == (p.in_t.format == CLDNN_HIP_FMT_B_FS_YX_FSV4 ? 1 : 0), CLDNN_HIP_INVALID_ARG,
                  "b_fs_yx_fsv4 input goes with the first-layer row of the tile table and only with it");
     pl.stream = (tile >= FIRST_STREAM_ROW && tile < FIRST_BDIR_ROW) || pl.stem ? 1 : 0;

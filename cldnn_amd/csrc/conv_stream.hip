@@ -1,5 +1,5 @@
 // Instances of the streaming (LDS-free) int8 MFMA convolution kernel:
-// 16 or 32 pixels per tile x 1, 2, 4 or 8 K-steps.
+// 16, 32 or 64 pixels per tile x 1, 2, 4 or 8 K-steps.
 #include "conv_mfma_kernel.h"
 
 namespace chip {
@@ -20,7 +20,8 @@ void launch_stream(hipStream_t s, const MfmaArgs& a, int nt, int grid, int epi)
 {
     if (nt == 1) by_ksteps<1>(s, a, a.ksteps, grid, epi);
     else if (nt == 2) by_ksteps<2>(s, a, a.ksteps, grid, epi);
-    else throw error(CLDNN_HIP_INVALID_ARG, "streaming kernel: pixels per tile must be 16 or 32");
+    else if (nt == 4) by_ksteps<4>(s, a, a.ksteps, grid, epi);
+    else throw error(CLDNN_HIP_INVALID_ARG, "streaming kernel: pixels per tile must be 16, 32 or 64");
 }
 
 }  // namespace chip

@@ -23,7 +23,7 @@ CONFIGS = {  # workload -> (layers, batch, residual fused, images compared)
 
 # kernels the per-layer tables under profiles/ show for these layers (kernel family and row of the tile table)
 EXPECTED = {
-    ("resnet50_b32_fused", "conv1"): "conv_stream<stem_p32",
+    ("resnet50_b32_fused", "conv1"): "conv_stream<stem_p64",
     ("resnet50_b32_fused", "res2a_branch2b"): "conv_chain<3 stages",
     ("resnet50_b32_fused", "res2c_branch2b"): "conv_chain<2 stages",
     ("resnet50_b32_fused", "res3a_branch2b"): "conv_bdir<bdir_p128_f64",

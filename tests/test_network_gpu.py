@@ -515,7 +515,7 @@ def test_first_layer_through_network(eng):
     for optimize in OPT:
         net, outs = run(eng, topo, {"input": cl.make_memory(eng, x)}, optimize)
         np.testing.assert_array_equal(outs["stem"].get_memory().read(), expected)
-    assert "stem_p32" in net.get_primitive_info("stem_fsv16")["kernel"]
+    assert "stem_p" in net.get_primitive_info("stem_fsv16")["kernel"]
     assert net.get_primitive_info("input_to_fsv4_0")["format"] == F.b_fs_yx_fsv4
 
 
