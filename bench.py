@@ -177,8 +177,6 @@ def build_stack(eng, layers, batch, fuse_residual, seed=1337, tile=0, in_dt=np.u
             M.follows, M.xin_from = False, out[i + n - 1]
             if want - n > 1:
                 M.spec = dict(M.spec, chain_len=want - n)
-            if n == 1:
-                log("bench.py: %s does not head a chain on this device, it runs alone" % L.spec["name"])
         i += n
     # two convolutions of one input in one launch, where the library has a short epilogue for the pair
     for H, M in zip(out, out[1:]):
