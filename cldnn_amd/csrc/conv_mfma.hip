@@ -160,6 +160,8 @@ int mfma_choose(const ConvProblem& p, int cus)
     }
     // long K
     if (m >= 50000) {
+        // 256 and more features: 64 pixels x 128 features per wave, two waves per SIMD (3x3 at 56x56 with 128 / 256 input features)
+        if (p.OFM >= 256 && p.OFM % 128 == 0) return ROW_BDIR_P256_F128;
         if (ksteps <= 18) return ksteps <= 9 && p.OFM <= 128 ? ROW_WSL_P128 : ROW_WSL_P64;  // 3x3 at 56x56 .. 112x112
         return p.OFM >= 128 ? ROW_P256_F128 : ROW_BDIR_P256_F64;
     }

@@ -664,6 +664,12 @@ __global__ void __launch_bounds__(256 * KG) conv_bdir_kernel(MfmaArgs a)
     constexpr int WP = NT * 16;       // pixels per wave
     constexpr int BM = 4 * WP;        // pixels per workgroup
     constexpr int A_LOADS = BN / 64;  // 16-byte weight chunks per thread per K-step
+    // 64 pixels x 128 features per wave: 128 accumulators.  It is the smallest wave tile that leaves both operand paths
+    // half empty at full matrix rate (LDS delivers 4096 / pixels bytes per clock, the vector memory path 4096 / features),
+    // but only with two waves per SIMD: one wave's own instruction stream does not hide its LDS reads.  To stay under 256
+    // registers the look-ahead is three steps and the weight fragments of a step are read when the step starts instead
+    // of one step early (the other wave covers the wait).
+    constexpr bool LEAN = BN == 128 && NT == 4 && KG == 1;
 
     // KG groups of four waves split the K-steps of the tile between them and add their partial sums through
     // LDS at the end: long-K layers with few pixels get KG times as many waves per tile to hide latencies with.
@@ -711,7 +717,7 @@ __global__ void __launch_bounds__(256 * KG) conv_bdir_kernel(MfmaArgs a)
     const v4i* wsrc = a.wpk + ((size_t)ntile * a.ksteps + step0) * (4 * BN) + t;
 
     // look-ahead in K-steps for both operands
-    constexpr int D = BDIR_PREFETCH_DISTANCE(A_LOADS + NT);
+    constexpr int D = LEAN ? 3 : BDIR_PREFETCH_DISTANCE(A_LOADS + NT);
     constexpr int DA = D;
     v4i ra[DA][A_LOADS], rb[D][NT];
     auto load_a = [&](int ks, v4i (&xa)[A_LOADS]) {
@@ -759,11 +765,45 @@ __global__ void __launch_bounds__(256 * KG) conv_bdir_kernel(MfmaArgs a)
     load_a(DA, ra[0]);
     load_a(DA + 1, ra[1]);
     lds_barrier();
+    int b1 = 1, b2 = 2, b0 = 0;  // ring positions of steps k+1, k+2, k
+    const int main_steps = (steps / DA) * DA;
+    if constexpr (LEAN) {
+        v4i fa[MT], fb[NT];
+        const int lean_main = (steps / D) * D;
+        for (int ks0 = 0; ks0 < lean_main; ks0 += D) {
+#pragma unroll
+            for (int u = 0; u < D; ++u) {
+                const int ks = ks0 + u;
+                read_a(b0, fa);
+                flip(rb[u], fb);
+                mma(fa, fb);
+                store_a(b2, ra[(u + 2) % DA]);
+                load_a(ks + 2 + DA, ra[(u + 2) % DA]);
+                load_b(ks + D, rb[u]);
+                lds_barrier();
+                step_fence();
+                const int tmp = b0;
+                b0 = b1, b1 = b2, b2 = tmp;
+            }
+        }
+        const int rest = steps - lean_main;
+#pragma unroll
+        for (int u = 0; u < D - 1; ++u) {
+            if (u < rest) {
+                read_a(b0, fa);
+                flip(rb[u], fb);
+                mma(fa, fb);
+                store_a(b2, ra[(u + 2) % DA]);
+                lds_barrier();
+                step_fence();
+                const int tmp = b0;
+                b0 = b1, b1 = b2, b2 = tmp;
+            }
+        }
+    } else {
     v4i fa_cur[MT], fa_nxt[MT], fb_cur[NT], fb_nxt[NT];
     read_a(0, fa_cur);
     flip(rb[0], fb_cur);
-    int b1 = 1, b2 = 2, b0 = 0;  // ring positions of steps k+1, k+2, k
-    const int main_steps = (steps / DA) * DA;
     for (int ks0 = 0; ks0 < main_steps; ks0 += DA) {
 #pragma unroll
         for (int u = 0; u < DA; ++u) {
@@ -804,6 +844,7 @@ __global__ void __launch_bounds__(256 * KG) conv_bdir_kernel(MfmaArgs a)
             const int tmp = b0;
             b0 = b1, b1 = b2, b2 = tmp;
         }
+    }
     }
 
     keep_until_here(early);

@@ -33,7 +33,7 @@ EXPECTED = {
     ("resnet50_b32_fused", "res2a_branch1|1"): "conv_stream<stream_p32",
     ("resnet50_b32_fused", "res4a_branch1|1"): "conv_mfma<p64_f128",
     ("resnet50_b32_fused", "res5a_branch1|1"): "conv_mfma<p64_f128",
-    ("vgg16_b16", "conv6"): "conv_mfma<p256_f128",
+    ("vgg16_b16", "conv6"): "conv_bdir<bdir_p256_f128",
     ("vgg16_b16", "conv9"): "conv_bdir<bdir_p128_f128",
     ("mobilenet_v2_b32", "b2_dw"): "conv_dwchain<3 stages",
     ("mobilenet_v2_b32", "b17_dw"): "conv_dw3x3_kernel",
