@@ -756,14 +756,34 @@ __global__ void __launch_bounds__(256 * KG) conv_bdir_kernel(MfmaArgs a)
     // pass through a ring of three LDS buffers, written two steps ahead of their use, so that the fragments of
     // step k+1 are read from LDS while the matrix instructions of step k run (one barrier per step).  The loop
     // is branch-free; the weight stream and the tap table carry zero slack for the steps requested past the end.
+    if constexpr (LEAN) {
+        // The requests go out in the order the loop issues them (weights of step k + 2, activations of step k), each
+        // group pinned: the wait at the head of the loop is computed over this path too, and if the scheduler moves one
+        // fragment of step 0 to the end of the queue that wait becomes "everything but one", once per trip of the loop.
+        load_a(0, ra[0]);
+        load_a(1, ra[1]);
+        step_fence();
+        load_a(2, ra[2]);
+        load_b(0, rb[0]);
+        step_fence();
+        store_a(0, ra[0]);
+        store_a(1, ra[1]);
+        load_a(3, ra[0]);
+        load_b(1, rb[1]);
+        step_fence();
+        load_a(4, ra[1]);
+        load_b(2, rb[2]);
+        step_fence();
+    } else {
 #pragma unroll
-    for (int u = 0; u < DA; ++u) load_a(u, ra[u]);
+        for (int u = 0; u < DA; ++u) load_a(u, ra[u]);
 #pragma unroll
-    for (int d = 0; d < D; ++d) load_b(d, rb[d]);
-    store_a(0, ra[0]);
-    store_a(1, ra[1]);
-    load_a(DA, ra[0]);
-    load_a(DA + 1, ra[1]);
+        for (int d = 0; d < D; ++d) load_b(d, rb[d]);
+        store_a(0, ra[0]);
+        store_a(1, ra[1]);
+        load_a(DA, ra[0]);
+        load_a(DA + 1, ra[1]);
+    }
     lds_barrier();
     int b1 = 1, b2 = 2, b0 = 0;  // ring positions of steps k+1, k+2, k
     const int main_steps = (steps / DA) * DA;
