@@ -59,7 +59,7 @@ def chain_groups(layers, fuse_residual):
     return out
 
 
-def build_stack(eng, layers, batch, fuse_residual, seed=1337, tile=0, in_dt=np.uint8, chains=True, siblings=None):
+def build_stack(eng, layers, batch, fuse_residual, seed=1337, tile=0, in_dt=np.uint8, chains=True, siblings=None, calibration="benchmark"):
     """Create device tensors and convolution objects for every layer (seeded synthetic data).
 
     chains: neighbouring layers that feed each other in the network (follows_prev) run as ONE launch of the
@@ -68,7 +68,10 @@ def build_stack(eng, layers, batch, fuse_residual, seed=1337, tile=0, in_dt=np.u
     result of a chain's first stage, which only the second stage reads, is never written.
     siblings (default: as chains): a layer that reads the same tensor as the one before it (shares_input: a block's
     opening 1x1 beside the shortcut projection) runs in that layer's launch; its result is the tail of the launch's
-    output buffer.  Such a layer reads the same input data as its neighbour either way."""
+    output buffer.  Such a layer reads the same input data as its neighbour either way.
+    calibration: "benchmark" = the baseline's factors, log-uniform in [1e-4, 1e-2] (most outputs end at 0 or 127);
+    "spread" = 40 / sigma(accumulator) * U(0.5, 2) per feature, which spreads the outputs over the int8 range so that a
+    wrong accumulator shows in the output (parity tests)."""
     siblings = chains if siblings is None else siblings
     out = []
     follows = set()  # indices of layers that run as stage 1 / 2 of a chain
@@ -100,6 +103,8 @@ def build_stack(eng, layers, batch, fuse_residual, seed=1337, tile=0, in_dt=np.u
         L.bias = r.integers(-1000, 1001, ofm).astype(np.int32)
         L.wqf = np.ones(ofm, np.float32)
         L.calib = np.exp(r.uniform(np.log(1e-4), np.log(1e-2), ofm)).astype(np.float32)
+        if calibration == "spread":
+            L.calib = (40.0 / (np.sqrt((ifm // g) * k * k) * 147.4 * 73.3) * r.uniform(0.5, 2.0, ofm)).astype(np.float32)
         L.fused = bool(fuse_residual and l["closes_block"])
         L.eltw = L.ecal = None
         act = l["act"]

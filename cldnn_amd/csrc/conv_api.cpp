@@ -1,6 +1,7 @@
 // Convolution objects of the C-ABI: validation, arithmetic-mode selection, kernel-family and
 // tile choice (the gfx950 tile-config table stands where the reference has kernel_selector and
 // its tuning cache), weight pre-packing, launch.
+#include <algorithm>
 #include <cstring>
 #include <vector>
 
@@ -294,8 +295,8 @@ void build(cldnn_hip_conv c, const void* weights, const void* bias, const float*
         if (const size_t g = mfma_gather_bytes(p, c->mplan)) c->gather = upload(c, nullptr, 0, g);
         const TileConfig& tc = tile_config(tile);
         inf.tile_index = tile, inf.tile_pixels = tc.tile_pixels, inf.tile_ofm = tc.tile_ofm;
-        inf.grid = c->mplan.grid, inf.block = c->mplan.gemv ? 64 * c->mplan.gemv_waves : 256, inf.lds_bytes = c->mplan.lds_bytes;
-        std::snprintf(inf.kernel_name, sizeof(inf.kernel_name), "conv_%s<%s,%s,%s>", c->mplan.gemv ? "gemv" : c->mplan.stream ? "stream" : (c->mplan.bdir ? "bdir" : (c->mplan.wsl ? "wsl" : "mfma")),
+        inf.grid = c->mplan.grid, inf.block = c->mplan.gemv ? 64 * c->mplan.gemv_waves : c->mplan.block, inf.lds_bytes = c->mplan.lds_bytes;
+        std::snprintf(inf.kernel_name, sizeof(inf.kernel_name), "conv_%s<%s,%s,%s>", c->mplan.gemv ? "gemv" : c->mplan.halo ? "halo" : c->mplan.stream ? "stream" : (c->mplan.bdir ? "bdir" : (c->mplan.wsl ? "wsl" : "mfma")),
                       tc.name, c->mplan.checked ? "checked" : "border", c->fast && !c->mplan.gemv ? "fast" : "generic");
     } else {
         c->dplan = dw_plan(p);
@@ -384,7 +385,7 @@ static void run(cldnn_hip_conv c, const void* in, void* out, const void* eltw, i
             CHIP_REQUIRE(need <= mfma_static_scratch_bytes(), CLDNN_HIP_UNSUPPORTED_SIZE,
                          "this convolution gathers " + std::to_string(need) + " bytes of activations, the static scratch holds "
                              + std::to_string(mfma_static_scratch_bytes()));
-            if (need) wb.gather = mfma_static_scratch(c->engine->device);
+            if (need) wb.gather = c->engine->static_scratch;
         }
         if (raw)
             launch_conv_mfma(s, p, c->mplan, wb, (const int32_t*)c->acc_init_raw, c->epi, nullptr, in, nullptr, nullptr, raw);
@@ -465,6 +466,17 @@ cldnn_hip_status cldnn_hip_conv_chain_create(cldnn_hip_engine e, int32_t count, 
                                       wqf ? wqf[k] : nullptr};
             }
             chain_pack_weights(ch->in, ch->plan, cus, w8, vec, packed.data());
+            // The chain launches none of its stage objects (they never leave this file): their own operand streams (packed weights, tap table, gather
+            // scratch) would only hold every chained layer's weights on the device a second time.
+            for (int k = 0; k < count; ++k) {
+                cldnn_hip_conv c = ch->stage[k];
+                for (void** buf : {&c->w_packed, &c->ktab, &c->gather}) {
+                    if (!*buf) continue;
+                    c->owned.erase(std::remove(c->owned.begin(), c->owned.end(), *buf), c->owned.end());
+                    CHIP_CHECK(hipFree(*buf));
+                    *buf = nullptr;
+                }
+            }
             CHIP_CHECK(hipMalloc(&ch->packed, packed.size()));
             CHIP_CHECK(hipMemcpyAsync(ch->packed, packed.data(), packed.size(), hipMemcpyHostToDevice, e->stream));
             CHIP_CHECK(hipStreamSynchronize(e->stream));

@@ -4,7 +4,7 @@
 #include <cmath>
 #include <cstring>
 
-#include "conv_mfma_kernel.h"
+#include "conv_halo_kernel.h"
 
 namespace chip {
 
@@ -23,6 +23,7 @@ void* gemv_static_scratch(int device);
 #define DECL_WSL(d) void launch_wsl_d##d(hipStream_t s, const MfmaArgs& a, int nt, int grid, int lds, int epi);
 DECL_WSL(1) DECL_WSL(2) DECL_WSL(3) DECL_WSL(4) DECL_WSL(6) DECL_WSL(8)
 #undef DECL_WSL
+void launch_halo(hipStream_t s, const HaloArgs& h, int row, int pl, int grid, int lds, int epi);
 
 typedef void (*tile_launcher)(hipStream_t, const MfmaArgs&, int, int, bool, int);
 
@@ -60,8 +61,15 @@ static const TileConfig g_tiles[] = {
     {"gemv_p16_f16", 16, 64, 16},
     // first layers with several K-steps (a 7x7 filter): 64 pixels per wave, so the weights are fetched half as often
     {"stem_p64", 64, 64, 64},
+    // nine-tap stride-1 kernel with both operands in LDS (direct global -> LDS loads); persistent workgroups; a wave
+    // owns 64 positions x 128 features.  tile_pixels counts positions of the bordered input.
+    {"halo_p256_f128", 256, 128, 64},   // 4 waves
+    {"halo_p128_f128", 128, 128, 64},   // 2 waves
+    {"halo_p128_f256", 128, 256, 64},   // 4 waves, 2 x 2
+    {"halo_p256_f256", 256, 256, 64},   // 8 waves, 4 x 2
 };
-enum { FIRST_STREAM_ROW = 6, FIRST_BDIR_ROW = 8, FIRST_WSL_ROW = 14, FIRST_BDIRK_ROW = 17, STEM_ROW = 20, GEMV_ROW = 21, STEM_P64_ROW = 22 };
+enum { FIRST_STREAM_ROW = 6, FIRST_BDIR_ROW = 8, FIRST_WSL_ROW = 14, FIRST_BDIRK_ROW = 17, STEM_ROW = 20, GEMV_ROW = 21, STEM_P64_ROW = 22, FIRST_HALO_ROW = 23 };
+enum { HALO_RING = 4, HALO_TAPS = 9 };
 enum { WSL_MAX_LDS = 160 * 1024 };
 enum { MFMA_SLACK_STEPS = 40 };  // >= weight look-ahead + activation look-ahead + 3
 static const tile_launcher g_launch[] = {launch_mfma_tile_0, launch_mfma_tile_1, launch_mfma_tile_2, launch_mfma_tile_3,
@@ -106,7 +114,8 @@ enum {
     ROW_STREAM_P16 = 6, ROW_STREAM_P32 = 7,
     ROW_BDIR_P64_F64 = 8, ROW_BDIR_P128_F64 = 9, ROW_BDIR_P256_F64 = 10, ROW_BDIR_P64_F128 = 11, ROW_BDIR_P128_F128 = 12,
     ROW_BDIR_P256_F128 = 13, ROW_WSL_P64 = 14, ROW_WSL_P128 = 15, ROW_WSL_P256 = 16,
-    ROW_BDIR_K2_P64_F64 = 17, ROW_BDIR_K4_P64_F64 = 18, ROW_BDIR_K2_P128_F64 = 19, ROW_STEM_P32 = 20, ROW_GEMV = 21, ROW_STEM_P64 = 22
+    ROW_BDIR_K2_P64_F64 = 17, ROW_BDIR_K4_P64_F64 = 18, ROW_BDIR_K2_P128_F64 = 19, ROW_STEM_P32 = 20, ROW_GEMV = 21, ROW_STEM_P64 = 22,
+    ROW_HALO_P256_F128 = 23, ROW_HALO_P128_F128 = 24, ROW_HALO_P128_F256 = 25, ROW_HALO_P256_F256 = 26
 };
 
 static int choose_lds_tile(const ConvProblem& p, int64_t m, int cus)
@@ -208,14 +217,16 @@ MfmaPlan mfma_plan(const ConvProblem& p, int tile, int cus)
                  "b_fs_yx_fsv4 input goes with the first-layer row of the tile table and only with it");
     pl.stream = (tile >= FIRST_STREAM_ROW && tile < FIRST_BDIR_ROW) || pl.stem ? 1 : 0;
     pl.gemv = tile == GEMV_ROW ? 1 : 0;
-    pl.bdir = ((tile >= FIRST_BDIR_ROW && tile < FIRST_WSL_ROW) || tile >= FIRST_BDIRK_ROW) && !pl.stem && !pl.gemv ? 1 : 0;
+    pl.halo = tile >= FIRST_HALO_ROW ? 1 : 0;
+    pl.block = 256;
+    pl.bdir = ((tile >= FIRST_BDIR_ROW && tile < FIRST_WSL_ROW) || tile >= FIRST_BDIRK_ROW) && !pl.stem && !pl.gemv && !pl.halo ? 1 : 0;
     pl.wsl = tile >= FIRST_WSL_ROW && tile < FIRST_BDIRK_ROW ? 1 : 0;
     CHIP_REQUIRE(!(pl.stream && pl.checked), CLDNN_HIP_INVALID_ARG,
                  "the streaming kernel needs an input whose physical zero border covers the convolution's padding");
     pl.cb = (p.IFM + 15) / 16;
     if (pl.stem) CHIP_REQUIRE(p.IFM <= 4 && p.dx == 1 && p.groups == 1, CLDNN_HIP_INVALID_ARG,
                               "the first-layer kernel takes at most 4 input features and no horizontal dilation");
-    CHIP_REQUIRE(!(pl.bdir || pl.wsl || pl.gemv) || (!pl.checked && pl.cb % 4 == 0), CLDNN_HIP_INVALID_ARG,
+    CHIP_REQUIRE(!(pl.bdir || pl.wsl || pl.gemv || pl.halo) || (!pl.checked && pl.cb % 4 == 0), CLDNN_HIP_INVALID_ARG,
                  "the direct-activation kernels need a zero border covering the padding and input features in multiples of 64");
     pl.kchunks = pl.stem ? p.FY * ((p.FX + 3) / 4) : p.FY * p.FX * pl.cb;  // first layer: a chunk is 4 horizontal taps
     pl.ksteps = (pl.kchunks + 3) / 4;
@@ -235,15 +246,35 @@ MfmaPlan mfma_plan(const ConvProblem& p, int tile, int cus)
     // by one pixel (or one row), so most activation loads of a 3x3 filter hit in the CU's L1 instead of going to L2.
     // The weights-stationary and streaming kernels walk the taps with counters in (tap, slice) order.
     pl.tap_minor = !pl.stream && !pl.wsl && pl.cb % 4 == 0 && p.FY * p.FX > 1 ? 1 : 0;
+    if (pl.halo) {
+        const cldnn_hip_tensor& t = p.in_t;
+        CHIP_REQUIRE(p.FY * p.FX == HALO_TAPS && p.sy == 1 && p.sx == 1 && p.groups == 1, CLDNN_HIP_INVALID_ARG,
+                     "the staged-patch kernel takes nine-tap filters at stride 1");
+        CHIP_REQUIRE(t.pad_lo_b == 0 && t.pad_hi_b == 0, CLDNN_HIP_INVALID_ARG, "the staged-patch kernel takes no batch padding");
+        const int wp = t.x + t.pad_lo_x + t.pad_hi_x, hp = t.y + t.pad_lo_y + t.pad_hi_y;
+        const int64_t pos_total = (int64_t)p.B * hp * wp;
+        const int halo_lo = p.py * wp + p.px;
+        const int halo_hi = ((p.FY - 1) * p.dy - p.py) * wp + ((p.FX - 1) * p.dx - p.px);
+        CHIP_REQUIRE(halo_lo >= 0 && halo_hi >= 0, CLDNN_HIP_INVALID_ARG, "the staged-patch kernel needs taps on both sides of the anchor");
+        const int waves = (tc.tile_pixels / 64) * (tc.tile_ofm / 128);
+        pl.block = waves * 64;
+        pl.halo_patch_len = (tc.tile_pixels + halo_lo + halo_hi + 63) / 64 * 64;
+        pl.halo_ptiles = (int)((pos_total + tc.tile_pixels - 1) / tc.tile_pixels);
+        // the next block's patch is requested in six steps of the current one, by every wave
+        const int slots = (HALO_TAPS - 1 - (HALO_RING - 2)) * waves;
+        pl.halo_pl = (4 * (pl.halo_patch_len / 64) + slots - 1) / slots;
+        CHIP_REQUIRE(pl.halo_pl <= 2, CLDNN_HIP_UNSUPPORTED_SIZE, "rows too long for the staged-patch kernel's request slots");
+    }
     pl.ofm_tiles = (p.OFM + tc.tile_ofm - 1) / tc.tile_ofm;
     pl.m_total = (int64_t)p.B * p.OH * p.OW;
     // every 16 pixels stream all the weights again (and take 1 KB of scratch per K-step when gathered)
     CHIP_REQUIRE(!pl.gemv || pl.m_total <= 4096, CLDNN_HIP_INVALID_ARG, "the small-batch kernel takes at most 4096 output pixels");
     CHIP_REQUIRE(pl.m_total < (1ll << 31), CLDNN_HIP_UNSUPPORTED_SIZE, "more than 2^31 output pixels");
     pl.mtiles = (int)((pl.m_total + tc.tile_pixels - 1) / tc.tile_pixels);
+    if (pl.halo) pl.mtiles = pl.halo_ptiles;
     // which operand do the eight dies share out?  the larger one (it is then read from memory once, not 8 times)
     const int64_t w_bytes = (int64_t)p.OFM * (p.IFM / p.groups) * p.FY * p.FX, in_bytes = (int64_t)p.B * p.IFM * p.IH * p.IW;
-    pl.by_features = !pl.stream && !pl.wsl && !pl.gemv && w_bytes > in_bytes && (p.OFM + tc.tile_ofm - 1) / tc.tile_ofm >= 8 ? 1 : 0;
+    pl.by_features = !pl.stream && !pl.wsl && !pl.gemv && !pl.halo && w_bytes > in_bytes && (p.OFM + tc.tile_ofm - 1) / tc.tile_ofm >= 8 ? 1 : 0;
     int64_t grid = pl.by_features ? (int64_t)((pl.ofm_tiles + 7) / 8) * 8 * pl.mtiles : (int64_t)((pl.mtiles + 7) / 8) * 8 * pl.ofm_tiles;
     if (pl.stream) grid = ((int64_t)pl.mtiles * pl.ofm_tiles + 3) / 4;  // one wave per (pixel tile, span)
     pl.lds_bytes = pl.stream ? 0 : (pl.bdir ? 3 * 4 * tc.tile_ofm * 16 : 2 * 4 * (tc.tile_ofm + tc.tile_pixels) * 16);
@@ -258,6 +289,18 @@ MfmaPlan mfma_plan(const ConvProblem& p, int tile, int cus)
         pl.wsl_tpp = (pl.mtiles + parts - 1) / parts;
         parts = ((pl.mtiles + pl.wsl_tpp - 1) / pl.wsl_tpp + 7) / 8 * 8;
         pl.wsl_parts = parts;
+        grid = (int64_t)parts * pl.ofm_tiles;
+    }
+    if (pl.halo) {
+        pl.lds_bytes = (HALO_RING * 4 * tc.tile_ofm + 2 * 4 * pl.halo_patch_len) * 16;
+        CHIP_REQUIRE(pl.lds_bytes <= WSL_MAX_LDS, CLDNN_HIP_UNSUPPORTED_SIZE, "rows too long for the staged-patch kernel's LDS");
+        // persistent workgroups: as many as the chip holds at once (two waves per SIMD by registers), split evenly over
+        // the feature tiles; partitions come in eights (one contiguous run of position tiles per die)
+        const int by_lds = WSL_MAX_LDS / pl.lds_bytes, by_regs = 8 / (pl.block / 64);
+        const int per_cu = std::max(1, std::min(by_lds, by_regs));
+        int parts = std::max(8, cus * per_cu / pl.ofm_tiles / 8 * 8);
+        parts = std::min(parts, (pl.halo_ptiles + 7) / 8 * 8);
+        pl.halo_parts = parts;
         grid = (int64_t)parts * pl.ofm_tiles;
     }
     if (pl.gemv) {
@@ -504,7 +547,25 @@ void launch_conv_mfma(hipStream_t s, const ConvProblem& p, const MfmaPlan& pl, c
         }
     }
     a.bpk = (const v4i*)wb.gather;
-    if (pl.gemv) launch_gemv(s, a, pl.grid, pl.gemv_waves, pl.mtiles);  // element-wise epilogue only
+    if (pl.halo) {
+        HaloArgs h{};
+        h.m = a;
+        const cldnn_hip_tensor& t = p.in_t;
+        h.Wp = t.x + t.pad_lo_x + t.pad_hi_x;
+        h.YXp = h.Wp * (t.y + t.pad_lo_y + t.pad_hi_y);
+        h.pos_total = p.B * h.YXp;
+        h.div_yxp = make_div((uint32_t)h.YXp), h.div_wp = make_div((uint32_t)h.Wp);
+        h.pad_lo_y = t.pad_lo_y, h.pad_lo_x = t.pad_lo_x;
+        h.halo_lo = p.py * h.Wp + p.px;
+        h.patch_len = pl.halo_patch_len, h.cps = pl.halo_patch_len / 64;
+        h.div_cps = make_div((uint32_t)h.cps);
+        h.blocks = pl.cb / 4;
+        h.ptiles = pl.halo_ptiles, h.parts = pl.halo_parts;
+        for (int k = 0; k < HALO_TAPS; ++k)
+            h.tap[k] = h.halo_lo + ((k / p.FX) * p.dy - p.py) * h.Wp + ((k % p.FX) * p.dx - p.px);
+        launch_halo(s, h, pl.tile - FIRST_HALO_ROW, pl.halo_pl, pl.grid, pl.lds_bytes, kind);
+    }
+    else if (pl.gemv) launch_gemv(s, a, pl.grid, pl.gemv_waves, pl.mtiles);  // element-wise epilogue only
     else if (pl.stream) launch_stream(s, a, tc.wave_pixels / 16, pl.grid, kind);
     else if (pl.bdir && tc.kgroups == 2) launch_bdir_k2(s, a, tc.wave_pixels / 16, pl.grid, pl.lds_bytes, kind);
     else if (pl.bdir && tc.kgroups == 4) launch_bdir_k4(s, a, tc.wave_pixels / 16, pl.grid, pl.lds_bytes, kind);

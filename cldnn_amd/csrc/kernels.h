@@ -51,6 +51,12 @@ struct MfmaPlan {
     int wsl_tpp;         // pixel tiles per partition
     int gemv;            // 1: few pixels, long K: 16-feature fragments, waves split K (no LDS in the loop)
     int gemv_waves;      // its waves per workgroup
+    int halo;            // 1: nine-tap stride-1 kernel with both operands staged in LDS by direct loads (conv_halo_kernel.h)
+    int halo_patch_len;  // its patch length in positions per slice (multiple of 64)
+    int halo_parts;      // its workgroups per feature tile (multiple of 8)
+    int halo_ptiles;     // its position tiles (positions count the input's border)
+    int halo_pl;         // its patch wave-loads per wave and requesting step
+    int block;           // threads per workgroup
     int checked;         // 1: taps bounds-checked per load, 0: input carries a sufficient zero border
     int tap_minor;       // K order: 1 = (group of 4 slices, tap), taps innermost; 0 = (tap, slice)
     int cb;              // input feature slices of 16

@@ -1,5 +1,6 @@
 // Engine / buffer / event half of the thin HIP layer: hipMalloc buffers with a pinned
 // lock() shadow, one hipStream per engine, pooled hipEvents.
+#include "kernels.h"
 #include "runtime.h"
 
 #include <chrono>
@@ -130,6 +131,7 @@ cldnn_hip_status cldnn_hip_engine_create(uint32_t device, uint32_t enable_profil
             e->make_current();
             CHIP_CHECK(hipGetDeviceProperties(&e->props, e->device));
             CHIP_CHECK(hipStreamCreateWithFlags(&e->stream, hipStreamNonBlocking));
+            e->static_scratch = mfma_static_scratch(e->device);
         } catch (...) {
             delete e;
             throw;

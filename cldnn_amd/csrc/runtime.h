@@ -17,6 +17,9 @@ struct cldnn_hip_engine_s {
     std::atomic<int64_t> used{0}, max_used{0};
     std::mutex pool_mutex;
     std::vector<hipEvent_t> event_pool;  // recycled hipEvents (the reference pools its cl events too)
+    // this device's copy of the scratch array inside the code object, looked up when the engine is created, so that
+    // cldnn_hip_conv_enqueue_static_scratch only launches
+    void* static_scratch = nullptr;
 
     hipEvent_t take_event();
     void give_event(hipEvent_t ev);

@@ -17,6 +17,7 @@ int hip_activation_code(int32_t f);
 cldnn_hip_pooling_desc pooling_descriptor(const node* n);
 void build_program(cldnn_program_impl* prog, cldnn_topology_impl* topo, const std::vector<std::string>& outputs);
 std::string describe_node(const node* n);
+std::vector<node*> launch_waits(const node* n);
 std::string describe_program(const cldnn_program_impl* prog);
 
 static thread_local std::string g_last_error;
@@ -131,6 +132,7 @@ static void submit(cldnn_network_impl* net, cldnn_event* deps, size_t ndeps, cld
 {
     cldnn_program_impl* prog = net->program.get();
     cldnn_engine_impl* eng = prog->engine.get();
+    std::lock_guard<std::mutex> state(net->run_state);
     if (ndeps) {
         std::vector<cldnn_hip_event> hs;
         for (size_t i = 0; i < ndeps; ++i) hs.push_back(deps[i]->h);
@@ -166,7 +168,8 @@ static void submit(cldnn_network_impl* net, cldnn_event* deps, size_t ndeps, cld
             net->stream_events.push_back(fork);
             hip_check(cldnn_hip_engine_wait_events(eng->side, &fork, 1));
         }
-        for (node* d : n->deps) {
+        // the launch at the head of a chain does the work of every member: it waits for what any of them reads
+        for (node* d : launch_waits(n)) {
             auto j = joins.find(d);
             if (j != joins.end()) hip_check(cldnn_hip_engine_wait_events(eng->h, &j->second, 1));
         }
@@ -290,6 +293,8 @@ static void submit(cldnn_network_impl* net, cldnn_event* deps, size_t ndeps, cld
     net->has_run = true;
 }
 
+static void finish_deferred_run(const std::shared_ptr<deferred_run>& run);
+
 // called by cldnn_hip_event_set (or at once, if the event got set in the meantime) for every user event a postponed
 // run waits for; the last one submits the run
 static void gate_opened(void* param)
@@ -302,12 +307,29 @@ static void gate_opened(void* param)
         last = --run->gates_left == 0;
     }
     if (!last) return;
+    finish_deferred_run(run);
+}
+
+// Submit a postponed run (or, when it was cancelled while being set up, only report): whoever waits for its marker or
+// for the network is released either way.
+static void finish_deferred_run(const std::shared_ptr<deferred_run>& run)
+{
     std::string error;
-    try {
-        submit(run->net, run->deps.data(), run->deps.size(), run->marker.get());
-    } catch (const std::exception& e) {
-        error = e.what();
-        (void)cldnn_hip_event_record_deferred(run->marker->h);  // nobody may wait for ever
+    bool cancelled = false;
+    {
+        std::lock_guard<std::mutex> g(run->m);
+        cancelled = run->cancelled;
+        error = run->error;
+    }
+    if (cancelled) {
+        (void)cldnn_hip_event_record_deferred(run->marker->h);
+    } else {
+        try {
+            submit(run->net, run->deps.data(), run->deps.size(), run->marker.get());
+        } catch (const std::exception& e) {
+            error = e.what();
+            (void)cldnn_hip_event_record_deferred(run->marker->h);  // nobody may wait for ever
+        }
     }
     for (cldnn_event d : run->deps) d->release();
     run->deps.clear();
@@ -352,17 +374,40 @@ static void execute(cldnn_network_impl* net, cldnn_event* deps, size_t ndeps)
     run->marker = ref<cldnn_event_impl>(new cldnn_event_impl(), false);
     run->marker->engine = ref<cldnn_engine_impl>(eng, true);
     hip_check(cldnn_hip_event_create_deferred(eng->h, &run->marker->h));
-    net->events.clear();
-    net->executed.clear();
-    for (auto& u : prog->nodes) {
-        node* n = u.get();
-        if (n->is_output) net->events[n] = run->marker;
-        if (!n->constant && n->p->type != prim_type::input_layout) net->executed.push_back(n->p->id);
+    {
+        std::lock_guard<std::mutex> state(net->run_state);
+        net->events.clear();
+        net->executed.clear();
+        for (auto& u : prog->nodes) {
+            node* n = u.get();
+            if (n->is_output) net->events[n] = run->marker;
+            if (!n->constant && n->p->type != prim_type::input_layout) net->executed.push_back(n->p->id);
+        }
+        net->has_run = true;
     }
-    net->has_run = true;
     net->pending = run;
-    for (cldnn_event g : gates)
-        hip_check(cldnn_hip_event_add_handler(g->h, gate_opened, new std::shared_ptr<deferred_run>(run)));
+    size_t registered = 0;
+    for (cldnn_event g : gates) {
+        auto* param = new std::shared_ptr<deferred_run>(run);
+        const cldnn_hip_status st = cldnn_hip_event_add_handler(g->h, gate_opened, param);
+        if (st == CLDNN_HIP_SUCCESS) {
+            ++registered;
+            continue;
+        }
+        // The gates registered so far still count down when their events are set; the others never will.  The run is
+        // cancelled: whoever reaches zero (here, or the last registered gate) releases the waiters and reports.
+        delete param;
+        bool finish = false;
+        {
+            std::lock_guard<std::mutex> lock(run->m);
+            run->cancelled = true;
+            run->error = "a user event of the dependency list could not be watched";
+            run->gates_left -= (int)(gates.size() - registered);
+            finish = run->gates_left == 0;
+        }
+        if (finish) finish_deferred_run(run);
+        hip_check(st);
+    }
 }
 
 }  // namespace host
@@ -1015,6 +1060,7 @@ void cldnn_get_network_executed_primitive_names(cldnn_network network, char* nam
 {
     guard_void(status, [&] {
         HOST_REQUIRE(network, CLDNN_INVALID_ARG, "Network should not be null.");
+        std::lock_guard<std::mutex> state(network->run_state);
         copy_names(network->executed, names, size, size_ret);
     });
 }
@@ -1057,6 +1103,7 @@ cldnn_network_output cldnn_get_network_output(cldnn_network network, const char*
 {
     return guard<cldnn_network_output>(status, cldnn_network_output{nullptr, nullptr}, [&] {
         node* n = output_node(network, name);
+        std::lock_guard<std::mutex> state(network->run_state);
         cldnn_network_output o{network->events.at(n).get(), network->mem.at(n).get()};
         o.event->retain();
         o.memory->retain();
@@ -1078,6 +1125,7 @@ cldnn_event cldnn_get_network_output_event(cldnn_network network, const char* na
 {
     return guard<cldnn_event>(status, nullptr, [&] {
         node* n = output_node(network, name);
+        std::lock_guard<std::mutex> state(network->run_state);
         cldnn_event e = network->events.at(n).get();
         e->retain();
         return e;

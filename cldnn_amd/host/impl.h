@@ -201,6 +201,7 @@ struct node {
     // two results share one buffer (the second is its contiguous tail: feature slices are the outermost axis).
     node* sibling = nullptr;
     node* sibling_head = nullptr;
+    cldnn_padding unpaired_padding{};  // the output padding this node had before it took the wider border of its pair
     // member of a chain whose result stays in registers: it has no buffer and nobody but the next member reads it
     bool chain_unkept() const
     {
@@ -233,6 +234,7 @@ struct deferred_run {
     std::condition_variable cv;
     int gates_left = 0;
     bool submitted = false;
+    bool cancelled = false;                // the run could not be set up: the last gate reports instead of submitting
     std::string error;                     // a failure of the late submission, reported by the next call on the network
     std::vector<cldnn_event> deps;         // retained dependency list
     host::ref<cldnn_event_impl> marker;    // the deferred event the outputs carry
@@ -242,6 +244,9 @@ struct deferred_run {
 struct cldnn_network_impl : host::refcounted {
     host::ref<cldnn_program_impl> program;
     std::shared_ptr<deferred_run> pending;  // a run that has not been submitted yet
+    // A postponed run is submitted by whichever thread sets its last user event, while the application's thread may ask
+    // for outputs, executed ids or profiling data: events, executed and stream_events are read and written under this lock.
+    std::mutex run_state;
     std::map<host::node*, host::ref<cldnn_memory_impl>> mem;
     std::map<host::node*, host::ref<cldnn_event_impl>> events;
     std::map<std::string, bool> input_set;

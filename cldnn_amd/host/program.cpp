@@ -946,6 +946,31 @@ static void prepare_conv(cldnn_program_impl* prog, node* n, conv_build& cb)
     d.impl = CLDNN_HIP_IMPL_AUTO;
 }
 
+// Build option tuning_config: which row of the tile table runs this convolution.  Reference
+// src/gpu/convolution_gpu.cpp:147-154, kernel_selector/core/kernel_selector.cpp GetAutoTuneBestKernel: take the cached choice;
+// in tune_and_cache mode measure what the cache does not hold and add it.  Applies to every convolution object the
+// program creates, a pair of convolutions in one launch included; a chain has no rows to choose from and is kept.
+static void apply_tuning(cldnn_program_impl* prog, cldnn_hip_conv_desc& d, const void* weights, const void* bias, const float* wqf,
+                         const float* calib, const float* eltw_calib)
+{
+    if (prog->tuning.mode == cldnn_tuning_disabled) return;
+    cldnn_hip_engine_info info{};
+    hip_check(cldnn_hip_engine_get_info(prog->engine->h, &info));
+    const std::string key = conv_signature(d);
+    std::string name;
+    int row = -1;
+    if (prog->tuning.find(info.cores_count, key, &name, &row)) {
+        if (row >= 0 && row < cldnn_hip_tile_config_count() && name == cldnn_hip_tile_config_name(row)) d.tile_override = row + 1;
+        ++prog->tuned_from_cache;
+    } else if (prog->tuning.mode == cldnn_tuning_tune_and_cache) {
+        float best_us = 0.0f;
+        hip_check(cldnn_hip_conv_tune(prog->engine->h, &d, weights, bias, wqf, calib, eltw_calib, 20, &row, &best_us, nullptr, nullptr));
+        prog->tuning.store(info.cores_count, key, row >= 0 ? cldnn_hip_tile_config_name(row) : "table", row);
+        if (row >= 0) d.tile_override = row + 1;
+        ++prog->tuned_now;
+    }
+}
+
 static void compile_conv(cldnn_program_impl* prog, node* n)
 {
     conv_build cb;
@@ -956,26 +981,7 @@ static void compile_conv(cldnn_program_impl* prog, node* n)
     const float* calib_ptr = cb.calib();
     const void* eltw_calib = cb.eltw_calib();
     std::vector<uint8_t>& wv = cb.wv;
-    if (prog->tuning.mode != cldnn_tuning_disabled) {
-        // reference src/gpu/convolution_gpu.cpp:147-154, kernel_selector/core/kernel_selector.cpp GetAutoTuneBestKernel: take
-        // the cached choice; in tune_and_cache mode measure what the cache does not hold and add it
-        cldnn_hip_engine_info info{};
-        hip_check(cldnn_hip_engine_get_info(prog->engine->h, &info));
-        const std::string key = conv_signature(d);
-        std::string name;
-        int row = -1;
-        if (prog->tuning.find(info.cores_count, key, &name, &row)) {
-            if (row >= 0 && row < cldnn_hip_tile_config_count() && name == cldnn_hip_tile_config_name(row)) d.tile_override = row + 1;
-            ++prog->tuned_from_cache;
-        } else if (prog->tuning.mode == cldnn_tuning_tune_and_cache) {
-            float best_us = 0.0f;
-            hip_check(cldnn_hip_conv_tune(prog->engine->h, &d, wv.data(), bias_ptr, wqf_ptr, calib_ptr, (const float*)eltw_calib, 20, &row,
-                                          &best_us, nullptr, nullptr));
-            prog->tuning.store(info.cores_count, key, row >= 0 ? cldnn_hip_tile_config_name(row) : "table", row);
-            if (row >= 0) d.tile_override = row + 1;
-            ++prog->tuned_now;
-        }
-    }
+    apply_tuning(prog, d, wv.data(), bias_ptr, wqf_ptr, calib_ptr, (const float*)eltw_calib);
     hip_check(cldnn_hip_conv_create(n->side_stream ? prog->engine->side : prog->engine->h, &d, wv.data(), bias_ptr, wqf_ptr, calib_ptr,
                                     (const float*)eltw_calib, &n->conv));
     hip_check(cldnn_hip_conv_get_info(n->conv, &n->conv_info));
@@ -1016,6 +1022,7 @@ static void pair_siblings(cldnn_program_impl* prog)
             if (gb.FY != ga.FY || gb.FX != ga.FX || gb.sy != ga.sy || gb.sx != ga.sx || gb.py != ga.py || gb.px != ga.px || gb.dy != ga.dy
                 || gb.dx != ga.dx || gb.ey != ga.ey || gb.ex != ga.ex || gb.vy != ga.vy || gb.vx != ga.vx || gb.OH != ga.OH || gb.OW != ga.OW)
                 continue;
+            a->unpaired_padding = a->out.padding, b->unpaired_padding = b->out.padding;
             for (int k = 0; k < 4; ++k) {
                 int32_t& la = a->out.padding.lower_size.sizes[k], &lb = b->out.padding.lower_size.sizes[k];
                 int32_t& ua = a->out.padding.upper_size.sizes[k], &ub = b->out.padding.upper_size.sizes[k];
@@ -1047,6 +1054,7 @@ static bool compile_siblings(cldnn_program_impl* prog, node* a)
         auto join = [](std::vector<uint8_t>& x, const std::vector<uint8_t>& y) { x.insert(x.end(), y.begin(), y.end()); };
         join(ca.wv, cb.wv), join(ca.bv, cb.bv), join(ca.qv, cb.qv), join(ca.cv, cb.cv);
         cldnn_hip_conv c = nullptr;
+        apply_tuning(prog, d, ca.weights(), ca.bias(), ca.wqf(), ca.calib(), nullptr);
         const cldnn_hip_status st = cldnn_hip_conv_create(prog->engine->h, &d, ca.weights(), ca.bias(), ca.wqf(), ca.calib(), nullptr, &c);
         if (st == CLDNN_HIP_SUCCESS) {
             cldnn_hip_conv_info info{};
@@ -1060,6 +1068,9 @@ static bool compile_siblings(cldnn_program_impl* prog, node* a)
             hip_check(st);
         }
     }
+    // taken apart: each side gets its own border back (nothing has been compiled against the wider one yet: the nodes
+    // that read these tensors come later in the order)
+    a->out.padding = a->unpaired_padding, b->out.padding = b->unpaired_padding;
     a->sibling = nullptr, b->sibling_head = nullptr;
     return false;
 }
@@ -1280,8 +1291,9 @@ void build_program(cldnn_program_impl* prog, cldnn_topology_impl* topo, const st
     if (prog->optimize_data && prog->engine && !prog->engine->memory_pool) conv_eltw_read_write_opt(prog);
     if (!prog->engine) return;  // planning only: the graph is inspected, nothing is compiled
     if (prog->engine->side) assign_streams(prog);
-    // chains with the graph optimisations only; a tuned program keeps one launch per node (its cache is per node)
-    if (prog->optimize_data && prog->tuning.mode == cldnn_tuning_disabled) {
+    // pairs and chains come with the graph optimisations; a tuning cache composes with them (it picks the rows of the
+    // launches that have rows: single convolutions and pairs)
+    if (prog->optimize_data) {
         pair_siblings(prog);
         for (auto& u : prog->nodes)
             if (u->sibling) compile_siblings(prog, u.get());
@@ -1306,6 +1318,22 @@ static std::string four(const int32_t* s)
 }
 
 // one node as JSON; sizes and paddings are [b, f, x, y] like cldnn_tensor::sizes
+// Primitives on the second stream whose completion the launch of n has to wait for: what n reads and, for the head of
+// a chain, what ANY member reads (its one kernel does the work of all of them, e.g. a follower's residual operand that
+// a shortcut convolution on the second stream produces).
+std::vector<node*> launch_waits(const node* n)
+{
+    std::vector<node*> w;
+    auto add = [&](const node* m) {
+        for (node* d : m->deps)
+            if (d->side_stream && std::find(w.begin(), w.end(), d) == w.end()) w.push_back(d);
+    };
+    add(n);
+    for (const node* m : n->chain_members) add(m);
+    if (n->sibling) add(n->sibling);
+    return w;
+}
+
 std::string describe_node(const node* n)
 {
     static const char* tn[] = {"input_layout", "data", "reorder", "activation", "eltwise", "convolution", "fused_conv_eltwise", "pooling",
@@ -1336,6 +1364,14 @@ std::string describe_node(const node* n)
     if (p.type == prim_type::concatenation) s += ",\"axis\":" + std::to_string(p.concat_axis) + ",\"in_place\":" + (n->concat_in_place ? "true" : "false");
     if (n->concat_into) s += ",\"concat_into\":\"" + n->concat_into->p->id + "\",\"concat_offset\":" + std::to_string(n->concat_offset);
     if (n->side_stream) s += ",\"stream\":1";
+    if (!n->chain_head && !n->sibling_head) {
+        const std::vector<node*> waits = launch_waits(n);
+        if (!waits.empty()) {
+            s += ",\"waits_for\":[";
+            for (size_t i = 0; i < waits.size(); ++i) s += (i ? ",\"" : "\"") + waits[i]->p->id + "\"";
+            s += "]";
+        }
+    }
     if (n->sibling) s += ",\"launches_also\":\"" + n->sibling->p->id + "\"";
     if (n->sibling_head) s += ",\"launched_by\":\"" + n->sibling_head->p->id + "\"";
     if (n->conv || n->chain || n->chain_head)

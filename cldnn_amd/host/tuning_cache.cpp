@@ -165,6 +165,7 @@ std::string conv_signature(const cldnn_hip_conv_desc& d)
       << d.fx << ";s=" << d.stride_y << "," << d.stride_x << ";d=" << d.dilation_y << "," << d.dilation_x << ";p=" << d.pad_y << "," << d.pad_x << "+"
       << d.pad_end_delta_y << "," << d.pad_end_delta_x << ";g=" << d.groups << ";bias=" << d.bias_dtype << ";q=" << d.has_wqf << d.has_calib
       << ";act=" << d.activation << ";fc=" << d.fully_connected << ";even=" << d.round_to_even;
+    if (d.sibling_split) o << ";pair=" << d.sibling_split << "," << d.sibling_activation;  // two convolutions of one input in one launch
     if (d.fused)
         o << ";eltw=" << (d.second_input_in_output ? std::string("inplace") : tensor(d.eltw)) << ";es=" << d.eltw_stride_y << "," << d.eltw_stride_x
           << ";eact=" << d.eltw_activation << ";ecal=" << d.has_eltw_calib << ";scale1=" << (d.non_conv_scale == 1.0f) << ";csat=" << d.conv_saturate;

@@ -742,3 +742,46 @@ def test_sibling_split_is_validated(eng):
     e = np.zeros((1, 96, 6, 6), np.int8)
     with pytest.raises(hip.HipError):  # not together with a fused second input
         hip.conv_forward(eng, x, w, bias, wqf, calib, fmt="fs_b_yx_fsv16", out_dt="s8", sibling_split=32, sibling_act="relu", eltw=e)
+
+
+# ------------------------------------------------------------------ the reference's differential recipe, as written
+# reference tests/test_cases/convolution_gpu_test.cpp:4931-5115 (TEST_P(convolution_gpu, b_fs_yx_fsv4)): iota-filled char
+# data 2 x F x 56 x 56 and iota-filled char weights 32 x F x k x k, offset -(k / 2), stride and output padding from the
+# parameter list; with "bias" also float bias / weight-quantization / calibration ramps (0.1 / 0.3 / 0.2, step 0.01,
+# wrapping at 0.9).  The reference compares its semantic kernel with its b_fs_yx_fsv4 kernel; here the oracle stands for
+# the semantic kernel and every layout the library computes in is compared with it byte for byte.
+B4_PARAMS = [(1, 32, 1, 0, False), (3, 32, 1, 0, False), (7, 3, 1, 0, False), (1, 32, 1, 0, True), (3, 32, 1, 0, True),
+             (7, 3, 1, 0, True), (1, 32, 1, 1, False), (3, 32, 1, 1, False), (7, 3, 1, 1, False), (1, 32, 2, 0, False),
+             (3, 32, 2, 0, False), (7, 3, 2, 0, False), (3, 64, 2, 1, True)]  # convolution_gpu_test.cpp:5091-5106
+
+
+def b4_ramp(start, n):
+    out, x = [], np.float32(start)
+    for _ in range(n):
+        x = np.float32(x + np.float32(0.01))
+        if x >= np.float32(0.9):
+            x = np.float32(start)
+        out.append(x)
+    return np.array(out, np.float32)
+
+
+@pytest.mark.parametrize("fmt", ["bfyx", "fs_b_yx_fsv16", "b_fs_yx_fsv4"])
+@pytest.mark.parametrize("k,F,stride,out_pad,with_bias", B4_PARAMS,
+                         ids=["k%d_f%d_s%d_op%d%s" % (p[0], p[1], p[2], p[3], "_bias" if p[4] else "") for p in B4_PARAMS])
+def test_reference_differential_recipe_with_iota_data(eng, fmt, k, F, stride, out_pad, with_bias):
+    if fmt == "b_fs_yx_fsv4" and F > 4:
+        pytest.skip("b_fs_yx_fsv4 feeds first layers (at most 4 input features) here")
+    B, H, W, OFM = 2, 56, 56, 32
+    x = (np.arange(B * F * H * W, dtype=np.int64) % 256).astype(np.uint8).view(np.int8).reshape(B, F, H, W)
+    w = (np.arange(OFM * F * k * k, dtype=np.int64) % 256).astype(np.uint8).view(np.int8).reshape(OFM, F, k, k)
+    bias = wqf = calib = None
+    if with_bias:
+        bias, calib, wqf = b4_ramp(0.1, OFM), b4_ramp(0.2, OFM), b4_ramp(0.3, OFM)
+    kw = dict(stride=(stride, stride), pad=(k // 2, k // 2), out_dt="s8")
+    border = (k // 2, k // 2) if fmt != "bfyx" else (0, 0)
+    # (the unquantized form wraps around in 8 bits: it has no int32 accumulators to compare)
+    ro, (go, info) = both(eng, x, w, bias, wqf, calib, fmt=fmt, in_pad=border, out_pad=(out_pad, out_pad), acc=False, **kw)
+    assert ro.shape == (B, OFM, (H + stride - 1) // stride, (W + stride - 1) // stride)
+    if with_bias and fmt != "bfyx":
+        assert info.impl == hip.IMPL_MFMA, info.kernel_name  # the quantized form runs on the matrix-core kernels
+    assert_same(ro, go)

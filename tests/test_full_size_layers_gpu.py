@@ -4,7 +4,11 @@ The row of the tile-config table depends on the pixel count, so the kernels prod
 not the ones the small-shape tests reach.  Here each distinct layer signature is built exactly as bench.py builds it
 (same seeded data, same descriptors, same chain grouping), run once at full size, and the first image(s) of its
 output are compared with the oracle bit for bit (a convolution is independent per image).  The kernels the committed
-profiles name as dominant are asserted by name."""
+profiles name as dominant are asserted by name.
+
+The benchmark's calibration factors saturate most outputs (about half are ReLU zeros, most of the rest 127), so a second
+test runs every signature with factors that spread the outputs over the int8 range, and compares the raw int32
+accumulators of the first image as well."""
 import numpy as np
 import pytest
 
@@ -89,4 +93,33 @@ def test_layer_at_its_real_batch_matches_the_oracle(eng, wl, group):
     kept = [L for L in stack if L.kept]
     assert checked == sum(min(images, batch) * L.spec["ofm"] * L.spec["out_hw"] ** 2 for L in kept)
     assert mismatches == 0, "%d of %d outputs differ from the oracle (%s)" % (mismatches, checked, name)
+    bench.release_stack(stack)
+
+
+@pytest.mark.parametrize("wl,group", cases())
+def test_layer_at_its_real_batch_with_spread_outputs_and_accumulators(eng, wl, group):
+    from oracle import refconv as rc
+    _, batch, fuse, images = CONFIGS[wl]
+    # outputs, launched as production launches them (chains, pairs), with factors under which a wrong sum shows
+    stack = bench.build_stack(eng, group, batch, fuse, calibration="spread")
+    bench.run_step(bench.launches(stack))
+    eng.finish()
+    _, _, checked, mismatches = bench.cpu_pass(eng, stack, 1, verify=True)
+    assert checked > 0 and mismatches == 0, "%d of %d outputs differ from the oracle" % (mismatches, checked)
+    for L in stack:
+        if L.kept and L.spec["act"] == "relu" and not L.fused:
+            got = hip.download(eng, L.out)[:1]
+            inside = np.count_nonzero((got > 0) & (got < 127))
+            assert inside > 0.2 * got.size, "the outputs of %s do not spread over the int8 range" % L.spec["name"]
+    bench.release_stack(stack)
+    # int32 accumulators of the first image, every layer a launch of its own on the row production picks at this batch
+    stack = bench.build_stack(eng, group, batch, fuse, chains=False, calibration="spread")
+    for L in stack:
+        l = L.spec
+        acc = L.conv.accumulators(L.xin)[:1]
+        _, ref_acc = rc.conv(L.x[:1], L.w, None, wqf=L.wqf, calib=L.calib, stride=(l["stride"],) * 2, pad=(l["pad"],) * 2,
+                             groups=l["groups"], out_dt="s8", want_acc=True)
+        assert acc.shape == ref_acc.shape
+        bad = int(np.count_nonzero(acc != ref_acc))
+        assert bad == 0, "%d of %d accumulators of %s differ (%s)" % (bad, acc.size, l["name"], L.info.kernel_name.decode())
     bench.release_stack(stack)

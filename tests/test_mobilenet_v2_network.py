@@ -109,3 +109,28 @@ def test_mobilenet_v2_int8_network_matches_the_oracle():
     assert len(both) == 10, both
     net.set_input_data("input", cl.make_memory(eng2, x))
     np.testing.assert_array_equal(net.execute()["fc1000"].get_memory().read(), run_oracle(x, params, folded=True)["fc1000"])
+
+
+@pytest.mark.gpu
+def test_mobilenet_v2_network_at_the_benchmark_batch_matches_the_oracle():
+    """Batch 32: the rows of the tile table, the depthwise chains and the memory pool as the benchmark runs them; the
+    oracle runs the first images.  One build with the logits as the only output (the production plan), one that also
+    watches linear points along the way."""
+    from cldnn_amd import api as cl
+    eng = cl.engine()
+    B, checked = 32, 2
+    x = np.random.default_rng(61).integers(0, 256, (B, 3, 224, 224)).astype(np.uint8)
+    params = mn.random_weights(seed=67)
+    run_oracle(x[:2], params, calibrate=True)
+    topo = mn.topology(cl, eng, params, B)
+    ref = run_oracle(x[:checked], params, folded=True)
+    for watch in (["fc1000"], ["b1_project", "b7_project", "b14_project", "b17_project", "fc1000"]):
+        net = cl.network(eng, topo, cl.build_options(optimize_data=True, outputs=watch))
+        kernels = {i: net.get_primitive_info(i).get("kernel", "") for i in net.get_all_primitive_ids()}
+        assert sum(k.startswith("in the chain of") for k in kernels.values()) >= 10, "no depthwise chains at the benchmark batch"
+        net.set_input_data("input", cl.make_memory(eng, x))
+        outs = net.execute()
+        for name in watch:
+            got = outs[name].get_memory().read()[:checked]
+            bad = int((got != ref[name]).sum())
+            assert bad == 0, "%s (outputs %s): %d of %d values differ" % (name, watch, bad, got.size)

@@ -183,8 +183,49 @@ def test_shortcut_convolutions_on_the_second_stream():
         net = cl.network(eng, topo, opts)
         side = [i for i in net.get_all_primitive_ids() if "_branch" in i and net.get_primitive_info(i).get("stream") == 1]
         assert side == ["res2a_branch1", "res3a_branch1", "res4a_branch1", "res5a_branch1"]
+        # whatever launch does the work of a shortcut's reader waits for the shortcut: the reader itself, or the head of
+        # the chain the reader is a member of (res2a_branch2b launches res2a_branch2c + sum as well)
+        for s in side:
+            waiting = []
+            for i in net.get_all_primitive_ids():
+                info = net.get_primitive_info(i)
+                if s in info.get("waits_for", []):
+                    waiting.append((i, info.get("kernel", "")))
+            assert waiting, "nothing waits for %s" % s
+            assert all(not k.startswith("in the chain of") for _, k in waiting), waiting
+        chained = [i for i in net.get_all_primitive_ids() if net.get_primitive_info(i).get("kernel", "").startswith("in the chain of")]
+        if any(i.startswith("res2a_branch2c") for i in chained):
+            assert "res2a_branch1" in net.get_primitive_info("res2a_branch2b").get("waits_for", [])
         for k in (0, 1, 0):
             net.set_input_data("input", cl.make_memory(eng, xs[k]))
             outs = net.execute()
             for name in watch:
                 np.testing.assert_array_equal(outs[name].get_memory().read(), refs[k][name], err_msg="%s pool=%s input %d" % (name, pool, k))
+
+
+@pytest.mark.gpu
+def test_resnet50_network_at_the_benchmark_batch_matches_the_oracle():
+    """Batch 32 is where the tile table, the paired launches, the chains and the memory pool take the rows and sizes the
+    benchmark runs (at batch 2 they take others).  The production plan has one output, the logits, which depend on every
+    layer; a second build watches the block ends to say where a difference starts.  The oracle runs the first images."""
+    from cldnn_amd import api as cl
+    eng = cl.engine()
+    B, checked = 32, 2
+    x = np.random.default_rng(57).integers(0, 256, (B, 3, 224, 224)).astype(np.uint8)
+    params = rn.random_weights(seed=59)
+    run_oracle(x[:2], params, fused=BLOCKS, calibrate=True)
+    topo = rn.topology(cl, eng, params, B)
+    for watch in (["fc1000"], ["res2c", "res3d", "res4f", "res5c", "fc1000"]):
+        opts = cl.build_options(optimize_data=True, outputs=watch)
+        fused = [n["id"].split("_fused_")[1] for n in cl.plan(topo, opts) if "_fused_" in n["id"]]
+        ref = run_oracle(x[:checked], params, fused=fused)
+        net = cl.network(eng, topo, opts)
+        kernels = {i: net.get_primitive_info(i).get("kernel", "") for i in net.get_all_primitive_ids()}
+        assert sum(k.startswith("in the chain of") for k in kernels.values()) >= 2, "no chains at the benchmark batch"
+        assert not any(k.startswith("conv_ref") for k in kernels.values()), kernels
+        net.set_input_data("input", cl.make_memory(eng, x))
+        outs = net.execute()
+        for name in watch:
+            got = outs[name].get_memory().read()[:checked]
+            bad = int((got != ref[name]).sum())
+            assert bad == 0, "%s (outputs %s): %d of %d values differ" % (name, watch, bad, got.size)

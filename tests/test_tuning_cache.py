@@ -65,8 +65,9 @@ def test_tune_and_cache_then_use_cache(tmp_path):
     w1 = r.integers(-127, 128, (64, 64, 3, 3)).astype(np.int8)
     w2 = r.integers(-127, 128, (256, 64, 1, 1)).astype(np.int8)
     c1, c2 = (r.uniform(1e-3, 4e-3, n).astype(np.float32) for n in (64, 256))
+    # the second convolution has a stride, so the two cannot run as a chain: every node is a launch with a row of its own
     ref = rc.conv(rc.conv(x, w1, None, wqf=np.ones(64, np.float32), calib=c1, pad=(1, 1), out_dt="s8", act="relu"),
-                  w2, None, wqf=np.ones(256, np.float32), calib=c2, out_dt="s8", act="relu")
+                  w2, None, wqf=np.ones(256, np.float32), calib=c2, stride=(2, 2), out_dt="s8", act="relu")
 
     def run(eng, opts):
         vec = lambda v: cl.make_memory(eng, np.asarray(v, np.float32).reshape(1, 1, 1, -1))  # noqa: E731
@@ -74,7 +75,7 @@ def test_tune_and_cache_then_use_cache(tmp_path):
                            cl.data("w1", cl.make_memory(eng, w1)), cl.data("w2", cl.make_memory(eng, w2)),
                            cl.data("q1", vec(np.ones(64))), cl.data("q2", vec(np.ones(256))), cl.data("c1", vec(c1)), cl.data("c2", vec(c2)),
                            cl.convolution("a", "in", ["w1"], None, ["q1"], ["c1"], input_offset=cl.tensor(0, 0, -1, -1, 0), with_activation=True),
-                           cl.convolution("b", "a", ["w2"], None, ["q2"], ["c2"], with_activation=True))
+                           cl.convolution("b", "a", ["w2"], None, ["q2"], ["c2"], stride=cl.tensor(1, 1, 2, 2), with_activation=True))
         net = cl.network(eng, topo, opts)
         net.set_input_data("in", cl.make_memory(eng, x))
         out = net.execute()["b"].get_memory().read()
@@ -99,13 +100,8 @@ def test_tune_and_cache_then_use_cache(tmp_path):
     assert used_kernels == tuned_kernels
     # the file decides: name another row for the second convolution and it runs on that row; a stale name is ignored
     key_b = [k for k in entries if "256x64x1x1" in k][0]
-    # the table's own choice: a program with a tuning cache keeps one launch per node (the cache is per node), an untuned
-    # one runs these two convolutions as a chain
-    empty = str(tmp_path / "empty.json")
-    json.dump({}, open(empty, "w"))
-    default_kernel = run(plain_eng, cl.build_options(optimize_data=True, tuning_config=(cl.tuning_mode.tuning_use_cache, empty)))[1]["b_fsv16"]
-    assert run(plain_eng, cl.build_options(optimize_data=True))[1] == {"a": run(plain_eng, cl.build_options(optimize_data=True))[1]["a"],
-                                                                        "b_fsv16": "in the chain of a"}
+    # the table's own choice
+    default_kernel = run(plain_eng, cl.build_options(optimize_data=True))[1]["b_fsv16"]
     forced = None
     for row in range(tile_config_count()):
         entries[key_b] = [tile_config_name(row), row]
@@ -122,3 +118,54 @@ def test_tune_and_cache_then_use_cache(tmp_path):
     entries[key_b] = ["no such row", 3]
     json.dump(cache, open(path, "w"))
     assert run(plain_eng, use)[1]["b_fsv16"] == default_kernel
+
+
+@pytest.mark.gpu
+def test_a_tuned_program_keeps_its_pairs_and_chains(tmp_path):
+    """The reference's tuning composes with every graph pass (src/program.cpp:305-309, kernel_selector.cpp:148-207); here
+    two convolutions of one input still run as one launch (whose row the cache decides) and a 3x3 with the 1x1 behind it
+    still run as a chain (which has no rows), with the same bits as the untuned program."""
+    path = str(tmp_path / "cache.json")
+    r = np.random.default_rng(5)
+    x = r.integers(-128, 128, (2, 64, 14, 14)).astype(np.int8)
+    wp = r.integers(-127, 128, (256, 64, 1, 1)).astype(np.int8)
+    wq = r.integers(-127, 128, (64, 64, 1, 1)).astype(np.int8)
+    wa = r.integers(-127, 128, (64, 64, 3, 3)).astype(np.int8)
+    wb = r.integers(-127, 128, (256, 64, 1, 1)).astype(np.int8)
+    cp, cq, ca, cb = (r.uniform(1e-3, 4e-3, n).astype(np.float32) for n in (256, 64, 64, 256))
+    one = lambda n: np.ones(n, np.float32)  # noqa: E731
+    ref_p = rc.conv(x, wp, None, wqf=one(256), calib=cp, out_dt="s8")
+    q = rc.conv(x, wq, None, wqf=one(64), calib=cq, out_dt="s8", act="relu")
+    a = rc.conv(q, wa, None, wqf=one(64), calib=ca, pad=(1, 1), out_dt="s8", act="relu")
+    ref_b = rc.conv(a, wb, None, wqf=one(256), calib=cb, out_dt="s8", act="relu")
+
+    def run(eng, opts):
+        vec = lambda v: cl.make_memory(eng, np.asarray(v, np.float32).reshape(1, 1, 1, -1))  # noqa: E731
+        topo = cl.topology(cl.input_layout("in", cl.layout(DT.i8, F.bfyx, cl.tensor(2, 64, 14, 14))),
+                           cl.data("wp", cl.make_memory(eng, wp)), cl.data("wq", cl.make_memory(eng, wq)),
+                           cl.data("wa", cl.make_memory(eng, wa)), cl.data("wb", cl.make_memory(eng, wb)),
+                           cl.data("q256", vec(one(256))), cl.data("q64", vec(one(64))),
+                           cl.data("cp", vec(cp)), cl.data("cq", vec(cq)), cl.data("ca", vec(ca)), cl.data("cb", vec(cb)),
+                           cl.convolution("p", "in", ["wp"], None, ["q256"], ["cp"]),
+                           cl.convolution("q", "in", ["wq"], None, ["q64"], ["cq"], with_activation=True),
+                           cl.convolution("a", "q", ["wa"], None, ["q64"], ["ca"], input_offset=cl.tensor(0, 0, -1, -1, 0), with_activation=True),
+                           cl.convolution("b", "a", ["wb"], None, ["q256"], ["cb"], with_activation=True))
+        net = cl.network(eng, topo, opts)
+        net.set_input_data("in", cl.make_memory(eng, x))
+        outs = net.execute()
+        info = {i: net.get_primitive_info(i) for i in net.get_all_primitive_ids()}
+        return outs["p"].get_memory().read(), outs["b"].get_memory().read(), info
+
+    eng = cl.engine(enable_profiling=True)
+    plain = run(eng, cl.build_options(optimize_data=True, outputs=["p", "b"]))
+    tuned = run(eng, cl.build_options(optimize_data=True, outputs=["p", "b"], tuning_config=(cl.tuning_mode.tuning_tune_and_cache, path)))
+    used = run(eng, cl.build_options(optimize_data=True, outputs=["p", "b"], tuning_config=(cl.tuning_mode.tuning_use_cache, path)))
+    for got_p, got_b, info in (plain, tuned, used):
+        np.testing.assert_array_equal(got_p, ref_p)
+        np.testing.assert_array_equal(got_b, ref_b)
+        pair = [i for i, d in info.items() if d.get("launches_also")]
+        assert len(pair) == 1 and info[pair[0]]["launches_also"] in ("q", "p_fsv16"), {i: d.get("launches_also") for i, d in info.items()}
+        assert info["b_fsv16"]["kernel"] == "in the chain of a"
+    entries = list(json.load(open(path)).values())[0]
+    assert any(";pair=" in k for k in entries), list(entries)
+    assert not any("3x3" in k for k in entries), "a chain has no row to tune"

@@ -65,3 +65,26 @@ def test_vgg16_int8_network_matches_the_oracle():
             assert got.reshape(ref[name].shape).shape == ref[name].shape, name
             bad = int((got.reshape(ref[name].shape) != ref[name]).sum())
             assert bad == 0, "%s (optimize_data=%s): %d of %d values differ" % (name, optimize, bad, got.size)
+
+
+@pytest.mark.gpu
+def test_vgg16_network_at_the_benchmark_batch_matches_the_oracle():
+    """Batch 16: the rows of the tile table the benchmark runs (the large-tile rows only apply from 50 000 pixels on); the
+    oracle runs the first image."""
+    from cldnn_amd import api as cl
+    eng = cl.engine()
+    B, checked = 16, 1
+    x = np.random.default_rng(71).integers(0, 256, (B, 3, 224, 224)).astype(np.uint8)
+    params = vg.random_weights(seed=73)
+    run_oracle(x[:1], params, calibrate=True)
+    ref = run_oracle(x[:checked], params)
+    topo = vg.topology(cl, eng, params, B)
+    for watch in (["fc8"], ["conv5", "pool3", "conv10", "pool5", "fc8"]):
+        net = cl.network(eng, topo, cl.build_options(optimize_data=True, outputs=watch))
+        net.set_input_data("input", cl.make_memory(eng, x))
+        outs = net.execute()
+        for name in watch:
+            got = outs[name].get_memory().read()
+            got = got.reshape((B,) + ref[name].shape[1:])[:checked]
+            bad = int((got != ref[name]).sum())
+            assert bad == 0, "%s (outputs %s): %d of %d values differ" % (name, watch, bad, got.size)
