@@ -52,27 +52,60 @@ __device__ __forceinline__ void static_for(F&& f)
 typedef const __attribute__((address_space(1))) void* halo_gptr;
 typedef __attribute__((address_space(3))) void* halo_lptr;
 
-// MT x NT fragments per wave (16 features x 16 positions each), WP x WF waves per workgroup, R stages in the weight
-// ring, PL patch wave-loads per wave in each of the first PSTEPS steps of a block.
-template <int MT, int NT, int WP, int WF, int R, int PL, int EPI, int DBG = 0>
+typedef int v16i __attribute__((ext_vector_type(16)));
+
+// LDS read issued behind the compiler's back: the destination register is written when the data arrives, which the caller
+// establishes with lds_wait (LDS reads of a wave return in order, so a count of younger reads names the one waited for)
+template <int OFFSET>
+__device__ __forceinline__ void lds_read(v4i& dst, uint32_t byte_address)
+{
+    asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(dst) : "v"(byte_address), "n"(OFFSET));
+}
+template <int YOUNGER>
+__device__ __forceinline__ void lds_wait(v4i& needed)
+{
+    asm volatile("s_waitcnt lgkmcnt(%1)" : "+v"(needed) : "n"(YOUNGER));
+}
+__device__ __forceinline__ uint32_t lds_offset(const void* p)
+{
+    return (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const char*)p;
+}
+
+// The matrix instruction here is v_mfma_i32_32x32x32_i8: a 32 feature x 32 position tile per instruction, 32 k values
+// (two feature slices of one tap: lanes 0-31 bring the 16 bytes of the first, lanes 32-63 those of the second, for both
+// operands alike).  Against the 16x16x64 form it needs half as many instructions per multiply-accumulate, which leaves
+// the issue port free for the LDS reads and the sign flips of the step (measured on a loop with both operands from LDS,
+// one barrier per step and two waves per SIMD: matrix pipe 91 % busy against 80 %).  A lane's 16 accumulators of a tile
+// are the features 8g + 4h + i (g = 0..3, i = 0..3, h = lane / 32) of position lane % 32; the weight rows of every 32-row
+// tile are stored permuted (row 8g + 4h + i holds feature 16h + 4g + i), so that the lane ends with 16 CONSECUTIVE
+// features of its position: one 16-byte store into fs_b_yx_fsv16, as in the other kernels.
+//
+// MT x NT tiles per wave (32 features x 32 positions each), WP x WF waves per workgroup, R stages in the weight ring,
+// PL patch wave-loads per wave in each of the first PSTEPS steps of a block.
+template <int MT, int NT, int WP, int WF, int R, int PL, int EPI>
 __global__ void __launch_bounds__(WP * WF * 64) conv_halo_kernel(HaloArgs h)
 {
     constexpr int TAPS = 9;
-    constexpr int LA = R - 2;                 // weight look-ahead in steps
-    constexpr int PSTEPS = TAPS - 1 - LA;     // steps of a block that request patch chunks of the next block
+    constexpr int PSTEPS = TAPS - R;          // steps of a block that request patch chunks of the next block
     constexpr int WAVES = WP * WF;
-    constexpr int BN = WF * MT * 16, BM = WP * NT * 16;
+    constexpr int BN = WF * MT * 32, BM = WP * NT * 32;
     constexpr int STAGE = 4 * BN;             // 16-byte units per ring stage
     constexpr int WL = STAGE / 64 / WAVES;    // weight wave-loads per wave and step
-    constexpr int SPANS = MT / 4;
-    constexpr int BAR_MT = MT - 3;            // the step's barrier sits behind this fragment row
+    constexpr int FRAGS = 2 * MT;             // weight fragments of a step: two k-halves x MT tiles
     static_assert(WL * 64 * WAVES == STAGE && WL >= 1, "weight stage must split evenly over the waves");
-    static_assert(MT % 4 == 0 && MT >= 4, "whole 64-feature spans per wave");
+    static_assert(MT == 4 && NT == 2 && R == 4, "the read schedule of the main loop is written out for this shape");
     const MfmaArgs& a = h.m;
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int wave_p = wave % WP, wave_f = wave / WP;
-    const int kq = lane >> 4, l16 = lane & 15;
+    const int half = lane >> 5, l32 = lane & 31;
+    // Everything the prologue and the loop read from the argument block is requested here, behind ONE wait: left to
+    // itself the compiler fetches arguments where they are first used, four dependent round trips to memory (about
+    // 0.4 us each) before the first operand request goes out.
+    asm volatile("" ::"s"(a.in), "s"(a.wpk), "s"(a.acc_init), "s"(a.ofm_tiles), "s"(a.ksteps), "s"(a.in_pf), "s"(a.xor_mask),
+                 "s"(h.pos_total), "s"(h.halo_lo), "s"(h.patch_len), "s"(h.cps), "s"(h.div_cps.mul), "s"(h.div_cps.shift),
+                 "s"(h.div_cps.one), "s"(h.blocks), "s"(h.ptiles), "s"(h.parts), "s"(h.tap[0]), "s"(h.tap[1]), "s"(h.tap[2]),
+                 "s"(h.tap[3]), "s"(h.tap[4]), "s"(h.tap[5]), "s"(h.tap[6]), "s"(h.tap[7]), "s"(h.tap[8]));
 
     // Workgroup ids are dealt round-robin to the eight dies.  A die takes a contiguous eighth of the partitions with
     // all their feature tiles adjacent in time: neighbouring position tiles share their halos, feature tiles their
@@ -80,17 +113,18 @@ __global__ void __launch_bounds__(WP * WF * 64) conv_halo_kernel(HaloArgs h)
     const int xcd = blockIdx.x & 7, jj = blockIdx.x >> 3;
     const int part = xcd * (h.parts >> 3) + jj / a.ofm_tiles;
     const int ntile = jj % a.ofm_tiles;
-    const int t_begin = (int)((long long)part * h.ptiles / h.parts);
-    const int t_end = (int)((long long)(part + 1) * h.ptiles / h.parts);
+    const int t_begin = (int)(((uint32_t)part * (uint32_t)h.ptiles) / (uint32_t)h.parts);
+    const int t_end = (int)(((uint32_t)(part + 1) * (uint32_t)h.ptiles) / (uint32_t)h.parts);
     if (t_begin >= t_end) return;
 
     extern __shared__ __align__(16) unsigned char smem[];
-    v4i* ring = reinterpret_cast<v4i*>(smem);  // [R][STAGE]
+    v4i* ring = reinterpret_cast<v4i*>(smem);  // [R][4 slices][BN rows]
     v4i* patch = ring + R * STAGE;             // [2][4 slices][patch_len]
     const int patch_v4 = 4 * h.patch_len;
 
-    const int a_lane = kq * BN + wave_f * MT * 16 + l16;
-    const int b_lane = kq * h.patch_len + wave_p * NT * 16 + l16;
+    // fragment (k-half kh, tile) of a lane: slice 2 * kh + half
+    const int a_lane = half * BN + wave_f * MT * 32 + l32;
+    const int b_lane = half * h.patch_len + wave_p * NT * 32 + l32;
     const v4i* wsrc = a.wpk + (size_t)ntile * a.ksteps * STAGE + wave * WL * 64 + lane;
     const v4i xm = {(int)a.xor_mask, (int)a.xor_mask, (int)a.xor_mask, (int)a.xor_mask};
 
@@ -111,38 +145,58 @@ __global__ void __launch_bounds__(WP * WF * 64) conv_halo_kernel(HaloArgs h)
         __builtin_amdgcn_global_load_lds((halo_gptr)src, (halo_lptr)(patch + buf * patch_v4 + sl * h.patch_len + i * 64), 16, 0, 0);
     };
 
-    v4i acc[MT][NT];
+    v16i acc[MT][NT];
     auto reset_acc = [&]() {
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) {
-            const int f = ntile * BN + ((wave_f * MT + mt) >> 2) * 64 + kq * 16 + (mt & 3) * 4;
-            const v4i init = *reinterpret_cast<const v4i*>(a.acc_init + f);
+            const int f = ntile * BN + (wave_f * MT + mt) * 32 + half * 16;
+            v16i init;
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                const v4i v = *reinterpret_cast<const v4i*>(a.acc_init + f + g * 4);
+                init[g * 4 + 0] = v[0], init[g * 4 + 1] = v[1], init[g * 4 + 2] = v[2], init[g * 4 + 3] = v[3];
+            }
 #pragma unroll
             for (int nt = 0; nt < NT; ++nt) acc[mt][nt] = init;
         }
     };
 
-    // ---- prologue: the first patch, the first LA + 1 weight stages
+    // ---- prologue: the first patch, the first R weight stages; the accumulator start values are requested behind
+    // them (the wait below then covers most of those too: loads complete in order)
     for (int c = wave; c < 4 * h.cps; c += WAVES) issue_patch(c, t_begin, 0, 0);
     step_fence();
 #pragma unroll
-    for (int u = 0; u <= LA; ++u) issue_weights(u, u);
+    for (int u = 0; u < R; ++u) issue_weights(u, u);
     step_fence();
     reset_acc();
-    asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(LA * WL) : "memory");
+    step_fence();
+    asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"((R - 2) * WL) : "memory");
 
+    // ---- main loop.  LDS reads are issued by hand (the compiler does not see them) and waited for by count: the reads of
+    // a step are a fixed sequence, returned in order, so "at most N outstanding" names exactly the fragment that is
+    // needed.  Per step and wave, in issue order: weight fragments 4..7 of this step (one in front of each of the
+    // first four fragments' matrix instructions), then, spread over the last four fragments, the next step's four
+    // activation fragments and its weight fragments 0..3.  Every fragment is requested 256 matrix-pipe clocks or more
+    // before its first use; nothing is read behind the step's barrier that the step itself still needs.
+    const uint32_t a_lane_b = lds_offset(ring) + (uint32_t)a_lane * 16u;
+    const uint32_t b_lane_b = lds_offset(patch) + (uint32_t)b_lane * 16u;
+    const uint32_t kh_bytes = 2u * (uint32_t)h.patch_len * 16u;   // from a k-half's slices to the next one's
+    constexpr int KH_A = 2 * BN * 16;                             // the same for the weights
     int rd_stage = 0;        // ring stage of the current step
-    int wnext = LA + 1;      // K-step of the tile whose weights are requested next
+    int wnext = R % TAPS;    // K-step of the tile whose weights are requested next (ksteps is a multiple of TAPS >= R)
     int pbuf = 0;            // patch buffer of the current block
-    v4i fa[4], fb[NT], fbn[NT];
+    v4i fa[FRAGS], fb[2][NT], fbn[2][NT];
     {
-        const v4i* st = ring + a_lane;
-        const v4i* pt = patch + b_lane + h.tap[0];
-#pragma unroll
-        for (int nt = 0; nt < NT; ++nt) fbn[nt] = pt[nt * 16];
-        fa[0] = st[0];
-        fa[1] = st[16];
+        const uint32_t b0 = b_lane_b + (uint32_t)h.tap[0] * 16u, b1 = b0 + kh_bytes;
+        lds_read<0>(fbn[0][0], b0), lds_read<512>(fbn[0][1], b0), lds_read<0>(fa[0], a_lane_b);
+        lds_read<0>(fbn[1][0], b1), lds_read<512>(fbn[1][1], b1), lds_read<512>(fa[1], a_lane_b);
+        lds_read<1024>(fa[2], a_lane_b), lds_read<1536>(fa[3], a_lane_b);
     }
+    auto mma = [&](int j) {
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt)
+            acc[j % MT][nt] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[j], fb[j / MT][nt], acc[j % MT][nt], 0, 0, 0);
+    };
 
     for (int tile = t_begin; tile < t_end; ++tile) {
         for (int cb = 0; cb < h.blocks; ++cb) {
@@ -151,89 +205,100 @@ __global__ void __launch_bounds__(WP * WF * 64) conv_halo_kernel(HaloArgs h)
             const int tile_n = last_cb ? tile + 1 : tile;
             static_for<0, TAPS>([&](auto ic) {
                 constexpr int S = decltype(ic)::value;
-                // loads younger than the weights of the next step when this step's barrier is reached
-                constexpr int YOUNGER = [] {
-                    int n = (LA - 1) * WL;
-                    for (int i = 0; i < LA; ++i) n += ((S - LA + i + TAPS) % TAPS) < PSTEPS ? PL : 0;
-                    return n;
-                }();
-                const v4i* st = ring + rd_stage * STAGE + a_lane;
+                // requests younger than the weights of step + 2 when this step's barrier is reached: the weights of
+                // step + 3 and the patch chunks of the last two steps
+                constexpr int YOUNGER = WL + (((S + TAPS - 2) % TAPS) < PSTEPS ? PL : 0) + (((S + TAPS - 1) % TAPS) < PSTEPS ? PL : 0);
+                const int nx_stage = rd_stage + 1 == R ? 0 : rd_stage + 1;
+                const uint32_t a_cur = a_lane_b + (uint32_t)(rd_stage * STAGE * 16);
+                const uint32_t a_nxt = a_lane_b + (uint32_t)(nx_stage * STAGE * 16);
+                const int nbuf = S == TAPS - 1 ? pbuf ^ 1 : pbuf;
+                const uint32_t b_nxt0 = b_lane_b + (uint32_t)(nbuf * patch_v4 + h.tap[(S + 1) % TAPS]) * 16u;
+                const uint32_t b_nxt1 = b_nxt0 + kh_bytes;
+                // this step's activation fragments and its first weight fragment have landed (three younger reads)
+                asm volatile("s_waitcnt lgkmcnt(3)" : "+v"(fbn[0][0]), "+v"(fbn[0][1]), "+v"(fbn[1][0]), "+v"(fbn[1][1]), "+v"(fa[0]));
 #pragma unroll
-                for (int nt = 0; nt < NT; ++nt) fb[nt] = fbn[nt] ^ xm;
+                for (int kh = 0; kh < 2; ++kh)
+#pragma unroll
+                    for (int nt = 0; nt < NT; ++nt) fb[kh][nt] = fbn[kh][nt] ^ xm;
                 step_fence();
+                lds_read<KH_A + 0>(fa[4], a_cur);
+                mma(0);
+                step_fence();
+                lds_read<KH_A + 512>(fa[5], a_cur);
+                lds_wait<4>(fa[1]);
+                mma(1);
+                step_fence();
+                lds_read<KH_A + 1024>(fa[6], a_cur);
+                lds_wait<4>(fa[2]);
+                mma(2);
+                step_fence();
+                lds_read<KH_A + 1536>(fa[7], a_cur);
+                lds_wait<4>(fa[3]);
+                mma(3);
+                step_fence();
+                lds_read<0>(fbn[0][0], b_nxt0), lds_read<512>(fbn[0][1], b_nxt0), lds_read<0>(fa[0], a_nxt);
+                lds_wait<6>(fa[4]);
+                mma(4);
+                step_fence();
+                lds_read<0>(fbn[1][0], b_nxt1), lds_read<512>(fbn[1][1], b_nxt1), lds_read<512>(fa[1], a_nxt);
+                lds_wait<8>(fa[5]);
+                mma(5);
+                step_fence();
+                lds_read<1024>(fa[2], a_nxt);
+                lds_wait<8>(fa[6]);
+                mma(6);
+                step_fence();
+                lds_read<1536>(fa[3], a_nxt);
+                lds_wait<8>(fa[7]);
+                // Every read of this step's ring stage has completed in this wave.  Behind the barrier that holds for all
+                // waves, so the stage can be refilled (with the weights of step + 4); and the weights of step + 2 and the
+                // patch chunks requested up to three steps ago are in LDS for everybody.
+                asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(YOUNGER) : "memory");
+                issue_weights(wnext, rd_stage);
+                wnext = wnext + 1 == a.ksteps ? 0 : wnext + 1;
+                if constexpr (S < PSTEPS) {
 #pragma unroll
-                for (int mt = 0; mt < MT; ++mt) {
-                    if (mt + 2 < MT) fa[(mt + 2) & 3] = st[(mt + 2) * 16];
-#pragma unroll
-                    for (int nt = 0; nt < NT; ++nt)
-                        acc[mt][nt] = __builtin_amdgcn_mfma_i32_16x16x64_i8(fa[mt & 3], fb[nt], acc[mt][nt], 0, 0, 0);
-                    step_fence();
-                    if (mt == BAR_MT) {
-                        // behind this barrier the next step's weights and (at a block's last step) the next patch are
-                        // in LDS for every wave, and nobody reads the ring stage of the previous step any more
-                        if constexpr (DBG & 1) { if constexpr (!(DBG & 2)) asm volatile("s_barrier" ::: "memory"); }
-                        else if constexpr (DBG & 2) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(YOUNGER) : "memory");
-                        else asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(YOUNGER) : "memory");
-                        const int nx_stage = rd_stage + 1 == R ? 0 : rd_stage + 1;
-                        const int wr_stage = rd_stage == 0 ? R - 1 : rd_stage - 1;
-                        if constexpr (!(DBG & 4)) issue_weights(wnext, wr_stage);
-                        wnext = wnext + 1 == a.ksteps ? 0 : wnext + 1;
-                        if constexpr (S < PSTEPS && !(DBG & 8)) {
-#pragma unroll
-                            for (int i = 0; i < PL; ++i) issue_patch((S * WAVES + wave) * PL + i, tile_n, cb_n, pbuf ^ 1);
-                        }
-                        step_fence();
-                        // first fragments of the next step
-                        const int nbuf = S == TAPS - 1 ? pbuf ^ 1 : pbuf;
-                        const v4i* pt = patch + nbuf * patch_v4 + b_lane + h.tap[(S + 1) % TAPS];
-                        const v4i* sn = ring + nx_stage * STAGE + a_lane;
-#pragma unroll
-                        for (int nt = 0; nt < NT; ++nt) fbn[nt] = pt[nt * 16];
-                        fa[0] = sn[0];
-                        fa[1] = sn[16];
-                        step_fence();
-                    }
+                    for (int i = 0; i < PL; ++i) issue_patch((S * WAVES + wave) * PL + i, tile_n, cb_n, pbuf ^ 1);
                 }
-                rd_stage = rd_stage + 1 == R ? 0 : rd_stage + 1;
+                step_fence();
+                mma(7);
+                step_fence();
+                rd_stage = nx_stage;
             });
             pbuf ^= 1;
         }
-
-        // ---- requantise and store the tile: lane (kq, l16) holds 16 consecutive features of one position per fragment
-        uint32_t ob[NT], eb[NT];
-        PixelPos pos[NT];
-        bool ok[NT];
+        // the compiler's own waits in the epilogue count LDS and scalar-memory returns together: start it with nothing of
+        // ours outstanding (the first fragments of the next tile, requested above)
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        // ---- requantise and store the tile: a lane holds 16 consecutive features of one position per tile
 #pragma unroll
         for (int nt = 0; nt < NT; ++nt) {
-            const uint32_t q = (uint32_t)tile * BM + (uint32_t)(wave_p * NT * 16 + nt * 16 + l16);
+            const uint32_t q = (uint32_t)tile * BM + (uint32_t)(wave_p * NT * 32 + nt * 32 + l32);
             const uint32_t b = h.div_yxp.div(q);
             const uint32_t r = q - b * (uint32_t)h.YXp;
             const uint32_t yp = h.div_wp.div(r);
             const int oy = (int)yp - h.pad_lo_y, ox = (int)(r - yp * (uint32_t)h.Wp) - h.pad_lo_x;
-            ok[nt] = q < (uint32_t)h.pos_total && (uint32_t)oy < (uint32_t)a.OH && (uint32_t)ox < (uint32_t)a.OW;
-            pos[nt] = PixelPos{b, (uint32_t)oy, (uint32_t)ox};
-            ob[nt] = (uint32_t)(a.out_off + (int)b * a.out_pb + oy * a.out_py + ox * 16);
-            eb[nt] = (uint32_t)(a.el_off + (int)b * a.el_pb + oy * a.esy * a.el_py + ox * a.esx * 16);
-        }
+            const bool ok = q < (uint32_t)h.pos_total && (uint32_t)oy < (uint32_t)a.OH && (uint32_t)ox < (uint32_t)a.OW;
+            if (!ok) continue;
+            const int ob = a.out_off + (int)b * a.out_pb + oy * a.out_py + ox * 16;
+            const int eb = a.el_off + (int)b * a.el_pb + oy * a.esy * a.el_py + ox * a.esx * 16;
 #pragma unroll
-        for (int sp = 0; sp < SPANS; ++sp) {
-            const int f0 = ntile * BN + (wave_f * SPANS + sp) * 64 + kq * 16;
-            if (f0 >= a.OFM) continue;
-            const int fs = f0 >> 4;
-            const int valid = a.OFM - f0;
-            LaneScales sc;
-            load_scales<EPI>(a, f0, sc);
-            const v4i(&acc_sp)[4][NT] = *reinterpret_cast<const v4i(*)[4][NT]>(&acc[sp * 4]);
+            for (int mt = 0; mt < MT; ++mt) {
+                const int f0 = ntile * BN + (wave_f * MT + mt) * 32 + half * 16;
+                if (f0 >= a.OFM) continue;
+                const int fs = f0 >> 4;
+                const int valid = a.OFM - f0;
+                LaneScales sc;
+                load_scales<EPI>(a, f0, sc);
+                v4i one[4][1];
 #pragma unroll
-            for (int nt = 0; nt < NT; ++nt) {
-                if (ok[nt]) {
-                    const int obase = (int)ob[nt] + fs * a.out_pf, ebase = (int)eb[nt] + fs * a.el_pf;
-                    v4i ev4 = {0, 0, 0, 0};
-                    if constexpr (EPI == EPI_KIND_FUSED) ev4 = *reinterpret_cast<const v4i*>((const int8_t*)a.eltw + ebase);
-                    else if constexpr (EPI == EPI_KIND_FAST)
-                        if (a.fe.fused) ev4 = *reinterpret_cast<const v4i*>((const int8_t*)a.eltw + ebase);
-                    finish_pixel<NT, EPI>(a, acc_sp, nt, f0, valid, obase, ebase, sc, ev4, pos[nt].b, pos[nt].oy, pos[nt].ox);
-                }
+                for (int c = 0; c < 16; ++c) one[c >> 2][0][c & 3] = acc[mt][nt][c];
+                const int obase = ob + fs * a.out_pf, ebase = eb + fs * a.el_pf;
+                v4i ev4 = {0, 0, 0, 0};
+                if constexpr (EPI == EPI_KIND_FUSED) ev4 = *reinterpret_cast<const v4i*>((const int8_t*)a.eltw + ebase);
+                else if constexpr (EPI == EPI_KIND_FAST)
+                    if (a.fe.fused) ev4 = *reinterpret_cast<const v4i*>((const int8_t*)a.eltw + ebase);
+                finish_pixel<1, EPI>(a, one, 0, f0, valid, obase, ebase, sc, ev4, b, (uint32_t)oy, (uint32_t)ox);
             }
         }
         reset_acc();
@@ -242,7 +307,7 @@ __global__ void __launch_bounds__(WP * WF * 64) conv_halo_kernel(HaloArgs h)
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 }
 
-template <int MT, int NT, int WP, int WF, int R, int PL, int DBG = 0>
+template <int MT, int NT, int WP, int WF, int R, int PL>
 void launch_halo_instance(hipStream_t s, const HaloArgs& h, int grid, int lds, int epi)
 {
     const dim3 g(grid), b(WP * WF * 64);
@@ -250,10 +315,10 @@ void launch_halo_instance(hipStream_t s, const HaloArgs& h, int grid, int lds, i
     {                                                                                                               \
         static std::once_flag allowed;                                                                              \
         std::call_once(allowed, [] {                                                                                \
-            CHIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(&conv_halo_kernel<MT, NT, WP, WF, R, PL, KIND, DBG>), \
+            CHIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(&conv_halo_kernel<MT, NT, WP, WF, R, PL, KIND>), \
                                            hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));                \
         });                                                                                                         \
-        hipLaunchKernelGGL((conv_halo_kernel<MT, NT, WP, WF, R, PL, KIND, DBG>), g, b, lds, s, h);                       \
+        hipLaunchKernelGGL((conv_halo_kernel<MT, NT, WP, WF, R, PL, KIND>), g, b, lds, s, h);                       \
     }
     switch (epi) {
     case EPI_KIND_RELU: HALO_LAUNCH(EPI_KIND_RELU) break;

@@ -63,10 +63,8 @@ static const TileConfig g_tiles[] = {
     {"stem_p64", 64, 64, 64},
     // nine-tap stride-1 kernel with both operands in LDS (direct global -> LDS loads); persistent workgroups; a wave
     // owns 64 positions x 128 features.  tile_pixels counts positions of the bordered input.
-    {"halo_p256_f128", 256, 128, 64},   // 4 waves
-    {"halo_p128_f128", 128, 128, 64},   // 2 waves
-    {"halo_p128_f256", 128, 256, 64},   // 4 waves, 2 x 2
-    {"halo_p256_f256", 256, 256, 64},   // 8 waves, 4 x 2
+    {"halo_p256_f128", 256, 128, 64},   // 4 waves, two workgroups per CU
+    {"halo_p512_f128", 512, 128, 64},   // 8 waves, one workgroup per CU (rows too long for two patches of 256 + halo in 80 KB)
 };
 enum { FIRST_STREAM_ROW = 6, FIRST_BDIR_ROW = 8, FIRST_WSL_ROW = 14, FIRST_BDIRK_ROW = 17, STEM_ROW = 20, GEMV_ROW = 21, STEM_P64_ROW = 22, FIRST_HALO_ROW = 23 };
 enum { HALO_RING = 4, HALO_TAPS = 9 };
@@ -115,7 +113,7 @@ enum {
     ROW_BDIR_P64_F64 = 8, ROW_BDIR_P128_F64 = 9, ROW_BDIR_P256_F64 = 10, ROW_BDIR_P64_F128 = 11, ROW_BDIR_P128_F128 = 12,
     ROW_BDIR_P256_F128 = 13, ROW_WSL_P64 = 14, ROW_WSL_P128 = 15, ROW_WSL_P256 = 16,
     ROW_BDIR_K2_P64_F64 = 17, ROW_BDIR_K4_P64_F64 = 18, ROW_BDIR_K2_P128_F64 = 19, ROW_STEM_P32 = 20, ROW_GEMV = 21, ROW_STEM_P64 = 22,
-    ROW_HALO_P256_F128 = 23, ROW_HALO_P128_F128 = 24, ROW_HALO_P128_F256 = 25, ROW_HALO_P256_F256 = 26
+    ROW_HALO_P256_F128 = 23, ROW_HALO_P512_F128 = 24
 };
 
 static int choose_lds_tile(const ConvProblem& p, int64_t m, int cus)
@@ -260,8 +258,8 @@ MfmaPlan mfma_plan(const ConvProblem& p, int tile, int cus)
         pl.block = waves * 64;
         pl.halo_patch_len = (tc.tile_pixels + halo_lo + halo_hi + 63) / 64 * 64;
         pl.halo_ptiles = (int)((pos_total + tc.tile_pixels - 1) / tc.tile_pixels);
-        // the next block's patch is requested in six steps of the current one, by every wave
-        const int slots = (HALO_TAPS - 1 - (HALO_RING - 2)) * waves;
+        // the next block's patch is requested in five steps of the current one, by every wave
+        const int slots = (HALO_TAPS - HALO_RING) * waves;
         pl.halo_pl = (4 * (pl.halo_patch_len / 64) + slots - 1) / slots;
         CHIP_REQUIRE(pl.halo_pl <= 2, CLDNN_HIP_UNSUPPORTED_SIZE, "rows too long for the staged-patch kernel's request slots");
     }
@@ -330,6 +328,11 @@ void mfma_pack_weights(const ConvProblem& p, const MfmaPlan& pl, const int8_t* w
     std::memset(packed, 0, pl.packed_bytes);
     auto row_of = [&](int f) {
         const int fl = f % BN, span = fl / 64, o = fl % 64;
+        if (pl.halo) {
+            // 32-row tiles of the 32x32x32 matrix instruction: row 8g + 4h + i holds feature 16h + 4g + i of the tile
+            const int tile = fl / 32, q = fl % 32;
+            return tile * 32 + ((q % 16) / 4) * 8 + (q / 16) * 4 + (q % 4);
+        }
         return span * 64 + ((o % 16) / 4) * 16 + (o / 16) * 4 + (o % 4);  // permuted row inside the span
     };
     if (pl.stem) {

@@ -211,6 +211,10 @@ def test_mfma_kernel_all_tiles(eng, shape, in_dt):
                 with pytest.raises(hip.HipError):  # the first-layer row goes with b_fs_yx_fsv4 input
                     hip.conv_forward(eng, x, w, bias, wqf, calib, **kw)
                 continue
+            if tile and names[tile - 1].startswith("halo") and (no_border or -(-IFM // 16) % 4 != 0 or (FY, FX) != (3, 3) or stride != (1, 1)):
+                with pytest.raises(hip.HipError):  # nine taps, stride 1, constant tap offsets, feature slices in fours
+                    hip.conv_forward(eng, x, w, bias, wqf, calib, **kw)
+                continue
             if tile and names[tile - 1].startswith(("bdir", "wsl", "gemv")) and (no_border or -(-IFM // 16) % 4 != 0):
                 with pytest.raises(hip.HipError):  # needs constant tap offsets and feature slices in fours
                     hip.conv_forward(eng, x, w, bias, wqf, calib, **kw)
@@ -225,8 +229,78 @@ def test_mfma_kernel_all_tiles(eng, shape, in_dt):
     assert any("stream" in n for n in seen) == (-(-(FY * FX * -(-IFM // 16)) // 4) <= 8)
     assert any("bdir" in n for n in seen) == (-(-IFM // 16) % 4 == 0)
     assert any("wsl" in n for n in seen) == (-(-IFM // 16) % 4 == 0)
+    assert any("halo" in n for n in seen) == (-(-IFM // 16) % 4 == 0 and (FY, FX) == (3, 3) and stride == (1, 1))
     if pad != (0, 0):
         assert any("checked" in n for n in seen)
+
+
+HALO_SHAPES = [
+    # B IFM H  W  OFM pad dilation border(y, x)
+    (2, 128, 56, 56, 256, (1, 1), (1, 1), (1, 1)),   # several position tiles per image, two feature blocks, two feature tiles
+    (40, 64, 9, 11, 128, (1, 1), (1, 1), (1, 1)),    # tiles that span several images; one feature block
+    (1, 64, 6, 150, 128, (1, 1), (1, 1), (1, 1)),    # long rows: the halo exceeds the tile, two patch requests per wave and step
+    (1, 64, 5, 200, 128, (1, 1), (1, 1), (1, 1)),    # rows too long for the 256-position row's request slots
+    (3, 192, 20, 20, 200, (1, 1), (1, 1), (2, 3)),   # border wider than the padding; partly filled last feature tile
+    (2, 64, 17, 15, 64, (2, 2), (2, 2), (2, 2)),     # dilated filter
+    (1, 64, 12, 12, 96, (0, 0), (1, 1), (0, 0)),     # no padding: the output is smaller than the input
+    (17, 256, 14, 14, 128, (1, 1), (1, 1), (1, 1)),  # four feature blocks; more tiles than one round of workgroups per feature tile needs
+]
+
+
+@pytest.mark.parametrize("row", ["halo_p256_f128", "halo_p512_f128"])
+@pytest.mark.parametrize("shape", HALO_SHAPES, ids=lambda s: "x".join(map(str, s[:5])))
+@pytest.mark.parametrize("in_dt", [np.uint8, np.int8], ids=["u8", "s8"])
+def test_staged_patch_kernel(eng, shape, in_dt, row):
+    """the nine-tap stride-1 kernel with both operands in LDS: accumulators and every epilogue form against the oracle"""
+    B, IFM, H, W, OFM, pad, dil, border = shape
+    tile = tile_names().index(row) + 1
+    x, w, bias, wqf, calib = problem(61, B, IFM, H, W, OFM, 3, 3, in_dt)
+    base = dict(pad=pad, dilation=dil, fmt="fs_b_yx_fsv16", in_pad=border, tile=tile, want_info=True)
+    plain = dict(pad=pad, dilation=dil)
+    if W == 200 and row == "halo_p256_f128":
+        with pytest.raises(hip.HipError, match="rows too long"):
+            hip.conv_forward(eng, x, w, bias, wqf, calib, out_dt="s8", act="relu", **base)
+        return
+    # requantised with relu (the short branch-free form) + raw accumulators
+    ref_o, ref_a = rc.conv(x, w, bias, wqf=wqf, calib=calib, out_dt="s8", act="relu", want_acc=True, **plain)
+    go, ga, info = hip.conv_forward(eng, x, w, bias, wqf, calib, out_dt="s8", act="relu", want_acc=True, **base)
+    assert info.impl == hip.IMPL_MFMA and info.kernel_name.decode().startswith("conv_halo<" + row), info.kernel_name
+    np.testing.assert_array_equal(ga, ref_a)
+    assert_same(ref_o, go)
+    # no activation, unsigned output, into a buffer with a border of its own
+    ref = rc.conv(x, w, bias, wqf=wqf, calib=calib, out_dt="u8", **plain)
+    assert_same(ref, hip.conv_forward(eng, x, w, bias, wqf, calib, out_dt="u8", out_pad=(1, 2), **base)[0])
+    # the run-time form (weight factors other than one) and the element-wise one (float output)
+    wq2 = (wqf * np.random.default_rng(5).uniform(0.5, 2.0, OFM)).astype(np.float32)
+    ref = rc.conv(x, w, bias, wqf=wq2, calib=calib, out_dt="s8", act="clamp", act_m=-1000.0, act_n=3000.0, **plain)
+    assert_same(ref, hip.conv_forward(eng, x, w, bias, wq2, calib, out_dt="s8", act="clamp", act_m=-1000.0, act_n=3000.0, **base)[0])
+    ref = rc.conv(x, w, bias, wqf=wq2, calib=calib, out_dt="f32", act="relu", **plain)
+    assert_same(ref, hip.conv_forward(eng, x, w, bias, wq2, calib, out_dt="f32", act="relu", **base)[0])
+    # fused residual sum with relu
+    OH, OW = ref.shape[2:]
+    e = np.random.default_rng(6).integers(-128, 128, (B, OFM, OH, OW)).astype(np.int8)
+    ecal = np.random.default_rng(7).uniform(0.3, 1.2, OFM).astype(np.float32)
+    kw = dict(out_dt="s8", act="none", eltw=e, eltw_act="relu", eltw_calib=ecal)
+    ref = rc.conv(x, w, bias, wqf=wqf, calib=calib, **kw, **plain)
+    got, info = hip.conv_forward(eng, x, w, bias, wqf, calib, **kw, **base)
+    assert "fast" in info.kernel_name.decode()
+    assert_same(ref, got)
+
+
+def test_staged_patch_kernel_refuses_what_it_cannot_run(eng):
+    tile = tile_names().index("halo_p256_f128") + 1
+    x, w, bias, wqf, calib = problem(62, 1, 64, 12, 12, 64, 3, 3)
+    kw = dict(out_dt="s8", fmt="fs_b_yx_fsv16", tile=tile)
+    for bad in (dict(pad=(1, 1), in_pad=(0, 0)),                      # no border: tap offsets are not constant
+                dict(pad=(1, 1), in_pad=(1, 1), stride=(2, 2))):      # stride
+        with pytest.raises(hip.HipError):
+            hip.conv_forward(eng, x, w, bias, wqf, calib, **kw, **bad)
+    x1, w1, b1, q1, c1 = problem(63, 1, 64, 12, 12, 64, 1, 1)
+    with pytest.raises(hip.HipError):                                 # one tap
+        hip.conv_forward(eng, x1, w1, b1, q1, c1, **kw)
+    x2, w2, b2, q2, c2 = problem(64, 1, 32, 12, 12, 64, 3, 3)
+    with pytest.raises(hip.HipError):                                 # 32 input features: not a whole block of 64
+        hip.conv_forward(eng, x2, w2, b2, q2, c2, pad=(1, 1), in_pad=(1, 1), **kw)
 
 
 @pytest.mark.parametrize("out_dt", ["s8", "u8", "f32"])
@@ -299,7 +373,7 @@ def test_residual_read_from_the_output_buffer(eng, out_dt, e_dt):
     kw = dict(out_dt=out_dt, act="none", eltw=e, eltw_act="relu", eltw_calib=ecal)
     ref = rc.conv(x, w, bias, wqf=wqf, calib=calib, **kw)
     seen = set()
-    for tile in [0] + [t for t in tiles() if not tile_names()[t - 1].startswith("stem")]:
+    for tile in [0] + [t for t in tiles() if not tile_names()[t - 1].startswith(("stem", "halo"))]:
         out, info = hip.conv_forward(eng, x, w, bias, wqf, calib, fmt="fs_b_yx_fsv16", tile=tile, in_place=True, want_info=True, **kw)
         seen.add(info.kernel_name.decode().split("<")[0])
         assert_same(ref, out)
@@ -335,7 +409,7 @@ def test_fused_sum_that_keeps_the_convolution_saturation(eng, in_dt):
     assert 0.02 < (ref != unsaturated).mean() < 0.9  # the two forms do differ on this data
     kw = dict(out_dt="s8", act="none", eltw=e, eltw_act="none", eltw_calib=ecal, conv_saturate=1)
     seen = set()
-    for tile in [0] + [t for t in tiles() if not tile_names()[t - 1].startswith("stem")]:
+    for tile in [0] + [t for t in tiles() if not tile_names()[t - 1].startswith(("stem", "halo"))]:
         out, info = hip.conv_forward(eng, x, w, bias, wqf, calib, fmt="fs_b_yx_fsv16", tile=tile, want_info=True, **kw)
         seen.add(info.kernel_name.decode().split("<")[0])
         assert_same(ref, out)
@@ -384,7 +458,7 @@ def test_mfma_fused_eltwise(eng, fast, eltw_dt):
     ecal = r.uniform(0.3, 1.2, 256).astype(np.float32)
     kw = dict(out_dt="s8", act="none", eltw=e, eltw_act="relu", eltw_calib=ecal,
               non_conv_scale=1.0 if fast else 0.5)
-    for tile in [0] + [t for t in tiles() if not tile_names()[t - 1].startswith("stem")]:
+    for tile in [0] + [t for t in tiles() if not tile_names()[t - 1].startswith(("stem", "halo"))]:
         (ro, ra), (go, ga, info) = both(eng, x, w, bias, wqf, calib, fmt="fs_b_yx_fsv16", tile=tile, **kw)
         assert (b"fast" in info.kernel_name) == (fast and b"gemv" not in info.kernel_name)  # the small-batch kernel has one epilogue
         np.testing.assert_array_equal(ga, ra)
@@ -416,7 +490,7 @@ def test_fused_eltwise_read_with_stride(eng, shape, es):
     for fmt, impl in (("bfyx", hip.IMPL_REF), ("fs_b_yx_fsv16", hip.IMPL_AUTO)):
         assert_same(ref, hip.conv_forward(eng, x, w, bias, wqf, calib, fmt=fmt, impl=impl, **kw))
     seen = set()
-    for tile in [t for t in tiles() if not tile_names()[t - 1].startswith("stem")]:
+    for tile in [t for t in tiles() if not tile_names()[t - 1].startswith(("stem", "halo"))]:
         try:
             got, info = hip.conv_forward(eng, x, w, bias, wqf, calib, fmt="fs_b_yx_fsv16", tile=tile, want_info=True,
                                          in_pad=(pad[0] + (1 if FY > 1 else 0), pad[1]), **kw)
