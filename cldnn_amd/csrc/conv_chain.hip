@@ -71,7 +71,7 @@ std::string chain_plan(const ChainStageIn* st, int n, int cus, ChainPlan* out)
         if (p.in_t.format != CLDNN_HIP_FMT_FS_B_YX_FSV16 || p.out_t.format != CLDNN_HIP_FMT_FS_B_YX_FSV16) return at + "needs fs_b_yx_fsv16";
         if (st[0].dw_wmask == nullptr && (p.IFM % 64 != 0 || p.OFM % 64 != 0)) return at + "feature counts must be multiples of 64";
         if (st[0].dw_wmask != nullptr && k < 2 && p.IFM % 16 != 0) return at + "a depthwise chain needs feature counts in multiples of 16 up to the projection";
-        if (st[k].fe->fused && (p.esy != 1 || p.esx != 1 || p.eltw_t.format != CLDNN_HIP_FMT_FS_B_YX_FSV16)) return at + "strided or unblocked residual";
+        if (st[k].fe->fused && p.eltw_t.format != CLDNN_HIP_FMT_FS_B_YX_FSV16) return at + "unblocked residual";
         if (tensor_elems(p.out_t) >= (1ull << 31) || tensor_elems(p.in_t) >= (1ull << 31)) return at + "tensor of 2 GiB or more";
         if (k > 0) {
             const ConvProblem& q = *st[k - 1].p;
@@ -179,7 +179,8 @@ static void fill_stage(ChainStage& c, const ChainStageIn& in, const ChainPlan& p
     CHIP_REQUIRE(!in.fe->fused || c.eltw, CLDNN_HIP_INVALID_ARG, "fused stage of a chain without its second input");
     c.OFM = p.OFM;
     c.out_off = (int32_t)p.out_p.off, c.out_pb = (int32_t)p.out_p.pb, c.out_pf = (int32_t)p.out_p.pf, c.out_py = (int32_t)p.out_p.py;
-    c.el_off = (int32_t)p.eltw_p.off, c.el_pb = (int32_t)p.eltw_p.pb, c.el_pf = (int32_t)p.eltw_p.pf, c.el_py = (int32_t)p.eltw_p.py;
+    c.el_off = (int32_t)p.eltw_p.off, c.el_pb = (int32_t)p.eltw_p.pb, c.el_pf = (int32_t)p.eltw_p.pf;
+    c.el_py = (int32_t)p.eltw_p.py * p.esy, c.el_px = 16 * p.esx;  // a strided residual: the shortcut sub-sampled in place
     c.xor_mask = p.in_dt == CLDNN_HIP_U8 ? 0x80808080u : 0u;
     c.unit0 = pl.unit0[k], c.kstride = pl.kstride[k], c.vec0 = pl.vec0[k];
     c.fe = *in.fe;

@@ -29,7 +29,7 @@ struct ChainStage {
     const void* eltw;          // residual operand of a fused stage
     int32_t OFM;
     int32_t out_off, out_pb, out_pf, out_py;  // elements
-    int32_t el_off, el_pb, el_pf, el_py;      // elements
+    int32_t el_off, el_pb, el_pf, el_py, el_px;  // elements; el_py / el_px carry the residual's stride (a sub-sampled shortcut)
     uint32_t xor_mask;         // applied to the fragments this stage READS (0x80808080: its input is u8)
     int32_t unit0;             // first 4 KB weight unit of the stage inside the LDS image
     int32_t kstride;           // units per 64-feature span (K-steps incl. zero padding)
@@ -178,7 +178,7 @@ __global__ void __launch_bounds__(256) conv_chain_kernel(ChainArgs a)
                 return st.out_off + (int)pp.b * st.out_pb + kq * st.out_pf + (int)pp.oy * st.out_py + (int)pp.ox * 16;
             };
             auto res = [&](const ChainStage& st) {
-                return st.el_off + (int)pp.b * st.el_pb + kq * st.el_pf + (int)pp.oy * st.el_py + (int)pp.ox * 16;
+                return st.el_off + (int)pp.b * st.el_pb + kq * st.el_pf + (int)pp.oy * st.el_py + (int)pp.ox * st.el_px;
             };
             r.o0[nt] = ok && s0.out ? at(s0) : -1;
             r.o1[nt] = ok && s1.out ? at(s1) : -1;

@@ -113,7 +113,7 @@ __global__ void __launch_bounds__(256) conv_dwchain_kernel(DwChainArgs a)
             r.o0[nt] = ok && s0.out ? at(s0) : -1;
             r.o1[nt] = ok && s1.out ? at(s1) : -1;
             r.o2[nt] = HAS2 && ok && s2.out ? at(s2) : -1;
-            r.e1[nt] = s1.el_off + (int)pp.b * s1.el_pb + kq * s1.el_pf + (int)pp.oy * s1.el_py + (int)pp.ox * 16;
+            r.e1[nt] = s1.el_off + (int)pp.b * s1.el_pb + kq * s1.el_pf + (int)pp.oy * s1.el_py + (int)pp.ox * s1.el_px;
         }
     };
     // walk over the (K-step, tap) sequence of the activation requests: the lane's slice of K-step ks is 4 * ks + kq; a

@@ -120,6 +120,37 @@ def test_chain_equals_separate_convolutions_on_a_full_size_slice(eng):
     ch.close()
 
 
+@pytest.mark.parametrize("B,H,W", [(3, 14, 14), (2, 56, 56)], ids=["14x14", "56x56"])
+def test_chain_with_a_strided_head_and_a_sub_sampled_shortcut(eng, B, H, W):
+    """the last block of a ResNet stage after eltwise_remove_stride: the 3x3 takes the stride of the block behind it, the
+    closing 1x1 adds a shortcut that it reads with that stride (fused_conv_eltwise eltw_stride)"""
+    r = np.random.default_rng(77)
+    mid = 64
+    x = r.integers(0, 256, (B, mid, H, W)).astype(np.uint8)
+    xin = hip.upload(eng, x, "fs_b_yx_fsv16", (1, 1))
+    w0, b0, q0, c0 = layer(r, mid, mid, 3, np.uint8)
+    w1, b1, q1, c1 = layer(r, mid, 4 * mid, 1, np.int8)
+    OH, OW = (H + 1) // 2, (W + 1) // 2
+    shortcut = r.integers(-128, 128, (B, 4 * mid, H, W)).astype(np.int8)   # full resolution, read at every second pixel
+    ecal = r.uniform(0.25, 1.0, 4 * mid).astype(np.float32)
+    ebuf = hip.upload(eng, shortcut, "fs_b_yx_fsv16")
+    d0 = hip.conv_desc(xin.tensor, w0.shape, "s8", stride=(2, 2), pad=(1, 1), bias_dt=hip.I32, has_wqf=True, has_calib=True, act="relu")
+    mid_t = hip.Tensor.make(hip.S8, hip.FS_B_YX_FSV16, B, mid, OH, OW)
+    d1 = hip.conv_desc(mid_t, w1.shape, "s8", bias_dt=hip.I32, has_wqf=True, has_calib=True, act="none", eltw_t=ebuf.tensor, eltw_act="relu",
+                       has_eltw_calib=True, eltw_stride=(2, 2))
+    ref0 = rc.conv(x, w0, b0, wqf=q0, calib=c0, stride=(2, 2), pad=(1, 1), out_dt="s8", act="relu")
+    ref1 = rc.conv(ref0, w1, b1, wqf=q1, calib=c1, out_dt="s8", act="none", eltw=shortcut, eltw_act="relu", eltw_calib=ecal, eltw_stride=(2, 2))
+    assert ref1.shape == (B, 4 * mid, OH, OW)
+    ch = hip.ConvChain(eng, [(d0, w0, b0, q0, c0, None), (d1, w1, b1, q1, c1, ecal)], [False, True])
+    out = hip.Buffer(eng, d1.output)
+    ch.enqueue(xin, [None, out], [None, ebuf])
+    eng.finish()
+    got = hip.download(eng, out)
+    bad = np.argwhere(got != ref1)
+    assert bad.size == 0, "%d of %d differ, first at %s" % (len(bad), got.size, bad[0])
+    ch.close(), xin.close(), out.close(), ebuf.close()
+
+
 def test_chain_refusals(eng):
     xin, spec, bufs, refs = bottleneck_tail(eng, 9, 1, 8, 8, 64, 3, True)
     # a second stage that is not 1x1
