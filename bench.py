@@ -405,6 +405,38 @@ def network_workload(args):
         in_flight = {"requests": len(nets), "steps_per_request": args.steps, "images_per_s": len(nets) * batch * args.steps / dt2,
                      "ms_per_request_step": dt2 / args.steps * 1e3,
                      "what": "independent requests: one network, engine (HIP stream at default priority) and host thread each"}
+    cpu, verified = None, None
+    if not args.no_cpu and args.cpu_seconds > 0:
+        # the same network through the CPU oracle, layer by layer, on the first images of the batch: a bounded sample
+        # (one image as a probe, then as many as the time budget holds) and a bit-exact check of the logits
+        from oracle import networks as oracle_networks
+        from oracle import refconv as rc
+        fused = [n["id"].split("_fused_")[1] for n in cl.plan(topo, opts) if "_fused_" in n["id"]]
+
+        def oracle_logits(xs):
+            if resnet:
+                return oracle_networks.resnet50(xs, params, fused=fused)[out_id]
+            if vgg:
+                return oracle_networks.vgg16(xs, params)[out_id]
+            return oracle_networks.mobilenet_v2(xs, params, folded=True)[out_id]
+        t1 = time.perf_counter()
+        ref = oracle_logits(x[:1])
+        seconds, images = time.perf_counter() - t1, 1
+        more = max(1, min(batch, int(args.cpu_seconds / max(seconds, 1e-3))))
+        if more > 1:
+            t1 = time.perf_counter()
+            ref = oracle_logits(x[:more])
+            seconds, images = time.perf_counter() - t1, more
+        threads = rc.lib().rc_threads_available()
+        mismatches = int((logits[:images] != ref).sum())
+        cpu = {"value": images / seconds, "unit": "images/s", "cores": threads, "kind": "port",
+               "sample": "first %d image(s) of the batch through every layer of the network in oracle/refconv.c (OpenMP over "
+                         "batch x ofm), %.1f s on %d threads = %.0f s of CPU work" % (images, seconds, threads, seconds * threads)}
+        verified = {"outputs_compared": int(ref.size), "mismatches": mismatches,
+                    "what": "logits of the first %d image(s) of the batch-%d execute() (they depend on every layer) vs the CPU "
+                            "oracle run layer by layer (bit-exact)" % (images, batch)}
+        if mismatches:
+            log("PARITY FAILURE in %s: %d mismatching logits" % (args.workload, mismatches))
     # multiply-adds the kernels execute: the graph passes let the layers in front of a stride-2 block compute only what
     # that block reads, so this can be less than the model's nominal count
     nominal = 2.0 * batch * (workloads.macs(layers) + sum(k * ofm for _, k, ofm in fcs))
@@ -434,7 +466,10 @@ def network_workload(args):
                    "executed_ops_per_step": ops, "nominal_ops_per_step": nominal},
         "roofline": {"bound": "mfma", "achieved": ops * args.steps / dt / 1e12, "peak": PEAK_INT8_OPS / 1e12, "unit": "TOP/s",
                      "frac": ops * args.steps / dt / PEAK_INT8_OPS, "traffic": None, "kernel": "all kernels of one network.execute()"},
-        "requests_in_flight": in_flight, "cpu_baseline": None, "distinct_logit_values": int(len(np.unique(logits)))}), flush=True)
+        "requests_in_flight": in_flight, "cpu_baseline": cpu, "verified": verified,
+        "distinct_logit_values": int(len(np.unique(logits)))}), flush=True)
+    if verified and verified["mismatches"]:
+        sys.exit(1)
 
 
 def kernel_sources_digest():

@@ -2,6 +2,7 @@
 // tile choice (the gfx950 tile-config table stands where the reference has kernel_selector and
 // its tuning cache), weight pre-packing, launch.
 #include <algorithm>
+#include <chrono>
 #include <cstring>
 #include <vector>
 
@@ -565,7 +566,12 @@ static float time_candidate(cldnn_hip_engine e, cldnn_hip_conv_desc d, int tile_
     try {
         CHIP_CHECK(hipEventCreate(&t0));
         CHIP_CHECK(hipEventCreate(&t1));
-        for (int i = 0; i < 3; ++i) run(c, in, out, eltw, nullptr);
+        // creating the candidate left the device idle for a while: bring its clocks back up before timing
+        const auto start = std::chrono::steady_clock::now();
+        do {
+            for (int i = 0; i < 10; ++i) run(c, in, out, eltw, nullptr);
+            CHIP_CHECK(hipStreamSynchronize(e->stream));
+        } while (std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now() - start).count() < 20.0);
         for (int batch = 0; batch < 3; ++batch) {
             CHIP_CHECK(hipEventRecord(t0, e->stream));
             for (int i = 0; i < runs; ++i) run(c, in, out, eltw, nullptr);
@@ -586,6 +592,24 @@ static float time_candidate(cldnn_hip_engine e, cldnn_hip_conv_desc d, int tile_
     (void)hipEventDestroy(t1);
     cldnn_hip_conv_release(c);
     return best;
+}
+
+static void warm_device(cldnn_hip_engine e, const cldnn_hip_conv_desc& d, const void* weights, const void* bias, const float* wqf,
+                        const float* calib, const float* eltw_calib, const void* in, void* out, const void* eltw, double milliseconds)
+{
+    cldnn_hip_conv c = nullptr;
+    if (cldnn_hip_conv_create(e, &d, weights, bias, wqf, calib, eltw_calib, &c) != CLDNN_HIP_SUCCESS) return;
+    try {
+        const auto start = std::chrono::steady_clock::now();
+        do {
+            for (int i = 0; i < 20; ++i) run(c, in, out, eltw, nullptr);
+            CHIP_CHECK(hipStreamSynchronize(e->stream));
+        } while (std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now() - start).count() < milliseconds);
+    } catch (...) {
+        cldnn_hip_conv_release(c);
+        throw;
+    }
+    cldnn_hip_conv_release(c);
 }
 
 cldnn_hip_status cldnn_hip_conv_tune(cldnn_hip_engine e, const cldnn_hip_conv_desc* desc, const void* weights, const void* bias,
@@ -626,6 +650,9 @@ cldnn_hip_status cldnn_hip_conv_tune(cldnn_hip_engine e, const cldnn_hip_conv_de
             CHIP_CHECK(hipMemcpy(in, host.data(), in_bytes, hipMemcpyHostToDevice));
             if (separate_eltw) CHIP_CHECK(hipMemcpy(eltw, host.data(), el_bytes, hipMemcpyHostToDevice));
             CHIP_CHECK(hipMemset(out, 0, out_bytes));
+            // the clocks of an idle device rise over tens of milliseconds: keep it busy first, or the candidates timed
+            // first (the table's own choice among them) lose against the later ones
+            warm_device(e, *desc, weights, bias, wqf, calib, eltw_calib, in, out, eltw, 150.0);
             const float base = time_candidate(e, *desc, 0, weights, bias, wqf, calib, eltw_calib, in, out, eltw, runs);
             CHIP_REQUIRE(base >= 0.0f, CLDNN_HIP_ERROR, std::string("the convolution cannot be created: ") + cldnn_hip_last_error());
             *best_tile_index = -1, *best_us = base;

@@ -169,15 +169,23 @@ int mfma_choose(const ConvProblem& p, int cus)
     if (m >= 50000) {
         // 256 and more features: 64 pixels x 128 features per wave, two waves per SIMD (3x3 at 56x56 with 128 / 256 input features)
         if (p.OFM >= 256 && p.OFM % 128 == 0) return ROW_BDIR_P256_F128;
-        if (ksteps <= 18) return ksteps <= 9 && p.OFM <= 128 ? ROW_WSL_P128 : ROW_WSL_P64;  // 3x3 at 56x56 .. 112x112
+        if (ksteps <= 18) return p.OFM <= 128 ? ROW_WSL_P128 : ROW_WSL_P64;  // 3x3 at 56x56 .. 224x224 with 64 / 128 input features
         return p.OFM >= 128 ? ROW_P256_F128 : ROW_BDIR_P256_F64;
     }
+    const int64_t grid_p128_f64 = ((m + 127) / 128) * ((p.OFM + 63) / 64);
     if (m >= 8192) {
-        if (p.OFM >= 512) return ksteps >= 64 ? ROW_BDIR_P128_F128 : ROW_BDIR_P256_F64;
+        if (p.OFM >= 512) {
+            if (m >= 20000 && p.OFM % 128 == 0) return ROW_BDIR_P256_F128;  // 3x3 at 28x28 with a batch of 32
+            return ksteps >= 64 ? ROW_BDIR_P128_F128 : ROW_BDIR_P256_F64;
+        }
+        if (ksteps <= 9 && m >= 32768) return ROW_WSL_P64;         // 64 input features under a 3x3 filter
+        if (ksteps >= 32 && m >= 16384) return ROW_BDIR_P256_F64;  // 3x3 at 56x56 with 256 features and a small batch
+        if (p.FY * p.FX > 1 && grid_p128_f64 <= cus) return ROW_BDIR_P64_F64;  // one workgroup per CU or fewer: halve the tile
         return ROW_BDIR_P128_F64;                                  // 3x3 at 28x28
     }
-    if (m >= 4096) return ROW_BDIR_P64_F64;                        // 14x14
-    if (ksteps >= 32) return m >= 2048 ? ROW_BDIR_K2_P128_F64 : ROW_BDIR_K2_P64_F64;  // few pixels, K >= 2048: split K
+    if (m >= 4096) return p.OFM >= 512 && ksteps >= 64 ? ROW_BDIR_P128_F64 : ROW_BDIR_P64_F64;  // 14x14
+    // few pixels, K >= 2048: split K; 128-pixel tiles when they still give three workgroups to every four CUs
+    if (ksteps >= 32) return m >= 2048 && grid_p128_f64 * 4 >= 3ll * cus ? ROW_BDIR_K2_P128_F64 : ROW_BDIR_K2_P64_F64;
     if (p.OFM > 2048 && m >= 512) return ROW_P64_F128;  // a 7x7 projection together with the block's opening 1x1
     if (p.OFM >= 1024 && m >= 512) return ROW_P128_F128;
     return ROW_BDIR_P64_F64;

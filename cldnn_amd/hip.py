@@ -507,6 +507,12 @@ class ConvChain:
             pass
 
 
+def tile_config_name(row):
+    """Name of row `row` (0-based) of the built-in tile table."""
+    name = lib().cldnn_hip_tile_config_name(row)
+    return None if name is None else name.decode()
+
+
 def conv_tune(engine, desc, w, bias=None, wqf=None, calib=None, eltw_calib=None, runs=20):
     """cldnn_hip_conv_tune: -> (best row or -1, its microseconds, microseconds of the table's own choice, per-row list)"""
     L = lib()

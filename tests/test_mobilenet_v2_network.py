@@ -5,52 +5,7 @@ import numpy as np
 import pytest
 
 from cldnn_amd import mobilenet_v2_net as mn
-from oracle import refconv as rc
-
-
-def run_oracle(x, params, folded=True, calibrate=False):
-    """Oracle forward pass.  folded: the clamp{0, 6} behind a convolution acts inside it on the dequantised value, before
-    the calibration (what optimize_data makes of the pair, as the reference's prepare_primitive_fusing does); otherwise
-    it is a primitive of its own and clamps the convolution's int8 output.  calibrate=True also chooses the factors:
-    the dequantised values of a ReLU6 layer get a root mean square of 3 and are requantised with 127 / 6; a linear
-    layer's outputs a root mean square of 30."""
-    t = {"input": x}
-    last = None
-    for step in mn.layer_plan():
-        if step[0] == "conv":
-            _, l, src = step
-            q, n = params[l["name"]], l["name"]
-            relu6 = l["act"] == "relu6"
-            kw = dict(stride=(l["stride"],) * 2, pad=(l["pad"],) * 2, groups=l["groups"], out_dt="s8")
-            if calibrate:
-                one = np.ones(l["ofm"], np.float32)
-                _, acc = rc.conv(t[src], q["w"], q["bias"], wqf=one, calib=one, want_acc=True, **kw)
-                full = acc.astype(np.float64) + q["bias"].reshape(1, -1, 1, 1)
-                rms = np.sqrt((full * full).mean(axis=(0, 2, 3))) + 1.0
-                q["wqf"] = ((3.0 if relu6 else 30.0) / rms).astype(np.float32)
-                q["calib"] = np.full(l["ofm"], 127.0 / 6.0 if relu6 else 1.0, np.float32)
-            if relu6 and folded:
-                t[n + "_relu6"] = rc.conv(t[src], q["w"], q["bias"], wqf=q["wqf"], calib=q["calib"], act="clamp", act_m=0.0, act_n=6.0, **kw)
-            else:
-                t[n] = rc.conv(t[src], q["w"], q["bias"], wqf=q["wqf"], calib=q["calib"], **kw)
-                if relu6:
-                    t[n + "_relu6"] = np.clip(t[n], 0, 6)  # the stand-alone activation clamps the int8 values themselves
-            last = n + ("_relu6" if relu6 else "")
-        elif step[0] == "sum":
-            _, n, shortcut, branch = step
-            if calibrate:
-                params[n] = dict(ecal=np.full(t[branch].shape[1], 0.75, np.float32))
-            t[n] = rc.eltwise([t[shortcut], t[branch]], "sum", calib=params[n]["ecal"])
-            last = n
-        elif step[0] == "pool":
-            t["pool"] = rc.pool(t[last], "average", None, global_pooling=True)
-        else:
-            q = params["fc1000"]
-            if calibrate:
-                acc = np.einsum("bfyx,ofyx->bo", t["pool"].astype(np.int64), q["w"].astype(np.int64)).astype(np.float64)
-                q["calib"] = np.full(q["w"].shape[0], 40.0 / (np.sqrt((acc * acc).mean()) + 1.0), np.float32)
-            t["fc1000"] = rc.fully_connected(t["pool"], q["w"], q["bias"], wqf=q["wqf"], calib=q["calib"])
-    return t
+from oracle.networks import mobilenet_v2 as run_oracle
 
 
 def test_layer_plan_shape():

@@ -5,48 +5,7 @@ import pytest
 
 from cldnn_amd import resnet50_net as rn
 from oracle import refconv as rc
-
-
-def run_oracle(x, params, fused=(), calibrate=False):
-    """Oracle forward pass, layer by layer.  `fused` names the blocks whose residual sum runs inside the closing
-    convolution (fused_conv_eltwise: the convolution's result is not saturated before the sum); the others use the
-    stand-alone eltwise on the saturated int8 tensor.  With calibrate=True the pass also chooses every layer's factors:
-    the root mean square of its outputs lands at about a quarter of the int8 range (what a calibration tool does), so
-    that few values saturate and no layer dies.  Returns the tensors by primitive id."""
-    t = {"input": x}
-    for step in rn.layer_plan():
-        if step[0] == "conv":
-            _, l, src, relu = step
-            q = params[l["name"]]
-            kw = dict(stride=(l["stride"],) * 2, pad=(l["pad"],) * 2)
-            if calibrate:
-                _, acc = rc.conv(t[src], q["w"], q["bias"], wqf=q["wqf"], calib=np.ones(l["ofm"], np.float32), out_dt="s8", want_acc=True, **kw)
-                full = acc.astype(np.float64) + q["bias"].reshape(1, -1, 1, 1)
-                q["calib"] = (32.0 / (np.sqrt((full * full).mean(axis=(0, 2, 3))) + 1.0)).astype(np.float32)
-            if l["closes_block"] and l["name"][:-9] in fused:
-                continue  # computed together with the residual sum
-            t[l["name"]] = rc.conv(t[src], q["w"], q["bias"], wqf=q["wqf"], calib=q["calib"], out_dt="s8", act="relu" if relu else "none", **kw)
-        elif step[0] == "pool1":
-            t["pool1"] = rc.pool(t["conv1"], "max", (3, 3), (2, 2))
-        elif step[0] == "sum":
-            _, n, shortcut, branch = step
-            if calibrate:
-                params[n] = dict(ecal=np.full(params[branch]["w"].shape[0], 0.6, np.float32))
-            if n in fused:
-                q = params[branch]
-                t[n] = rc.conv(t[n + "_branch2b"], q["w"], q["bias"], wqf=q["wqf"], calib=q["calib"], out_dt="s8", eltw=t[shortcut],
-                               eltw_act="relu", eltw_calib=params[n]["ecal"])
-            else:
-                t[n] = rc.eltwise_sum(t[shortcut], t[branch], calib=params[n]["ecal"], relu=True)
-        elif step[0] == "pool5":
-            t["pool5"] = rc.pool(t["res5c"], "average", None, global_pooling=True)
-        else:
-            q = params["fc1000"]
-            if calibrate:
-                acc = np.einsum("bfyx,ofyx->bo", t["pool5"].astype(np.int64), q["w"].astype(np.int64)).astype(np.float64)
-                q["calib"] = np.full(q["w"].shape[0], 40.0 / (np.sqrt((acc * acc).mean()) + 1.0), np.float32)
-            t["fc1000"] = rc.fully_connected(t["pool5"], q["w"], q["bias"], wqf=q["wqf"], calib=q["calib"])
-    return t
+from oracle.networks import resnet50 as run_oracle
 
 
 BLOCKS = [s[1] for s in rn.layer_plan() if s[0] == "sum"]

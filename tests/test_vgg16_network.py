@@ -4,34 +4,7 @@ import numpy as np
 import pytest
 
 from cldnn_amd import vgg16_net as vg
-from oracle import refconv as rc
-
-
-def run_oracle(x, params, calibrate=False):
-    """Oracle forward pass; calibrate=True also chooses every layer's factors (root mean square of the outputs at about a
-    quarter of the int8 range)."""
-    t = {"input": x}
-    for step in vg.layer_plan():
-        if step[0] == "conv":
-            _, l, src = step
-            q = params[l["name"]]
-            if calibrate:
-                _, acc = rc.conv(t[src], q["w"], q["bias"], wqf=q["wqf"], calib=np.ones(l["ofm"], np.float32), pad=(1, 1), out_dt="s8", want_acc=True)
-                full = acc.astype(np.float64) + q["bias"].reshape(1, -1, 1, 1)
-                q["calib"] = (32.0 / (np.sqrt((full * full).mean(axis=(0, 2, 3))) + 1.0)).astype(np.float32)
-            t[l["name"]] = rc.conv(t[src], q["w"], q["bias"], wqf=q["wqf"], calib=q["calib"], pad=(1, 1), out_dt="s8", act="relu")
-        elif step[0] == "pool":
-            _, n, src = step
-            t[n] = rc.pool(t[src], "max", (2, 2), (2, 2))
-        else:
-            _, n, src, ifm, plane, ofm, relu = step
-            q = params[n]
-            xin = t[src].reshape(x.shape[0], ifm, plane, plane)
-            if calibrate:
-                acc = np.einsum("bfyx,ofyx->bo", xin.astype(np.int64), q["w"].astype(np.int64)).astype(np.float64)
-                q["calib"] = np.full(ofm, 40.0 / (np.sqrt((acc * acc).mean()) + 1.0), np.float32)
-            t[n] = rc.fully_connected(xin, q["w"], q["bias"], wqf=q["wqf"], calib=q["calib"], act="relu" if relu else "none")
-    return t
+from oracle.networks import vgg16 as run_oracle
 
 
 def test_layer_plan_shape():
