@@ -371,6 +371,9 @@ def network_workload(args):
         outs[out_id].get_event().wait()
         return outs
 
+    t0 = time.perf_counter()
+    while time.perf_counter() - t0 < CLOCK_WARMUP_SECONDS:  # see clock_warmup()
+        run()
     for _ in range(args.warmup):
         run()
     t0 = time.perf_counter()
@@ -460,6 +463,7 @@ def network_workload(args):
         "unit": "images/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": dt / args.steps * 1e3,
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "i8xi8->i32 (f32 requantisation)", "data": "synthetic",
         "config": {"workload": args.workload, "batch": batch, "primitives": primitives,
+                   "clock_warmup_s": CLOCK_WARMUP_SECONDS,
                    "build": "optimize_data" + (", tuning cache" if args.tuning_cache else "") + (", second stream" if args.second_stream else ""), "primitives_per_execute": len(executed), "launches_per_execute": len(executed) - len(followers) - len(paired),
                    "convolutions_in_a_neighbours_launch": len(paired),
                    "chained_convolutions": len(followers) + len({str(infos[i]["kernel"]) for i in followers}),
@@ -574,6 +578,21 @@ def kernel_rooflines(heads, times):
     return rows
 
 
+CLOCK_WARMUP_SECONDS = 0.3
+
+
+def clock_warmup(eng, step):
+    """The clocks of an idle device rise over tens of milliseconds of load (a layer timed right after idling runs
+    10 % and more slower than in a steady stream of work), and a short run (--steps 20 --warmup 5 is 15 ms) would be
+    timed on that ramp.  Untimed steps for CLOCK_WARMUP_SECONDS of wall time come first, then the W warm-up steps, then
+    exactly K timed steps; the JSON line names this under config.clock_warmup_s."""
+    t0 = time.perf_counter()
+    while time.perf_counter() - t0 < CLOCK_WARMUP_SECONDS:
+        for _ in range(5):
+            step()
+        eng.finish()
+
+
 def measure_stack(args, wl, steps, warmup, in_flight_n, cpu_seconds, extras):
     """Build one workload's stack, time `steps` whole steps, per-kernel times, optionally requests in flight and the
     CPU oracle leg (bounded sample + bit-exact check).  -> result dict, parity ok"""
@@ -594,6 +613,7 @@ def measure_stack(args, wl, steps, warmup, in_flight_n, cpu_seconds, extras):
 
     ops = sum(L.info.ops for L in heads)
     nbytes = sum(L.info.bytes for L in heads)
+    clock_warmup(eng, lambda: run_step(seq))
     for _ in range(warmup):
         run_step(seq)
     eng.finish()
@@ -715,7 +735,8 @@ def measure_stack(args, wl, steps, warmup, in_flight_n, cpu_seconds, extras):
                    "layers_in_a_neighbours_launch": sum(1 for L in stack if L.sibling is not None),
                    "layout": "fs_b_yx_fsv16",
                    "variant": "stride on the first 1x1 (Caffe form)" if wl.startswith("resnet50") else wl,
-                   "fused_residual_layers": sum(1 for L in stack if L.fused)},
+                   "fused_residual_layers": sum(1 for L in stack if L.fused),
+                   "clock_warmup_s": CLOCK_WARMUP_SECONDS},
         "achieved_tops": ops * steps / t_gpu / 1e12,
         "roofline": {
             "bound": "hbm" if hbm_bound else "mfma",
