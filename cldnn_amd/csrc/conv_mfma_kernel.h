@@ -172,11 +172,32 @@ __device__ __forceinline__ float rha(float v) { return truncf(v + copysignf(0.49
 __device__ __forceinline__ float med3(float x, float lo, float hi) { return __builtin_amdgcn_fmed3f(x, lo, hi); }
 __device__ __forceinline__ float relu1(float x) { return __builtin_amdgcn_fmed3f(x, 0.0f, __builtin_inff()); }
 
-// four values already inside [0, 255] -> one dword
-__device__ __forceinline__ int pack_nonneg(const float* v)
+// Sixteen values inside [0, 255.5) -> four dwords of bytes, one instruction per value.  v_cvt_pk_u8_f32 converts with
+// the wave's rounding mode and inserts the byte into a dword; with the mode set to round-toward-zero it gives, for every
+// float from -inf to +inf, what the truncating conversion of the value clamped to [0, 255] gives (all 2^32 bit patterns
+// but the NaNs were compared on the device).  Only the conversions run in that mode: the first asm takes every value as
+// an input, so the arithmetic that made them (rounded to nearest even, as the reference's) is complete before the mode
+// changes, and it hands out the zero that every dword starts from, so no conversion can start before it; the second asm
+// takes the four dwords.  The scheduling fences keep unrelated float arithmetic of the surrounding code out of the window.
+__device__ __forceinline__ void pack_nonneg16(const float (&v)[16], v4i& packed)
 {
-    const unsigned q0 = (unsigned)(int)v[0], q1 = (unsigned)(int)v[1], q2 = (unsigned)(int)v[2], q3 = (unsigned)(int)v[3];
-    return (int)(q0 | (q1 << 8) | (q2 << 16) | (q3 << 24));
+    unsigned w0, w1, w2, w3;
+    __builtin_amdgcn_sched_barrier(0);
+    asm volatile("s_setreg_imm32_b32 hwreg(HW_REG_MODE, 0, 2), 3\n\tv_mov_b32 %0, 0"
+                 : "=v"(w0)
+                 : "v"(v[0]), "v"(v[1]), "v"(v[2]), "v"(v[3]), "v"(v[4]), "v"(v[5]), "v"(v[6]), "v"(v[7]), "v"(v[8]), "v"(v[9]),
+                   "v"(v[10]), "v"(v[11]), "v"(v[12]), "v"(v[13]), "v"(v[14]), "v"(v[15]));
+    w1 = w2 = w3 = w0;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        w0 = __builtin_amdgcn_cvt_pk_u8_f32(v[i], i, w0);
+        w1 = __builtin_amdgcn_cvt_pk_u8_f32(v[4 + i], i, w1);
+        w2 = __builtin_amdgcn_cvt_pk_u8_f32(v[8 + i], i, w2);
+        w3 = __builtin_amdgcn_cvt_pk_u8_f32(v[12 + i], i, w3);
+    }
+    asm volatile("s_setreg_imm32_b32 hwreg(HW_REG_MODE, 0, 2), 0" : "+v"(w0), "+v"(w1), "+v"(w2), "+v"(w3));
+    __builtin_amdgcn_sched_barrier(0);
+    packed[0] = (int)w0, packed[1] = (int)w1, packed[2] = (int)w2, packed[3] = (int)w3;
 }
 // four values inside [-128, 255] -> one dword of bytes
 __device__ __forceinline__ int pack_signed(const float* v)
@@ -268,8 +289,7 @@ __device__ __forceinline__ v4i epilogue_fast16(const Args& a, const v4i (&acc)[4
         v4i packed;
 #pragma unroll
         for (int c = 0; c < 16; ++c) v[c] = med3(v[c] * wq[c], F.act_m, F.act_n) * cal[c] + 0.49999997f;
-#pragma unroll
-        for (int d = 0; d < 4; ++d) packed[d] = pack_nonneg(v + d * 4);
+        pack_nonneg16(v, packed);
         zero_padding_features(packed, valid);
         return packed;
     }
@@ -293,8 +313,7 @@ __device__ __forceinline__ v4i epilogue_fast16(const Args& a, const v4i (&acc)[4
 #pragma unroll
             for (int c = 0; c < 16; ++c) v[c] = med3(v[c] * ecal[c], 0.0f, F.hi) + 0.49999997f;
         }
-#pragma unroll
-        for (int d = 0; d < 4; ++d) packed[d] = pack_nonneg(v + d * 4);
+        pack_nonneg16(v, packed);
         zero_padding_features(packed, valid);
         return packed;
     }
@@ -317,8 +336,7 @@ __device__ __forceinline__ v4i epilogue_fast16(const Args& a, const v4i (&acc)[4
         // the host has checked to be inside the output range
 #pragma unroll
         for (int c = 0; c < 16; ++c) v[c] = med3(v[c], F.act_m, F.act_n) * cal[c] + 0.49999997f;
-#pragma unroll
-        for (int d = 0; d < 4; ++d) packed[d] = pack_nonneg(v + d * 4);
+        pack_nonneg16(v, packed);
     } else if (F.fc) {
         // reference fully_connected_gpu_bfyx_ref.cl:63-84: (char)round((acc * wqf * iqf + bias) * factor), then the
         // activation on the char; ecal[] holds the bias
@@ -339,8 +357,7 @@ __device__ __forceinline__ v4i epilogue_fast16(const Args& a, const v4i (&acc)[4
     } else if (F.relu_folded) {
 #pragma unroll
         for (int c = 0; c < 16; ++c) v[c] = med3(v[c] * cal[c], 0.0f, F.hi) + 0.49999997f;
-#pragma unroll
-        for (int d = 0; d < 4; ++d) packed[d] = pack_nonneg(v + d * 4);
+        pack_nonneg16(v, packed);
     } else {
         if (F.act == CLDNN_HIP_ACT_RELU) {
 #pragma unroll
@@ -364,8 +381,7 @@ __device__ __forceinline__ v4i epilogue_fast16(const Args& a, const v4i (&acc)[4
             if (F.eltw_relu_folded) {
 #pragma unroll
                 for (int c = 0; c < 16; ++c) v[c] = med3(v[c] * ecal[c], 0.0f, F.hi) + 0.49999997f;
-#pragma unroll
-                for (int d = 0; d < 4; ++d) packed[d] = pack_nonneg(v + d * 4);
+                pack_nonneg16(v, packed);
                 finished = true;
             } else if (F.eltw_act == CLDNN_HIP_ACT_RELU) {
 #pragma unroll
