@@ -216,7 +216,9 @@ __device__ __forceinline__ void keep_branch() { asm volatile(""); }
 __device__ __forceinline__ void zero_padding_features(v4i& packed, int valid)
 {
     if (valid < 16) {
-        keep_branch();
+        // the masks depend on `valid` alone; unless it passes through the asm they are computed ahead of the branch, for
+        // every wave (16 compares and selects), whether a slice is partly filled or not
+        asm volatile("" : "+v"(valid));
 #pragma unroll
         for (int d = 0; d < 4; ++d) {
             unsigned keep = 0;
@@ -486,6 +488,23 @@ struct PixelPos {
     uint32_t b, oy, ox;
 };
 
+// Everything a kernel's prologue reads from the argument block, fetched behind one wait.  Left to itself the compiler
+// fetches an argument where it is first used, and a wave makes five or six dependent round trips to memory (a few
+// hundred nanoseconds each) before its first operand request goes out.
+__device__ __forceinline__ void fetch_arguments(const MfmaArgs& a)
+{
+    asm volatile("" ::"s"(a.in), "s"(a.wpk), "s"(a.ktab), "s"(a.acc_init), "s"(a.out), "s"(a.eltw), "s"(a.M), "s"(a.OFM),
+                 "s"(a.ofm_tiles), "s"(a.mtiles), "s"(a.OHW), "s"(a.OW), "s"(a.div_ohw.mul), "s"(a.div_ohw.shift),
+                 "s"(a.div_ohw.one), "s"(a.div_ow.mul), "s"(a.div_ow.shift), "s"(a.div_ow.one), "s"(a.sy), "s"(a.sx), "s"(a.py),
+                 "s"(a.px), "s"(a.esy), "s"(a.esx));
+    asm volatile("" ::"s"(a.in_off), "s"(a.in_pb), "s"(a.in_pf), "s"(a.in_py), "s"(a.out_off), "s"(a.out_pb), "s"(a.out_pf),
+                 "s"(a.out_py), "s"(a.el_off), "s"(a.el_pb), "s"(a.el_pf), "s"(a.el_py), "s"(a.ksteps), "s"(a.CB), "s"(a.FX),
+                 "s"(a.kchunks), "s"(a.tap_dy), "s"(a.tap_dx), "s"(a.linear), "s"(a.px_bytes), "s"(a.by_features));
+    asm volatile("" ::"s"(a.div_cb.mul), "s"(a.div_cb.shift), "s"(a.div_cb.one), "s"(a.div_fx.mul), "s"(a.div_fx.shift),
+                 "s"(a.div_fx.one), "s"(a.xor_mask), "s"(a.wsl_parts), "s"(a.wsl_tpp), "s"(a.FY), "s"(a.epi.calib),
+                 "s"(a.epi.eltw_calib), "s"(a.epi.wqf), "s"(a.fe.hi), "s"(a.fe.lo));
+}
+
 __device__ __forceinline__ PixelPos pixel_pos(const MfmaArgs& a, uint32_t m)
 {
     PixelPos p;
@@ -505,6 +524,7 @@ __device__ __forceinline__ PixelPos pixel_pos(const MfmaArgs& a, uint32_t m)
 template <int BM, int BN, int WP, bool CHECKED, int EPI>
 __global__ void __launch_bounds__(256) conv_mfma_kernel(MfmaArgs a)
 {
+    fetch_arguments(a);
     constexpr int NT = WP / 16;         // pixel tiles per wave
     constexpr int WAVES_F = BN / 64;    // waves along features
     constexpr int A_LOADS = BN / 64;    // 16-byte weight chunks per thread per K-step
@@ -675,6 +695,7 @@ __global__ void __launch_bounds__(256) conv_mfma_kernel(MfmaArgs a)
 template <int BN, int NT, int KG, int EPI>
 __global__ void __launch_bounds__(256 * KG) conv_bdir_kernel(MfmaArgs a)
 {
+    fetch_arguments(a);
     constexpr int MT = BN / 16;       // weight fragments (16 features each) per wave and K-step
     constexpr int SPANS = BN / 64;
     constexpr int WP = NT * 16;       // pixels per wave
@@ -975,6 +996,7 @@ __device__ __forceinline__ void tap_advance(const MfmaArgs& a, TapWalk& w, int c
 template <int NT, int D, int EPI>
 __global__ void __launch_bounds__(256) conv_wsl_kernel(MfmaArgs a)
 {
+    fetch_arguments(a);
     constexpr int WP = NT * 16;  // pixels per wave and tile
     const int t = threadIdx.x;
     const int lane = t & 63;
@@ -1141,6 +1163,7 @@ __global__ void __launch_bounds__(256) conv_stream_kernel(MfmaArgs a)
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int kq = lane >> 4;
     const int l16 = lane & 15;
+    fetch_arguments(a);
     const uint32_t gw = blockIdx.x * 4u + (uint32_t)wave;
     const int nspans = a.ofm_tiles;
     const int span = (int)(gw % (uint32_t)nspans);
