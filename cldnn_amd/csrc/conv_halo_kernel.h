@@ -18,6 +18,12 @@
 // (tile, feature block) pairs without draining: the next pair's patch lands in the other patch buffer while the
 // current one is multiplied, the weight ring never stops, and the requantisation of a finished tile overlaps the
 // loads of the next.
+//
+// Measured on VGG-16's layers at batch 16 and 32, this kernel is within 5 % of the best other row of the tile table on
+// every layer and better than it on none by more than the noise: its loop keeps the matrix pipe 70-75 % busy, but a launch
+// of such a layer spends about 12 us outside the loop (launch, start skew, prologue, a 3.6 us epilogue of 128 outputs
+// per lane, and a last round of tiles that is four fifths full).  The built-in table therefore never selects its rows;
+// a tuning cache or tile_override may.
 #pragma once
 #include <type_traits>
 
