@@ -108,7 +108,7 @@ __global__ void __launch_bounds__(WP * WF * 64) conv_halo_kernel(HaloArgs h)
     // Everything the prologue and the loop read from the argument block is requested here, behind ONE wait: left to
     // itself the compiler fetches arguments where they are first used, four dependent round trips to memory (about
     // 0.4 us each) before the first operand request goes out.
-    asm volatile("" ::"s"(a.in), "s"(a.wpk), "s"(a.acc_init), "s"(a.ofm_tiles), "s"(a.ksteps), "s"(a.in_pf), "s"(a.xor_mask),
+    asm volatile("" ::"s"(a.in), "s"(a.wpk), "s"(a.acc_init), "s"(a.ofm_tiles), "s"(a.div_ofm_tiles.mul), "s"(a.div_ofm_tiles.shift), "s"(a.div_ofm_tiles.one), "s"(a.ksteps), "s"(a.in_pf), "s"(a.xor_mask),
                  "s"(h.pos_total), "s"(h.halo_lo), "s"(h.patch_len), "s"(h.cps), "s"(h.div_cps.mul), "s"(h.div_cps.shift),
                  "s"(h.div_cps.one), "s"(h.blocks), "s"(h.ptiles), "s"(h.parts), "s"(h.tap[0]), "s"(h.tap[1]), "s"(h.tap[2]),
                  "s"(h.tap[3]), "s"(h.tap[4]), "s"(h.tap[5]), "s"(h.tap[6]), "s"(h.tap[7]), "s"(h.tap[8]));
@@ -117,8 +117,9 @@ __global__ void __launch_bounds__(WP * WF * 64) conv_halo_kernel(HaloArgs h)
     // all their feature tiles adjacent in time: neighbouring position tiles share their halos, feature tiles their
     // whole patch, through that die's L2.
     const int xcd = blockIdx.x & 7, jj = blockIdx.x >> 3;
-    const int part = xcd * (h.parts >> 3) + jj / a.ofm_tiles;
-    const int ntile = jj % a.ofm_tiles;
+    const int jj_by_f = (int)a.div_ofm_tiles.div((uint32_t)jj);
+    const int part = xcd * (h.parts >> 3) + jj_by_f;
+    const int ntile = jj - jj_by_f * a.ofm_tiles;
     const int t_begin = (int)(((uint32_t)part * (uint32_t)h.ptiles) / (uint32_t)h.parts);
     const int t_end = (int)(((uint32_t)(part + 1) * (uint32_t)h.ptiles) / (uint32_t)h.parts);
     if (t_begin >= t_end) return;

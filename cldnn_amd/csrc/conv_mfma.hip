@@ -513,6 +513,7 @@ void launch_conv_mfma(hipStream_t s, const ConvProblem& p, const MfmaPlan& pl, c
     a.OFM = p.OFM, a.ofm_tiles = pl.ofm_tiles, a.mtiles = pl.mtiles;
     a.OHW = p.OH * p.OW, a.OW = p.OW, a.OH = p.OH, a.IH = p.IH, a.IW = p.IW;
     a.div_ohw = make_div((uint32_t)a.OHW), a.div_ow = make_div((uint32_t)a.OW);
+    a.div_mtiles = make_div((uint32_t)a.mtiles), a.div_ofm_tiles = make_div((uint32_t)a.ofm_tiles);
     a.sy = p.sy, a.sx = p.sx, a.py = p.py, a.px = p.px, a.esy = p.esy, a.esx = p.esx;
     a.in_off = (int32_t)p.in_p.off, a.in_pb = (int32_t)p.in_p.pb, a.in_pf = (int32_t)p.in_p.pf, a.in_py = (int32_t)p.in_p.py;
     a.out_off = (int32_t)p.out_p.off, a.out_pb = (int32_t)p.out_p.pb, a.out_pf = (int32_t)p.out_p.pf;

@@ -70,6 +70,9 @@ struct MfmaArgs {
     // bytes per pixel of one input slice: 16 (fs_b_yx_fsv16) or 4 (b_fs_yx_fsv4, first layers; streaming kernel only)
     int32_t px_bytes;
     FastDiv div_cb, div_fx;
+    // workgroup id -> (pixel tile, feature tile): a plain division of two kernel arguments costs a wave some forty
+    // instructions with four trips between the vector and the scalar unit, before its first load is requested
+    FastDiv div_mtiles, div_ofm_tiles;
     uint32_t xor_mask;  // 0x80808080 for u8 activations, 0 for s8
     const v4i* bpk;     // small-batch kernel: scratch for the activations in fragment order (nullptr: read them in place)
     FastEpi fe;
@@ -488,9 +491,9 @@ struct PixelPos {
     uint32_t b, oy, ox;
 };
 
-// Everything a kernel's prologue reads from the argument block, fetched behind one wait.  Left to itself the compiler
-// fetches an argument where it is first used, and a wave makes five or six dependent round trips to memory (a few
-// hundred nanoseconds each) before its first operand request goes out.
+// Everything a kernel reads from the argument block, fetched behind one wait.  Left to itself the compiler fetches an
+// argument where it is first used, and a wave makes five or six dependent round trips to memory (a few hundred
+// nanoseconds each) before its first operand request goes out, and one or two more in front of its epilogue.
 __device__ __forceinline__ void fetch_arguments(const MfmaArgs& a)
 {
     asm volatile("" ::"s"(a.in), "s"(a.wpk), "s"(a.ktab), "s"(a.acc_init), "s"(a.out), "s"(a.eltw), "s"(a.M), "s"(a.OFM),
@@ -501,8 +504,9 @@ __device__ __forceinline__ void fetch_arguments(const MfmaArgs& a)
                  "s"(a.out_py), "s"(a.el_off), "s"(a.el_pb), "s"(a.el_pf), "s"(a.el_py), "s"(a.ksteps), "s"(a.CB), "s"(a.FX),
                  "s"(a.kchunks), "s"(a.tap_dy), "s"(a.tap_dx), "s"(a.linear), "s"(a.px_bytes), "s"(a.by_features));
     asm volatile("" ::"s"(a.div_cb.mul), "s"(a.div_cb.shift), "s"(a.div_cb.one), "s"(a.div_fx.mul), "s"(a.div_fx.shift),
-                 "s"(a.div_fx.one), "s"(a.xor_mask), "s"(a.wsl_parts), "s"(a.wsl_tpp), "s"(a.FY), "s"(a.epi.calib),
-                 "s"(a.epi.eltw_calib), "s"(a.epi.wqf), "s"(a.fe.hi), "s"(a.fe.lo));
+                 "s"(a.div_fx.one), "s"(a.div_mtiles.mul), "s"(a.div_mtiles.shift), "s"(a.div_mtiles.one), "s"(a.div_ofm_tiles.mul),
+                 "s"(a.div_ofm_tiles.shift), "s"(a.div_ofm_tiles.one), "s"(a.xor_mask), "s"(a.wsl_parts), "s"(a.wsl_tpp), "s"(a.FY),
+                 "s"(a.epi.calib), "s"(a.epi.eltw_calib), "s"(a.epi.wqf), "s"(a.fe.hi), "s"(a.fe.lo));
 }
 
 __device__ __forceinline__ PixelPos pixel_pos(const MfmaArgs& a, uint32_t m)
@@ -547,8 +551,9 @@ __global__ void __launch_bounds__(256) conv_mfma_kernel(MfmaArgs a)
     // with by_features it takes every eighth feature tile with all pixel tiles (sharing the weights).
     const int xcd = blockIdx.x & 7;
     const int j = blockIdx.x >> 3;
-    const int ptile = a.by_features ? j % a.mtiles : (j / a.ofm_tiles) * 8 + xcd;
-    const int ntile = a.by_features ? (j / a.mtiles) * 8 + xcd : j % a.ofm_tiles;
+    const int j_by_m = (int)a.div_mtiles.div((uint32_t)j), j_by_f = (int)a.div_ofm_tiles.div((uint32_t)j);
+    const int ptile = a.by_features ? j - j_by_m * a.mtiles : j_by_f * 8 + xcd;
+    const int ntile = a.by_features ? j_by_m * 8 + xcd : j - j_by_f * a.ofm_tiles;
     if (ptile >= a.mtiles || ntile >= a.ofm_tiles) return;
     const uint32_t m0 = (uint32_t)ptile * BM;
 
@@ -720,8 +725,9 @@ __global__ void __launch_bounds__(256 * KG) conv_bdir_kernel(MfmaArgs a)
     // same workgroup order as the LDS-staged kernel: a die takes every eighth tile of one kind
     const int xcd = blockIdx.x & 7;
     const int j = blockIdx.x >> 3;
-    const int ptile = a.by_features ? j % a.mtiles : (j / a.ofm_tiles) * 8 + xcd;
-    const int ntile = a.by_features ? (j / a.mtiles) * 8 + xcd : j % a.ofm_tiles;
+    const int j_by_m = (int)a.div_mtiles.div((uint32_t)j), j_by_f = (int)a.div_ofm_tiles.div((uint32_t)j);
+    const int ptile = a.by_features ? j - j_by_m * a.mtiles : j_by_f * 8 + xcd;
+    const int ntile = a.by_features ? j_by_m * 8 + xcd : j - j_by_f * a.ofm_tiles;
     if (ptile >= a.mtiles || ntile >= a.ofm_tiles) return;
     const uint32_t m0 = (uint32_t)ptile * BM + (uint32_t)wave * WP;
 
@@ -754,7 +760,10 @@ __global__ void __launch_bounds__(256 * KG) conv_bdir_kernel(MfmaArgs a)
     const v4i* wsrc = a.wpk + ((size_t)ntile * a.ksteps + step0) * (4 * BN) + t;
 
     // look-ahead in K-steps for both operands
-    constexpr int D = LEAN ? 3 : BDIR_PREFETCH_DISTANCE(A_LOADS + NT);
+    // 32 pixels x 128 features per wave with a look-ahead of six steps needs 250-262 registers depending on what the
+    // register allocator makes of the prologue, and above 256 the kernel loses its second wave per SIMD (25 % slower):
+    // five steps keep it clear of the limit
+    constexpr int D = LEAN ? 3 : (BN == 128 && NT == 2 && KG == 1 ? 5 : BDIR_PREFETCH_DISTANCE(A_LOADS + NT));
     constexpr int DA = D;
     v4i ra[DA][A_LOADS], rb[D][NT];
     auto load_a = [&](int ks, v4i (&xa)[A_LOADS]) {
@@ -1008,8 +1017,9 @@ __global__ void __launch_bounds__(256) conv_wsl_kernel(MfmaArgs a)
     // in time: they run on the same accelerator die and share the activations through its L2
     const int xcd = blockIdx.x & 7;
     const int j = blockIdx.x >> 3;
-    const int part = (j / a.ofm_tiles) * 8 + xcd;
-    const int ntile = j % a.ofm_tiles;
+    const int j_by_f = (int)a.div_ofm_tiles.div((uint32_t)j);
+    const int part = j_by_f * 8 + xcd;
+    const int ntile = j - j_by_f * a.ofm_tiles;
     const int t_begin = part * a.wsl_tpp;
     const int t_end = min(t_begin + a.wsl_tpp, a.mtiles);
     if (t_begin >= t_end) return;
@@ -1166,8 +1176,8 @@ __global__ void __launch_bounds__(256) conv_stream_kernel(MfmaArgs a)
     fetch_arguments(a);
     const uint32_t gw = blockIdx.x * 4u + (uint32_t)wave;
     const int nspans = a.ofm_tiles;
-    const int span = (int)(gw % (uint32_t)nspans);
-    const uint32_t pt = gw / (uint32_t)nspans;
+    const uint32_t pt = a.div_ofm_tiles.div(gw);
+    const int span = (int)(gw - pt * (uint32_t)nspans);
     if (pt >= (uint32_t)a.mtiles) return;  // no barriers below: a wave may leave on its own
 
     const int f0 = span * 64 + kq * 16;
