@@ -198,6 +198,8 @@ static void launch_dwchain(hipStream_t s, const ChainStageIn* st, const ChainPla
     a.units = pl.units;
     a.vec_quads = (pl.lds_bytes - a.dw_quads * 16 - pl.units * 4096) / 16;
     a.granules = pl.granules;
+    a.gpw = pl.granules / (pl.grid * 4), a.grem = pl.granules % (pl.grid * 4);
+    a.div_waves = make_fast_div((uint32_t)pl.grid * 4u);
     a.M = (uint32_t)pl.m_total;
     a.OHW = p0.OH * p0.OW, a.OW = p0.OW;
     a.div_ohw = make_fast_div((uint32_t)a.OHW), a.div_ow = make_fast_div((uint32_t)a.OW);
@@ -287,6 +289,8 @@ void launch_conv_chain(hipStream_t s, const ChainStageIn* st, const ChainPlan& p
     a.units = pl.units;
     a.vec_quads = (pl.lds_bytes - pl.units * 4096) / 16;
     a.granules = pl.granules;
+    a.gpw = pl.granules / (pl.grid * 4), a.grem = pl.granules % (pl.grid * 4);
+    a.div_waves = make_fast_div((uint32_t)pl.grid * 4u);
     a.M = (uint32_t)pl.m_total;
     a.OHW = p0.OH * p0.OW, a.OW = p0.OW;
     a.div_ohw = make_fast_div((uint32_t)a.OHW), a.div_ow = make_fast_div((uint32_t)a.OW);

@@ -44,6 +44,8 @@ struct ChainArgs {
     int32_t units;
     int32_t vec_quads;         // 16-byte pieces of per-feature vectors behind the units
     int32_t granules;          // ceil(M / (16 * NT))
+    int32_t gpw, grem;         // granules / waves of the grid and the remainder
+    FastDiv div_waves;         // wave w starts at granule w * gpw + (w * grem) / waves = floor(w * granules / waves)
     uint32_t M;
     int32_t OHW, OW;
     FastDiv div_ohw, div_ow;
@@ -153,9 +155,10 @@ __global__ void __launch_bounds__(256) conv_chain_kernel(ChainArgs a)
     // times what the better balance saved.)
     const int per_xcd = gridDim.x >> 3;  // the grid is a multiple of 8
     const uint32_t vb = (blockIdx.x & 7u) * (uint32_t)per_xcd + (blockIdx.x >> 3);
-    const uint32_t gw = vb * 4u + (uint32_t)wave, waves = gridDim.x * 4u;
-    const int g_begin = (int)(((uint64_t)gw * (uint32_t)a.granules) / waves);
-    const int g1 = (int)(((uint64_t)(gw + 1) * (uint32_t)a.granules) / waves);
+    // (a 64-bit division of two run-time values here costs every wave a few hundred instructions before its first request)
+    const uint32_t gw = vb * 4u + (uint32_t)wave;
+    const int g_begin = (int)(gw * (uint32_t)a.gpw + a.div_waves.div(gw * (uint32_t)a.grem));
+    const int g1 = (int)((gw + 1) * (uint32_t)a.gpw + a.div_waves.div((gw + 1) * (uint32_t)a.grem));
 
     const v4i xm0 = {(int)s0.xor_mask, (int)s0.xor_mask, (int)s0.xor_mask, (int)s0.xor_mask};
     const v4i xm1 = {(int)s1.xor_mask, (int)s1.xor_mask, (int)s1.xor_mask, (int)s1.xor_mask};

@@ -28,6 +28,8 @@ struct DwChainArgs {
     int32_t dw_quads;          // 16-byte pieces of the diagonal-weight table (KS * 9 * 64)
     int32_t units, vec_quads;
     int32_t granules;          // ceil(M / (16 * NT))
+    int32_t gpw, grem;         // granules / waves of the grid and the remainder
+    FastDiv div_waves;         // wave w starts at granule w * gpw + (w * grem) / waves = floor(w * granules / waves)
     uint32_t M;
     int32_t OHW, OW;
     FastDiv div_ohw, div_ow;
@@ -76,9 +78,9 @@ __global__ void __launch_bounds__(256) conv_dwchain_kernel(DwChainArgs a)
 
     const int per_xcd = gridDim.x >> 3;  // the grid is a multiple of 8
     const uint32_t vb = (blockIdx.x & 7u) * (uint32_t)per_xcd + (blockIdx.x >> 3);
-    const uint32_t gw = vb * 4u + (uint32_t)wave, waves = gridDim.x * 4u;
-    const int g_begin = (int)(((uint64_t)gw * (uint32_t)a.granules) / waves);
-    const int g_end = (int)(((uint64_t)(gw + 1) * (uint32_t)a.granules) / waves);
+    const uint32_t gw = vb * 4u + (uint32_t)wave;
+    const int g_begin = (int)(gw * (uint32_t)a.gpw + a.div_waves.div(gw * (uint32_t)a.grem));
+    const int g_end = (int)((gw + 1) * (uint32_t)a.gpw + a.div_waves.div((gw + 1) * (uint32_t)a.grem));
     if (g_begin >= g_end) {
         __syncthreads();
         return;

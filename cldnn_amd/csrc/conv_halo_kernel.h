@@ -43,6 +43,8 @@ struct HaloArgs {
     FastDiv div_cps;
     int32_t blocks;            // blocks of 64 input features
     int32_t ptiles, parts;     // position tiles; workgroups per feature tile (multiple of 8)
+    int32_t tpp, trem;         // ptiles / parts and the remainder
+    FastDiv div_parts;         // partition p starts at tile p * tpp + (p * trem) / parts = floor(p * ptiles / parts)
     int32_t tap[9];            // halo_lo + distance of tap k, in positions (>= 0)
 };
 
@@ -120,8 +122,8 @@ __global__ void __launch_bounds__(WP * WF * 64) conv_halo_kernel(HaloArgs h)
     const int jj_by_f = (int)a.div_ofm_tiles.div((uint32_t)jj);
     const int part = xcd * (h.parts >> 3) + jj_by_f;
     const int ntile = jj - jj_by_f * a.ofm_tiles;
-    const int t_begin = (int)(((uint32_t)part * (uint32_t)h.ptiles) / (uint32_t)h.parts);
-    const int t_end = (int)(((uint32_t)(part + 1) * (uint32_t)h.ptiles) / (uint32_t)h.parts);
+    const int t_begin = (int)((uint32_t)part * (uint32_t)h.tpp + h.div_parts.div((uint32_t)part * (uint32_t)h.trem));
+    const int t_end = (int)((uint32_t)(part + 1) * (uint32_t)h.tpp + h.div_parts.div((uint32_t)(part + 1) * (uint32_t)h.trem));
     if (t_begin >= t_end) return;
 
     extern __shared__ __align__(16) unsigned char smem[];

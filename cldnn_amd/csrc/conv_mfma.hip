@@ -573,6 +573,8 @@ void launch_conv_mfma(hipStream_t s, const ConvProblem& p, const MfmaPlan& pl, c
         h.div_cps = make_div((uint32_t)h.cps);
         h.blocks = pl.cb / 4;
         h.ptiles = pl.halo_ptiles, h.parts = pl.halo_parts;
+        h.tpp = pl.halo_ptiles / pl.halo_parts, h.trem = pl.halo_ptiles % pl.halo_parts;
+        h.div_parts = make_div((uint32_t)pl.halo_parts);
         for (int k = 0; k < HALO_TAPS; ++k)
             h.tap[k] = h.halo_lo + ((k / p.FX) * p.dy - p.py) * h.Wp + ((k % p.FX) * p.dx - p.px);
         launch_halo(s, h, pl.tile - FIRST_HALO_ROW, pl.halo_pl, pl.grid, pl.lds_bytes, kind);
