@@ -113,7 +113,9 @@ std::string chain_plan(const ChainStageIn* st, int n, int cus, ChainPlan* out)
         pl.ksteps0 = pl.sp[0];  // K-steps the depthwise stage delivers to stage 1
         pl.lds_bytes = pl.sp[0] * 9 * 1024 + pl.units * 4096 + vec * 4;  // diagonal-weight table, units, vectors
         if (pl.lds_bytes > CHAIN_MAX_LDS) return "the weights of the chain (" + std::to_string(pl.lds_bytes / 1024) + " KiB) do not fit into LDS";
-        const int per_cu = std::min(4, CHAIN_MAX_LDS / pl.lds_bytes);
+        // workgroups a CU holds at once: by LDS, and by registers (16-pixel granules: 137-167 registers = three waves per
+        // SIMD; 32-pixel granules: 206-239 = two).  The grid is what is resident, so that no workgroup waits for a slot.
+        const int per_cu = std::min(pl.nt == 1 ? 3 : 2, CHAIN_MAX_LDS / pl.lds_bytes);
         int grid = cus * per_cu / 8 * 8;
         const int wanted = ((pl.granules + 3) / 4 + 7) / 8 * 8;  // at least one granule per wave
         if (grid > wanted) grid = wanted;
