@@ -287,10 +287,12 @@ MfmaPlan mfma_plan(const ConvProblem& p, int tile, int cus)
     if (tc.kgroups > 1)  // per-group weight buffers, later reused for the partial sums of groups 1..
         pl.lds_bytes = std::max(tc.kgroups * pl.lds_bytes, (tc.kgroups - 1) * (tc.tile_ofm / 16) * (tc.wave_pixels / 16) * 4096);
     if (pl.wsl) {
-        // persistent workgroups: as many as the chip holds at once (LDS and registers allow two per CU at most),
-        // split evenly over the feature tiles; partitions come in eights (one per accelerator die)
+        // persistent workgroups: as many as the chip holds at once, by LDS and by registers (16 pixels per wave: 118-168
+        // registers = three waves per SIMD; 32 and 64 pixels per wave: two), split evenly over the feature tiles;
+        // partitions come in eights (one per accelerator die)
         pl.lds_bytes = pl.ksteps * 4096;
-        const int per_cu = pl.lds_bytes * 2 <= WSL_MAX_LDS ? 2 : 1;
+        const int by_regs = tc.wave_pixels == 16 ? 3 : 2;
+        const int per_cu = std::max(1, std::min(by_regs, (int)WSL_MAX_LDS / pl.lds_bytes));
         int parts = std::max(8, cus * per_cu / pl.ofm_tiles / 8 * 8);
         pl.wsl_tpp = (pl.mtiles + parts - 1) / parts;
         parts = ((pl.mtiles + pl.wsl_tpp - 1) / pl.wsl_tpp + 7) / 8 * 8;
