@@ -8,6 +8,7 @@
 // network are normally fused into the convolution before them and never reach this kernel.
 #include "epilogue.h"
 #include "kernels.h"
+#include "conv_mfma_kernel.h"  // FastDiv
 
 namespace chip {
 
@@ -132,6 +133,7 @@ struct EltwiseBlockedArgs {
     int count, mode;
     int doff, dpb, dpf, dpy;
     int B, F, Y, X, slices;
+    FastDiv div_x;
     int quantized, calib_vec4;
     const float* calib;
     float oqf;
@@ -139,12 +141,17 @@ struct EltwiseBlockedArgs {
     float m, n;
 };
 
+// MODE: the operation fixed at compile time (the sum of a residual block: the common case), or -1 = read it from the
+// arguments.  Left to the run-time value alone, the sixteen switch statements of a lane stay sixteen chains of scalar
+// branches, each with the division sequences of the div and mod modes behind them.
+template <int MODE>
 __global__ void __launch_bounds__(256) eltwise_blocked_kernel(EltwiseBlockedArgs p, uint8_t* __restrict__ dst)
 {
+    const int mode = MODE >= 0 ? MODE : p.mode;
     // grid: x over the pixels of a plane, y = batch, z = feature slice
     const unsigned pixel = blockIdx.x * blockDim.x + threadIdx.x;
     if (pixel >= (unsigned)(p.Y * p.X)) return;
-    const int y = (int)(pixel / (unsigned)p.X), x = (int)(pixel - (unsigned)y * p.X);
+    const int y = (int)p.div_x.div(pixel), x = (int)(pixel - (unsigned)y * p.X);
     const int b = (int)blockIdx.y, fs = (int)blockIdx.z;
     int v[16];
     {
@@ -166,7 +173,7 @@ __global__ void __launch_bounds__(256) eltwise_blocked_kernel(EltwiseBlockedArgs
             int o = p.is_u8[i] ? (int)byte : (int)(signed char)byte;
             // an operand of the other 8-bit type is cast to the first input's type first
             if (p.is_u8[i] != p.is_u8[0]) o = wrap_unsigned ? (int)(unsigned char)o : (int)(signed char)o;
-            int t = eltwise_op_int(p.mode, v[c], o);
+            int t = eltwise_op_int(mode, v[c], o);
             if (!p.quantized) t = wrap_unsigned ? (int)(unsigned char)t : (int)(signed char)t;
             v[c] = t;
         }
@@ -230,8 +237,10 @@ static bool launch_eltwise_blocked(hipStream_t s, const cldnn_hip_eltwise_desc& 
     const int64_t plane = (int64_t)p.Y * p.X;
     if (plane == 0 || p.B == 0) return true;
     if (p.B > 65535 || p.slices > 65535) return false;
-    hipLaunchKernelGGL(eltwise_blocked_kernel, dim3((unsigned)((plane + 255) / 256), (unsigned)p.B, (unsigned)p.slices), dim3(256), 0, s, p,
-                       (uint8_t*)dst);
+    p.div_x = make_fast_div((uint32_t)p.X);
+    const dim3 grid((unsigned)((plane + 255) / 256), (unsigned)p.B, (unsigned)p.slices);
+    if (p.mode == CLDNN_HIP_ELTWISE_SUM) hipLaunchKernelGGL(eltwise_blocked_kernel<CLDNN_HIP_ELTWISE_SUM>, grid, dim3(256), 0, s, p, (uint8_t*)dst);
+    else hipLaunchKernelGGL(eltwise_blocked_kernel<-1>, grid, dim3(256), 0, s, p, (uint8_t*)dst);
     CHIP_CHECK(hipGetLastError());
     return true;
 }
