@@ -159,7 +159,7 @@ int mfma_choose(const ConvProblem& p, int cus)
         if (m >= 16384) return ROW_WSL_P64;                       // 1x1 reductions at 56x56 and 28x28
         if (m >= 4096) {
             if (p.OFM > 1024) return ROW_P64_F128;  // a 14x14 projection together with the block's opening 1x1
-            if (p.OFM >= 512) return ksteps <= 4 ? ROW_WSL_P128 : ROW_BDIR_P128_F128;  // 14x14 expansions / projections
+            if (p.OFM >= 512) return ksteps <= 4 ? ROW_WSL_P64 : ROW_BDIR_P128_F128;  // 14x14 expansions / projections
             return stream_fits ? stream_row : ROW_BDIR_P64_F64;
         }
         if (p.OFM >= 1024 && m >= 512) return ROW_P64_F128;       // 7x7 expansions; at a few hundred pixels 64-feature tiles give more workgroups
