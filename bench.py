@@ -372,7 +372,7 @@ def network_workload(args):
         return outs
 
     t0 = time.perf_counter()
-    while time.perf_counter() - t0 < CLOCK_WARMUP_SECONDS:  # see clock_warmup()
+    while time.perf_counter() - t0 < args.clock_warmup:  # see clock_warmup()
         run()
     for _ in range(args.warmup):
         run()
@@ -463,7 +463,7 @@ def network_workload(args):
         "unit": "images/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": dt / args.steps * 1e3,
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "i8xi8->i32 (f32 requantisation)", "data": "synthetic",
         "config": {"workload": args.workload, "batch": batch, "primitives": primitives,
-                   "clock_warmup_s": CLOCK_WARMUP_SECONDS,
+                   "clock_warmup_s": args.clock_warmup,
                    "build": "optimize_data" + (", tuning cache" if args.tuning_cache else "") + (", second stream" if args.second_stream else ""), "primitives_per_execute": len(executed), "launches_per_execute": len(executed) - len(followers) - len(paired),
                    "convolutions_in_a_neighbours_launch": len(paired),
                    "chained_convolutions": len(followers) + len({str(infos[i]["kernel"]) for i in followers}),
@@ -581,13 +581,14 @@ def kernel_rooflines(heads, times):
 CLOCK_WARMUP_SECONDS = 0.3
 
 
-def clock_warmup(eng, step):
+def clock_warmup(eng, step, seconds=None):
     """The clocks of an idle device rise over tens of milliseconds of load (a layer timed right after idling runs
     10 % and more slower than in a steady stream of work), and a short run (--steps 20 --warmup 5 is 15 ms) would be
     timed on that ramp.  Untimed steps for CLOCK_WARMUP_SECONDS of wall time come first, then the W warm-up steps, then
     exactly K timed steps; the JSON line names this under config.clock_warmup_s."""
+    seconds = CLOCK_WARMUP_SECONDS if seconds is None else seconds
     t0 = time.perf_counter()
-    while time.perf_counter() - t0 < CLOCK_WARMUP_SECONDS:
+    while time.perf_counter() - t0 < seconds:
         for _ in range(5):
             step()
         eng.finish()
@@ -613,7 +614,7 @@ def measure_stack(args, wl, steps, warmup, in_flight_n, cpu_seconds, extras):
 
     ops = sum(L.info.ops for L in heads)
     nbytes = sum(L.info.bytes for L in heads)
-    clock_warmup(eng, lambda: run_step(seq))
+    clock_warmup(eng, lambda: run_step(seq), args.clock_warmup)
     for _ in range(warmup):
         run_step(seq)
     eng.finish()
@@ -736,7 +737,7 @@ def measure_stack(args, wl, steps, warmup, in_flight_n, cpu_seconds, extras):
                    "layout": "fs_b_yx_fsv16",
                    "variant": "stride on the first 1x1 (Caffe form)" if wl.startswith("resnet50") else wl,
                    "fused_residual_layers": sum(1 for L in stack if L.fused),
-                   "clock_warmup_s": CLOCK_WARMUP_SECONDS},
+                   "clock_warmup_s": args.clock_warmup},
         "achieved_tops": ops * steps / t_gpu / 1e12,
         "roofline": {
             "bound": "hbm" if hbm_bound else "mfma",
@@ -812,6 +813,9 @@ def main():
                     help="after the headline measurement also time this many independent requests of the same workload in "
                          "flight at once, one engine (HIP stream) and one host thread each; reported under "
                          "requests_in_flight, never as the headline value (0 or 1 = skip)")
+    ap.add_argument("--clock-warmup", type=float, default=CLOCK_WARMUP_SECONDS,
+                    help="seconds of untimed steps before the warm-up steps (0 for counter runs under rocprofv3 --pmc, where "
+                         "every dispatch is serialised and recorded)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline / full-size check")
     ap.add_argument("--no-others", action="store_true", help="default workload only: do not time the other four configurations")
     ap.add_argument("--host-io", action="store_true",
