@@ -378,8 +378,10 @@ int32_t cldnn_hip_conv_out_extent(int32_t in, int32_t pad, int32_t filt, int32_t
 /* Kernel runner for tuning: times the table's own choice and every row of the tile-config table that accepts this
  * convolution, on scratch tensors of the descriptor's shapes filled with pseudo-random bytes, and reports the fastest.
  * Replaces the reference's kernel_runner (src/gpu/kernel_runner.cpp:106-190, used by tuning_mode tune_and_cache through
- * kernel_selector/core/kernel_selector.cpp GetAutoTuneBestKernel): each candidate is created, warmed up and run
- * `runs` times back to back on the engine's stream between two events; the best of three such batches counts.
+ * kernel_selector/core/kernel_selector.cpp GetAutoTuneBestKernel): the device is kept busy for 150 ms first (the
+ * clocks of an idle device rise over tens of milliseconds, and the candidates timed first would lose to the later ones),
+ * then each candidate is created, run for 20 ms untimed and `runs` times back to back on the engine's stream between
+ * two events; the best of three such batches counts.
  * best_tile_index = -1 when the table's own choice is the fastest (or no row applies: depthwise, plain layouts).
  * row_us (may be NULL) receives cldnn_hip_tile_config_count() entries, negative where a row does not apply.
  * Blocks until done; allocates and frees its scratch tensors. */
