@@ -9,7 +9,8 @@ table's own choice.  Two groups of layer shapes:
     whatever branch covers them.
 
 Each shape is tuned several times and every row takes the median of its passes, so that one noisy pass of a 5-40 us
-kernel on a shared box does not decide the test.  The table's row may be 15 % + 0.5 us slower than the best row."""
+kernel on a shared box does not decide the test; a shape that fails is measured once more with seven passes before it
+counts.  The table's row may be 15 % + 0.5 us slower than the best row."""
 import numpy as np
 import pytest
 
@@ -74,7 +75,7 @@ def shape_id(s):
     return "b%d_%dx%dx%d_to_%d_k%d_s%d" % (s[0], s[1], s[2], s[2], s[3], s[4], s[5])
 
 
-def tuned(shape):
+def tuned(shape, passes=PASSES):
     """-> (median microseconds of the table's row, {row index: median microseconds})"""
     B, IFM, HW, OFM, K, S = shape
     eng = hip.Engine(0, profiling=True)
@@ -87,7 +88,7 @@ def tuned(shape):
     calib = np.exp(r.uniform(np.log(1e-4), np.log(1e-2), OFM)).astype(np.float32)
     desc = hip.conv_desc(x_t, w.shape, "s8", stride=(S, S), pad=(pad, pad), bias_dt=hip.I32, has_wqf=True, has_calib=True, act="relu")
     default, rows = [], []
-    for _ in range(PASSES):
+    for _ in range(passes):
         _, _, default_us, row_us = hip.conv_tune(eng, desc, w, bias, wqf, calib, runs=RUNS)
         default.append(default_us)
         rows.append(row_us)
@@ -101,6 +102,10 @@ def test_table_choice_is_close_to_the_tuned_one(shape):
     default_us, rows = tuned(shape)
     assert len(rows) >= 3, rows  # several rows of the table take the shape
     best = min(rows, key=rows.get)
+    if default_us > 1.15 * rows[best] + 0.5:
+        # a second opinion before the verdict: more passes (a neighbour's burst on a shared box outlasts three)
+        default_us, rows = tuned(shape, passes=7)
+        best = min(rows, key=rows.get)
     ratio = default_us / rows[best]
     print("%s: the table's row %.1f us, best row %s %.1f us, ratio %.3f" % (shape_id(shape), default_us, hip.tile_config_name(best), rows[best], ratio))
     assert default_us <= 1.15 * rows[best] + 0.5, "the table's row takes %.1f us, row %s takes %.1f us (all rows: %s)" % (
