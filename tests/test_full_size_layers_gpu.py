@@ -135,3 +135,26 @@ def test_layer_at_its_real_batch_with_spread_outputs_and_accumulators(eng, wl, g
         bad = int(np.count_nonzero(acc != ref_acc))
         assert bad == 0, "%d of %d accumulators of %s differ (%s)" % (bad, acc.size, l["name"], L.info.kernel_name.decode())
     bench.release_stack(stack)
+
+
+def vgg_layer(name):
+    return [dict(l) for l in workloads.vgg16() if l["name"] == name]
+
+
+@pytest.mark.parametrize("row", ["halo_p256_f128", "halo_p512_f128"])
+@pytest.mark.parametrize("name", ["conv4", "conv6", "conv9"])
+def test_staged_patch_rows_at_full_size(eng, name, row):
+    """The two rows that only a tuning cache or tile_override selects, on VGG-16's layers at the benchmark batch: one
+    patch request per step and two, 128 to 512 features, several feature tiles per position tile."""
+    L_ = hip.lib()
+    names = [L_.cldnn_hip_tile_config_name(i).decode() for i in range(L_.cldnn_hip_tile_config_count())]
+    stack = bench.build_stack(eng, vgg_layer(name), 16, False, tile=names.index(row) + 1, calibration="spread")
+    kernel = stack[0].info.kernel_name.decode()
+    if not kernel.startswith("conv_halo<" + row):
+        bench.release_stack(stack)
+        pytest.skip("%s does not take %s (%s runs it)" % (row, name, kernel))
+    bench.run_step(bench.launches(stack))
+    eng.finish()
+    _, _, checked, mismatches = bench.cpu_pass(eng, stack, 1, verify=True)
+    assert checked > 0 and mismatches == 0, "%d of %d outputs differ from the oracle (%s)" % (mismatches, checked, kernel)
+    bench.release_stack(stack)
